@@ -1,0 +1,100 @@
+// Internal interfaces between the engine's translation units.
+//   f3m_geom.hip  : bounding box, Morton keys, counting sort, tree levels, interaction lists
+//                   (compiled with -ffp-contract=off: every fp32 operation rounds once)
+//   f3m_field.hip : exact products, near field, P2M / M2L / L2P
+//   f3m_plan.hip  : host orchestration and the C ABI
+#pragma once
+#include "f3m_rt.h"
+
+namespace f3m {
+
+struct Geo {
+    float origin[kMaxD];
+    float edge0;
+    int d;
+    int L;   // key depth: number of levels encoded in a Morton key (d*L <= 31)
+};
+
+struct TreeLevel {
+    int depth = 0;
+    float edge = 0.f;
+    int nb = 0;          // non-empty boxes
+    int maxcount = 0;
+    DBuf<int> off;       // nb+1 offsets into the Morton-sorted point order
+    DBuf<uint32_t> prefix;  // nb Morton prefixes (depth*d bits)
+    DBuf<float> ctr;     // nb*d box centres, row-major
+    DBuf<int> childstart;   // nb+1: compact id at depth+1 of each box's first child (set by the next level)
+};
+
+struct Tree {
+    Geo geo;
+    long long n = 0;
+    DBuf<float> pts;     // d*n, dimension-major, Morton-sorted
+    DBuf<uint32_t> keys; // n sorted keys
+    DBuf<int> perm;      // sorted position -> original row
+    std::vector<TreeLevel> lev;   // lev[0] is the root
+};
+
+struct PairList {
+    long long n = 0;
+    DBuf<int> pairs;     // (n,2) int32: (bx, by), sorted by (bx, by)
+    DBuf<int> rowptr;    // nbx+1: range of each x box
+};
+
+struct ClassifyParams {
+    int nr_interp;
+    int small_limit;
+    int var_comp;
+    int do_init, en_pair, en_all;
+    float crit, lcs, edge;
+};
+
+struct PlanLevel {
+    PairList far, small_, keep;
+    int num_nodes = 0;
+};
+
+// per-stage timing with HIP events (f3m_plan.hip); no-ops unless enabled through the C ABI
+enum Stage { kPlan = 0, kNear, kP2M, kM2L, kL2P, kPerm, kNumStages };
+void timer_begin(int stage, hipStream_t s);
+void timer_end(hipStream_t s);
+
+// --- f3m_geom.hip ---
+void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s);
+void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s);
+// adds lev[k] from lev[k-1]; returns false (and adds nothing) if the key depth is exhausted
+bool divide_tree(Tree &t, hipStream_t s);
+void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+                  PlanLevel &out, hipStream_t s);
+void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
+void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
+void build_rowptr(PairList &l, int nbx, hipStream_t s);
+
+// --- f3m_field.hip ---
+struct NodeSet {
+    int d = 0, P = 0, S1 = 0;
+    int n[kMaxD] = {0};
+    int start[kMaxD] = {0};
+    std::vector<float> t, w;        // concatenated 1-D nodes and barycentric weights (host)
+    DBuf<float> dt, dw;             // device copies
+    DBuf<float> noff;               // (P,d) node offsets of a box of the current level
+};
+void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s);
+void set_node_offsets(NodeSet &ns, float edge, hipStream_t s);
+
+void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s);
+void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
+void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
+
+void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
+                const float *bs, float *outs, float lcs, hipStream_t s);
+void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
+               NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
+               float *mom_out, float *loc_out, hipStream_t s);
+
+void exact_f32(int d, const float *X, long long N, const float *Y, long long M, const float *b, int c, float ls,
+               bool grad, float *out, hipStream_t s);
+void exact_f64(int d, const double *X, long long N, const double *Y, long long M, const double *b, int c, double ls,
+               double *out, hipStream_t s);
+
+}  // namespace f3m

@@ -1,0 +1,656 @@
+// Field kernels for gfx950: exact dense products, the near field, and the far field
+// (P2M -> M2L -> L2P) on Morton-sorted, dimension-major point arrays.
+#include "f3m_engine.h"
+
+#include <cmath>
+
+namespace f3m {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+// ------------------------------------------------------------------------------------------------
+// permutations between caller order and sorted order
+
+__global__ void gather_points_kernel(const float *__restrict__ X, const int *__restrict__ perm, long long n, int d,
+                                     float *__restrict__ pts)
+{
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    long long src = perm[i];
+    for (int j = 0; j < d; j++) pts[(long long)j * n + i] = X[src * d + j];
+}
+void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s)
+{
+    F3M_LAUNCH(gather_points_kernel, cdiv(n, 256), 256, 0, s, X, perm, n, d, pts);
+    check_launch("gather_points");
+}
+
+__global__ void gather_column_kernel(const float *__restrict__ b, const int *__restrict__ perm, long long n, int c, int col,
+                                     float *__restrict__ bs)
+{
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) bs[i] = b[(long long)perm[i] * c + col];
+}
+void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s)
+{
+    F3M_LAUNCH(gather_column_kernel, cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs);
+    check_launch("gather_column");
+}
+
+__global__ void scatter_column_kernel(const float *__restrict__ outs, const int *__restrict__ perm, long long n, int c,
+                                      int col, float *__restrict__ out)
+{
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[(long long)perm[i] * c + col] = outs[i];
+}
+void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s)
+{
+    F3M_LAUNCH(scatter_column_kernel, cdiv(n, 256), 256, 0, s, outs, perm, n, c, col, out);
+    check_launch("scatter_column");
+}
+
+// ------------------------------------------------------------------------------------------------
+// exact dense product (F3M_src/1_d_conv.cu:171-214; gradient form :126-169): one target per lane,
+// source tiles staged through LDS.
+
+template <typename T> __device__ inline T kernel_exp(T negr2_scaled);
+template <> __device__ inline float kernel_exp<float>(float v) { return fast_exp2(v); }   // v already times log2(e)
+template <> __device__ inline double kernel_exp<double>(double v) { return exp(v); }
+
+template <typename T, int D, bool GRAD>
+__global__ void __launch_bounds__(256) exact_kernel(const T *__restrict__ X, long long N, const T *__restrict__ Y, long long M,
+                                                     const T *__restrict__ b, int c, int col, T scale, T post,
+                                                     T *__restrict__ out)
+{
+    __shared__ T sy[D][256];
+    __shared__ T sb[256];
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    T x[D];
+#pragma unroll
+    for (int k = 0; k < D; k++) x[k] = (i < N) ? X[i * D + k] : (T)0;
+    T acc = 0;
+    for (long long j0 = 0; j0 < M; j0 += 256) {
+        long long j = j0 + threadIdx.x;
+        __syncthreads();
+        if (j < M) {
+#pragma unroll
+            for (int k = 0; k < D; k++) sy[k][threadIdx.x] = Y[j * D + k];
+            sb[threadIdx.x] = b[j * c + col];
+        }
+        __syncthreads();
+        int cnt = (int)((M - j0) < 256 ? (M - j0) : 256);
+        for (int jj = 0; jj < cnt; jj++) {
+            T r2 = 0;
+#pragma unroll
+            for (int k = 0; k < D; k++) { T t = x[k] - sy[k][jj]; r2 += t * t; }
+            T e = kernel_exp<T>(-r2 * scale);
+            if (GRAD) e *= r2;
+            acc += e * sb[jj];
+        }
+    }
+    if (i < N) out[i * c + col] = GRAD ? acc * post : acc;
+}
+
+template <typename T, bool GRAD>
+static void exact_dispatch(int d, const T *X, long long N, const T *Y, long long M, const T *b, int c, T scale, T post,
+                           T *out, hipStream_t s)
+{
+    unsigned grid = cdiv(N, 256);
+    for (int col = 0; col < c; col++) {
+#define F3M_CASE(DD)                                                                                               \
+    case DD:                                                                                                       \
+        F3M_LAUNCH((exact_kernel<T, DD, GRAD>), grid, 256, 0, s, X, N, Y, M, b, c, col, scale, post, out);         \
+        break;
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
+#undef F3M_CASE
+        check_launch("exact");
+    }
+}
+
+void exact_f32(int d, const float *X, long long N, const float *Y, long long M, const float *b, int c, float ls, bool grad,
+               float *out, hipStream_t s)
+{
+    if (N == 0) return;
+    float lcs = 1 / (2 * ls * ls);              // F3M_src/n_tree.cu:194
+    float post = 1 / (ls * ls * ls);            // F3M_src/n_tree.cu:223
+    if (grad) exact_dispatch<float, true>(d, X, N, Y, M, b, c, lcs * kLog2e, post, out, s);
+    else exact_dispatch<float, false>(d, X, N, Y, M, b, c, lcs * kLog2e, post, out, s);
+}
+
+void exact_f64(int d, const double *X, long long N, const double *Y, long long M, const double *b, int c, double ls,
+               double *out, hipStream_t s)
+{
+    if (N == 0) return;
+    double lcs = 1 / (2 * ls * ls);
+    exact_dispatch<double, false>(d, X, N, Y, M, b, c, lcs, 1.0, out, s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// tiles: work items (box, tile of `tile` consecutive points) for the boxes with flag != 0
+
+__global__ void tiles_per_box_kernel(const int *__restrict__ off, const int *__restrict__ flag, int nb, int tile,
+                                     int *__restrict__ ntiles)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nb) return;
+    int cnt = off[b + 1] - off[b];
+    ntiles[b] = (flag == nullptr || flag[b]) ? (cnt + tile - 1) / tile : 0;
+}
+
+__global__ void mark_rows_kernel(const int *__restrict__ rowptr, int nb, int *__restrict__ flag)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b < nb) flag[b] = rowptr[b + 1] > rowptr[b] ? 1 : 0;
+}
+
+__global__ void mark_cols_kernel(const int *__restrict__ pairs, long long n, int *__restrict__ flag)
+{
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) flag[pairs[2 * t + 1]] = 1;
+}
+
+// tileoff (nb+1) = exclusive scan of tiles per box; returns the total number of tiles
+static int build_tiles(const int *off, const int *flag, int nb, int tile, DBuf<int> &tileoff, hipStream_t s)
+{
+    DBuf<int> nt((size_t)nb);
+    tileoff.reset((size_t)nb + 1);
+    F3M_LAUNCH(tiles_per_box_kernel, cdiv(nb, 256), 256, 0, s, off, flag, nb, tile, nt.get());
+    check_launch("tiles_per_box");
+    exclusive_scan_i32(nt.get(), nb, tileoff.get(), s);
+    int total = 0;
+    d2h(&total, tileoff.get() + nb, 1, s);
+    return total;
+}
+
+__device__ inline int find_box(const int *__restrict__ tileoff, int nb, int tileid)
+{
+    int lo = 0, hi = nb;   // last b with tileoff[b] <= tileid
+    while (hi - lo > 1) {
+        int mid = lo + ((hi - lo) >> 1);
+        if (tileoff[mid] <= tileid) lo = mid; else hi = mid;
+    }
+    return lo;
+}
+
+// ------------------------------------------------------------------------------------------------
+// near field (F3M_src/1_d_conv.cu:255-335): out_i += sum over the y boxes listed for the box of i of
+// sum_j exp(-|x_i-y_j|^2 lcs) b_j.  One workgroup per (x box, tile of targets); the sources of a y
+// box are staged through LDS already shifted to the x box centre and scaled by sqrt(lcs*log2 e), in
+// the form (2y', -|y'|^2, b), so that a pair costs D fused multiply-adds, one add, one exp2 and one
+// fused multiply-add:  exp2(2x'.y' - |y'|^2 - |x'|^2) b.
+
+constexpr int kNearCap = 512;   // sources per LDS tile
+
+template <int D, int T>
+__global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs, long long N, const float *__restrict__ ys,
+                                                    long long M, const float *__restrict__ bs, float *__restrict__ outs,
+                                                    const int *__restrict__ offx, const int *__restrict__ offy,
+                                                    const float *__restrict__ ctrx, const int *__restrict__ pairs,
+                                                    const int *__restrict__ rowptr, const int *__restrict__ tileoff,
+                                                    int nbx, float sc)
+{
+    constexpr int NV = (D + 1 + 3) / 4;
+    __shared__ float4 sv[NV][kNearCap];
+    __shared__ float sb[kNearCap];
+    const int tid = threadIdx.x, BD = blockDim.x;
+    const int bx = find_box(tileoff, nbx, blockIdx.x);
+    const int tile = blockIdx.x - tileoff[bx];
+    const int x0 = offx[bx] + tile * BD * T, x1 = offx[bx + 1];
+    float cx[D];
+#pragma unroll
+    for (int k = 0; k < D; k++) cx[k] = ctrx[(long long)bx * D + k];
+    float x[T][D], nx2[T], acc[T];
+#pragma unroll
+    for (int r = 0; r < T; r++) {
+        int i = x0 + r * BD + tid;
+        nx2[r] = 0.f;
+        acc[r] = 0.f;
+#pragma unroll
+        for (int k = 0; k < D; k++) {
+            float v = (i < x1) ? xs[(long long)k * N + i] : cx[k];
+            x[r][k] = sc * (v - cx[k]);
+            nx2[r] -= x[r][k] * x[r][k];
+        }
+    }
+    // a wavefront whose lanes all lie past the end of the box only helps with staging
+    const bool wave_live = x0 + (tid & ~(kWave - 1)) < x1;
+    const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    for (int m = m0; m < m1; m++) {
+        const int by = pairs[2 * (long long)m + 1];
+        const int s0 = offy[by], s1 = offy[by + 1];
+        for (int base = s0; base < s1; base += kNearCap) {
+            const int cnt = (s1 - base) < kNearCap ? (s1 - base) : kNearCap;
+            __syncthreads();
+            for (int jj = tid; jj < cnt; jj += BD) {
+                float v[NV * 4];
+                float ny2 = 0.f;
+#pragma unroll
+                for (int k = 0; k < D; k++) {
+                    float y = sc * (ys[(long long)k * M + base + jj] - cx[k]);
+                    v[k] = 2.f * y;
+                    ny2 -= y * y;
+                }
+                v[D] = ny2;
+#pragma unroll
+                for (int k = D + 1; k < NV * 4; k++) v[k] = 0.f;
+#pragma unroll
+                for (int q = 0; q < NV; q++) sv[q][jj] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+                sb[jj] = bs[base + jj];
+            }
+            __syncthreads();
+            if (!wave_live) continue;
+#pragma unroll 4
+            for (int jj = 0; jj < cnt; jj++) {
+                float v[NV * 4];
+#pragma unroll
+                for (int q = 0; q < NV; q++) {
+                    float4 f = sv[q][jj];
+                    v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
+                }
+                const float bj = sb[jj];
+#pragma unroll
+                for (int r = 0; r < T; r++) {
+                    float t = v[D];
+#pragma unroll
+                    for (int k = 0; k < D; k++) t = fmaf(x[r][k], v[k], t);
+                    t += nx2[r];
+                    acc[r] = fmaf(fast_exp2(t), bj, acc[r]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < T; r++) {
+        int i = x0 + r * BD + tid;
+        if (i < x1) outs[i] += acc[r];
+    }
+}
+
+void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
+                const float *bs, float *outs, float lcs, hipStream_t s)
+{
+    if (list.n == 0) return;
+    constexpr int T = 1;
+    // workgroup size: whole boxes where possible (multiple of the wave size, at most 512 lanes)
+    int bd = ((lx.maxcount + kWave - 1) / kWave) * kWave;
+    if (bd > 512) bd = 256;
+    if (bd < kWave) bd = kWave;
+    DBuf<int> flag((size_t)lx.nb), tileoff;
+    F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
+    check_launch("mark_rows");
+    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, bd * T, tileoff, s);
+    if (ntiles == 0) return;
+    float sc = sqrtf(lcs * kLog2e);
+    timer_begin(kNear, s);
+#define F3M_CASE(DD)                                                                                                  \
+    case DD:                                                                                                          \
+        F3M_LAUNCH((near_kernel<DD, T>), ntiles, bd, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs, outs,          \
+                   lx.off.get(), ly.off.get(), lx.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
+                   lx.nb, sc);                                                                                        \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
+    timer_end(s);
+    check_launch("near_field");
+}
+
+// ------------------------------------------------------------------------------------------------
+// interpolation nodes (F3M_src/n_tree.cu:265-349, F3M_src/1_d_conv.cu:850-884)
+
+void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s)
+{
+    ns.d = d;
+    // node counts per dimension (n_tree.cu:328-346); the reference then shuffles the dimensions
+    // at random (:347), which is the identity whenever max_nodes is a perfect d-th power; the order
+    // of :328-346 is kept here
+    float ref_val = (float)pow((double)max_nodes, 1.0 / (double)(float)d);
+    int hi = (int)std::ceil(ref_val), lo = (int)std::floor(ref_val), acc = 1;
+    ns.P = 1;
+    ns.S1 = 0;
+    for (int i = 0; i < d; i++) {
+        int fut = (int)((double)acc * pow((double)lo, (double)(d - (i + 1))) * (double)hi);
+        int pick = fut <= max_nodes ? hi : lo;
+        if (pick < 1) pick = 1;
+        ns.n[i] = pick;
+        acc *= pick;
+        ns.start[i] = ns.S1;
+        ns.S1 += pick;
+        ns.P *= pick;
+    }
+    ns.t.assign(ns.S1, 0.f);
+    ns.w.assign(ns.S1, 0.f);
+    const float PI = (float)(atan(1.) * 4.);
+    for (int j = 0; j < d; j++)
+        for (int i = 0; i < ns.n[j]; i++) {
+            float a = (float)i;
+            a = a * 2.0f;
+            a = a + 1.0f;
+            a = a * PI;
+            a = a / (float)(2 * (ns.n[j] - 1) + 2);
+            ns.t[ns.start[j] + i] = cosf(a);
+            double sgn = (i % 2 == 0) ? 1.0 : -1.0;
+            ns.w[ns.start[j] + i] =
+                (float)(sgn * sin(((2. * (double)(float)i + 1.) * (double)PI) / (2. * (double)(float)(ns.n[j] - 1.0) + 2.)));
+        }
+    ns.dt.reset(ns.S1);
+    ns.dw.reset(ns.S1);
+    h2d(ns.dt.get(), ns.t.data(), ns.S1, s);
+    h2d(ns.dw.get(), ns.w.data(), ns.S1, s);
+    ns.noff.reset((size_t)ns.P * d);
+}
+
+void set_node_offsets(NodeSet &ns, float edge, hipStream_t s)
+{
+    // node position inside a box relative to its centre: cheb*edge/2 + edge/2 (n_tree.cu:510)
+    std::vector<float> h((size_t)ns.P * ns.d);
+    int cum = 1;
+    for (int j = 0; j < ns.d; j++) {
+        for (int m = 0; m < ns.P; m++) {
+            int a = (m / cum) % ns.n[j];
+            float v = ns.t[ns.start[j] + a] * edge;
+            v = v / 2.f;
+            h[(size_t)m * ns.d + j] = v + edge / 2.f;
+        }
+        cum *= ns.n[j];
+    }
+    h2d(ns.noff.get(), h.data(), h.size(), s);
+}
+
+struct NodeMeta {
+    int n[kMaxD];
+    int start[kMaxD];
+    int S1, P;
+};
+
+// 1-D barycentric basis values of one coordinate (F3M_src/1_d_conv.cu:418-448 and :217-238):
+// l_a = (w_a/(t-t_a)) / sum_l w_l/(t-t_l), or the unit vector when t hits a node exactly.
+__device__ inline void basis_1d(float t, const float *__restrict__ nt, const float *__restrict__ nw, int n,
+                                float *__restrict__ out, float scale)
+{
+    float sum = 0.f;
+    int hit = -1;
+    for (int a = 0; a < n; a++) {
+        float diff = t - nt[a];
+        if (diff == 0.f) { hit = a; break; }
+        sum += nw[a] / diff;
+    }
+    if (hit >= 0) {
+        for (int a = 0; a < n; a++) out[a] = (a == hit) ? scale : 0.f;
+    } else {
+        float inv = scale / sum;
+        for (int a = 0; a < n; a++) out[a] = (nw[a] / (t - nt[a])) * inv;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// P2M (F3M_src/1_d_conv.cu:451-552): Mom[box][m] = sum_j L_m(y_j) b_j.  One workgroup per
+// (box, chunk of points), one lane per node; per-chunk partial sums are combined in a fixed order
+// by p2m_reduce_kernel, so the result does not depend on scheduling.
+
+constexpr int kP2MChunk = 512;
+constexpr int kP2MSub = 64;
+
+template <int D>
+__global__ void __launch_bounds__(1024) p2m_kernel(const float *__restrict__ ys, long long M, const float *__restrict__ bs,
+                                                    const int *__restrict__ off, const float *__restrict__ ctr,
+                                                    const int *__restrict__ tileoff, int nb, NodeMeta nm,
+                                                    const float *__restrict__ nt, const float *__restrict__ nw, float factor,
+                                                    float *__restrict__ partial)
+{
+    F3M_DYN_SHARED(float, smem);
+    float *snt = smem;                       // S1
+    float *snw = smem + nm.S1;               // S1
+    float *sl = smem + 2 * nm.S1;            // kP2MSub * S1: per point, per dimension basis values
+    const int tid = threadIdx.x, BD = blockDim.x;
+    const int box = find_box(tileoff, nb, blockIdx.x);
+    const int chunk = blockIdx.x - tileoff[box];
+    const int p0 = off[box] + chunk * kP2MChunk;
+    const int p1 = min(off[box + 1], p0 + kP2MChunk);
+    for (int a = tid; a < nm.S1; a += BD) { snt[a] = nt[a]; snw[a] = nw[a]; }
+    // LDS offsets of this lane's node along every dimension
+    int moff[D];
+    {
+        int rem = tid;
+#pragma unroll
+        for (int k = 0; k < D; k++) { moff[k] = nm.start[k] + rem % nm.n[k]; rem /= nm.n[k]; }
+    }
+    float acc = 0.f;
+    for (int s0 = p0; s0 < p1; s0 += kP2MSub) {
+        const int cnt = min(kP2MSub, p1 - s0);
+        __syncthreads();
+        for (int task = tid; task < cnt * D; task += BD) {
+            int pt = task % cnt, k = task / cnt;
+            float t = factor * (ys[(long long)k * M + s0 + pt] - ctr[(long long)box * D + k]);
+            float scale = (k == 0) ? bs[s0 + pt] : 1.f;      // the weight rides on dimension 0
+            basis_1d(t, snt + nm.start[k], snw + nm.start[k], nm.n[k], sl + pt * nm.S1 + nm.start[k], scale);
+        }
+        __syncthreads();
+        if (tid < nm.P) {
+            for (int pt = 0; pt < cnt; pt++) {
+                const float *row = sl + pt * nm.S1;
+                float v = row[moff[0]];
+#pragma unroll
+                for (int k = 1; k < D; k++) v *= row[moff[k]];
+                acc += v;
+            }
+        }
+    }
+    if (tid < nm.P) partial[(long long)blockIdx.x * nm.P + tid] = acc;
+}
+
+__global__ void p2m_reduce_kernel(const float *__restrict__ partial, const int *__restrict__ tileoff, int nb, int P,
+                                  float *__restrict__ mom)
+{
+    long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= (long long)nb * P) return;
+    int box = (int)(e / P), m = (int)(e % P);
+    float acc = 0.f;
+    for (int t = tileoff[box]; t < tileoff[box + 1]; t++) acc += partial[(long long)t * P + m];
+    mom[e] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// M2L, direct form (F3M_src/1_d_conv.cu:741-817): Loc[bx][i] = sum over far y boxes, sum_m
+// exp(-|(n_i+c_bx)-(n_m+c_by)|^2 lcs) Mom[by][m].  One workgroup per x box, one lane per node.
+
+template <int D>
+__global__ void __launch_bounds__(1024) m2l_direct_kernel(const float *__restrict__ noff, int P, const float *__restrict__ ctrx,
+                                                           const float *__restrict__ ctry, const int *__restrict__ pairs,
+                                                           const int *__restrict__ rowptr, const float *__restrict__ mom,
+                                                           float lcs2, float *__restrict__ loc)
+{
+    F3M_DYN_SHARED(float, smem);
+    float *sy = smem;              // P*D
+    float *sm = smem + P * D;      // P
+    const int bx = blockIdx.x, tid = threadIdx.x;
+    const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    if (m0 == m1) return;          // uniform over the workgroup
+    float x[D], no[D];
+#pragma unroll
+    for (int k = 0; k < D; k++) {
+        no[k] = (tid < P) ? noff[(long long)tid * D + k] : 0.f;
+        x[k] = no[k] + ctrx[(long long)bx * D + k];
+    }
+    float acc = 0.f;
+    for (int m = m0; m < m1; m++) {
+        const int by = pairs[2 * (long long)m + 1];
+        __syncthreads();
+        if (tid < P) {
+#pragma unroll
+            for (int k = 0; k < D; k++) sy[tid * D + k] = no[k] + ctry[(long long)by * D + k];
+            sm[tid] = mom[(long long)by * P + tid];
+        }
+        __syncthreads();
+        if (tid < P) {
+            for (int j = 0; j < P; j++) {
+                float r2 = 0.f;
+#pragma unroll
+                for (int k = 0; k < D; k++) { float t = x[k] - sy[j * D + k]; r2 = fmaf(t, t, r2); }
+                acc = fmaf(fast_exp2(-r2 * lcs2), sm[j], acc);
+            }
+        }
+    }
+    if (tid < P) loc[(long long)bx * P + tid] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// L2P (F3M_src/1_d_conv.cu:554-659): out_i += sum_m L_m(x_i) Loc[box][m].  One lane per point; the
+// product over dimensions >= 1 is reused along dimension 0.
+
+constexpr int kL2PBlock = 128;
+
+template <int D>
+__global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict__ xs, long long N, float *__restrict__ outs,
+                                                         const int *__restrict__ off, const float *__restrict__ ctr,
+                                                         const int *__restrict__ tileoff, int nb, NodeMeta nm,
+                                                         const float *__restrict__ nt, const float *__restrict__ nw,
+                                                         float factor, const float *__restrict__ loc)
+{
+    F3M_DYN_SHARED(float, smem);
+    const int S1p = nm.S1 | 1;               // odd stride: lanes hit distinct LDS banks
+    float *snt = smem;
+    float *snw = smem + nm.S1;
+    float *sloc = smem + 2 * nm.S1;          // P
+    float *sl = sloc + nm.P;                 // kL2PBlock * S1p
+    const int tid = threadIdx.x;
+    const int box = find_box(tileoff, nb, blockIdx.x);
+    const int chunk = blockIdx.x - tileoff[box];
+    const int i = off[box] + chunk * kL2PBlock + tid;
+    const bool live = i < off[box + 1];
+    for (int a = tid; a < nm.S1; a += kL2PBlock) { snt[a] = nt[a]; snw[a] = nw[a]; }
+    for (int m = tid; m < nm.P; m += kL2PBlock) sloc[m] = loc[(long long)box * nm.P + m];
+    __syncthreads();
+    if (!live) return;
+    float *mine = sl + tid * S1p;
+#pragma unroll
+    for (int k = 0; k < D; k++) {
+        float t = factor * (xs[(long long)k * N + i] - ctr[(long long)box * D + k]);
+        basis_1d(t, snt + nm.start[k], snw + nm.start[k], nm.n[k], mine + nm.start[k], 1.f);
+    }
+    int idx[D];
+#pragma unroll
+    for (int k = 0; k < D; k++) idx[k] = 0;
+    float acc = 0.f;
+    const int n0 = nm.n[0];
+    for (int m = 0; m < nm.P; m += n0) {
+        float hi = 1.f;
+#pragma unroll
+        for (int k = 1; k < D; k++) hi *= mine[nm.start[k] + idx[k]];
+        float inner = 0.f;
+        for (int a = 0; a < n0; a++) inner = fmaf(mine[a], sloc[m + a], inner);
+        acc = fmaf(hi, inner, acc);
+        // advance the multi-index of dimensions 1..D-1
+#pragma unroll
+        for (int k = 1; k < D; k++) {
+            idx[k]++;
+            if (idx[k] < nm.n[k]) break;
+            idx[k] = 0;
+        }
+    }
+    outs[i] += acc;
+}
+
+static NodeMeta meta_of(const NodeSet &ns)
+{
+    NodeMeta nm;
+    for (int k = 0; k < kMaxD; k++) { nm.n[k] = ns.n[k] > 0 ? ns.n[k] : 1; nm.start[k] = ns.start[k]; }
+    nm.S1 = ns.S1;
+    nm.P = ns.P;
+    return nm;
+}
+
+void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
+               NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode, float *mom_out, float *loc_out,
+               hipStream_t s)
+{
+    if (far.n == 0) return;
+    const int P = ns.P;
+    F3M_REQUIRE(P <= 1024, 30, "at most 1024 interpolation nodes per box are supported (got %d)", P);
+    (void)m2l_mode;
+    set_node_offsets(ns, lx.edge, s);
+    NodeMeta nm = meta_of(ns);
+    const float factor = 2 / lx.edge;                  // F3M_src/1_d_conv.cu:473
+    // participating boxes: x boxes with a non-empty far row, y boxes that occur in the far list
+    DBuf<int> fx((size_t)lx.nb), fy((size_t)ly.nb);
+    F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, far.rowptr.get(), lx.nb, fx.get());
+    check_launch("mark_rows");
+    F3M_HIP(hipMemsetAsync(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s));
+    F3M_LAUNCH(mark_cols_kernel, cdiv(far.n, 256), 256, 0, s, far.pairs.get(), far.n, fy.get());
+    check_launch("mark_cols");
+
+    // P2M
+    DBuf<int> tiley;
+    int nty = build_tiles(ly.off.get(), fy.get(), ly.nb, kP2MChunk, tiley, s);
+    DBuf<float> partial((size_t)std::max(1, nty) * P), mom((size_t)ly.nb * P), loc((size_t)lx.nb * P);
+    int bdp = ((P + kWave - 1) / kWave) * kWave;
+    size_t shp = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)kP2MSub * ns.S1);
+#define F3M_CASE(DD)                                                                                                   \
+    case DD:                                                                                                           \
+        F3M_LAUNCH((p2m_kernel<DD>), nty, bdp, shp, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(), \
+                   ly.nb, nm, ns.dt.get(), ns.dw.get(), factor, partial.get());                                        \
+        break;
+    if (nty > 0) {
+        timer_begin(kP2M, s);
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
+        check_launch("p2m");
+    }
+#undef F3M_CASE
+    F3M_LAUNCH(p2m_reduce_kernel, cdiv((long long)ly.nb * P, 256), 256, 0, s, partial.get(), tiley.get(), ly.nb, P, mom.get());
+    if (nty > 0) timer_end(s);
+    check_launch("p2m_reduce");
+
+    // M2L
+    F3M_HIP(hipMemsetAsync(loc.get(), 0, sizeof(float) * (size_t)lx.nb * P, s));
+    size_t shm = sizeof(float) * (size_t)P * (d + 1);
+    timer_begin(kM2L, s);
+#define F3M_CASE(DD)                                                                                                   \
+    case DD:                                                                                                           \
+        F3M_LAUNCH((m2l_direct_kernel<DD>), lx.nb, bdp, shm, s, ns.noff.get(), P, lx.ctr.get(), ly.ctr.get(),          \
+                   far.pairs.get(), far.rowptr.get(), mom.get(), lcs * kLog2e, loc.get());                             \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
+    timer_end(s);
+    check_launch("m2l");
+
+    // L2P
+    DBuf<int> tilex;
+    int ntx = build_tiles(lx.off.get(), fx.get(), lx.nb, kL2PBlock, tilex, s);
+    size_t shl = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)P + (size_t)kL2PBlock * (ns.S1 | 1));
+#define F3M_CASE(DD)                                                                                                   \
+    case DD:                                                                                                           \
+        F3M_LAUNCH((l2p_kernel<DD>), ntx, kL2PBlock, shl, s, tx.pts.get(), tx.n, outs, lx.off.get(), lx.ctr.get(),     \
+                   tilex.get(), lx.nb, nm, ns.dt.get(), ns.dw.get(), factor, loc.get());                               \
+        break;
+    if (ntx > 0) {
+        timer_begin(kL2P, s);
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
+        timer_end(s);
+        check_launch("l2p");
+    }
+#undef F3M_CASE
+    if (mom_out) F3M_HIP(hipMemcpyAsync(mom_out, mom.get(), sizeof(float) * (size_t)ly.nb * P, hipMemcpyDeviceToDevice, s));
+    if (loc_out) F3M_HIP(hipMemcpyAsync(loc_out, loc.get(), sizeof(float) * (size_t)lx.nb * P, hipMemcpyDeviceToDevice, s));
+}
+
+}  // namespace f3m

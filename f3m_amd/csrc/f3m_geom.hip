@@ -1,0 +1,617 @@
+// Box division and interaction lists for gfx950.
+//
+// Replaces the reference's per-level hash + atomic histogram + scatter (F3M_src/n_tree.cu:105-179,
+// F3M_src/1_d_conv.cu:1127-1191) by one Morton sort: every point gets the key of its finest cell
+// once, a wavefront-ballot counting sort orders the points, and the boxes of every depth are the
+// runs of equal key prefixes, found by binary search.  The compact box index of the reference
+// equals the rank of the Morton prefix among non-empty boxes, so box ids, counts, centres and the
+// interaction lists come out identical.
+//
+// This file is compiled with -ffp-contract=off: every fp32 operation below rounds exactly once,
+// in the order the reference's tensor code performs it.
+#include "f3m_engine.h"
+
+namespace f3m {
+
+// ------------------------------------------------------------------------------------------------
+// exclusive scan (n inputs, n+1 outputs; out[n] is the total)
+
+constexpr int kScanBlock = 256;
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kScanBlock * kScanItems;
+
+template <typename Tin, typename Tout>
+__global__ void scan_tile_kernel(const Tin *__restrict__ in, long long n, Tout *__restrict__ out, Tout *__restrict__ tilesum)
+{
+    __shared__ Tout sh[kScanBlock];
+    const int tid = threadIdx.x;
+    const long long base = (long long)blockIdx.x * kScanTile + (long long)tid * kScanItems;
+    Tout v[kScanItems];
+    Tout sum = 0;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        long long i = base + e;
+        v[e] = (i < n) ? (Tout)in[i] : (Tout)0;   // element n (the extra output slot) reads as 0
+        sum += v[e];
+    }
+    sh[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanBlock; off <<= 1) {
+        Tout t = (tid >= off) ? sh[tid - off] : (Tout)0;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    Tout run = sh[tid] - sum;   // exclusive prefix of this thread inside the tile
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        long long i = base + e;
+        if (i <= n) out[i] = run;
+        run += v[e];
+    }
+    if (tid == kScanBlock - 1) tilesum[blockIdx.x] = sh[tid];
+}
+
+template <typename Tout>
+__global__ void scan_add_kernel(Tout *__restrict__ out, long long n1, const Tout *__restrict__ tileoff)
+{
+    long long i = (long long)blockIdx.x * kScanTile + threadIdx.x;
+    Tout add = tileoff[blockIdx.x];
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++, i += kScanBlock)
+        if (i < n1) out[i] += add;
+}
+
+template <typename Tin, typename Tout>
+static void exclusive_scan(const Tin *in, long long n, Tout *out, hipStream_t s)
+{
+    long long n1 = n + 1;
+    unsigned ntiles = cdiv(n1, kScanTile);
+    DBuf<Tout> tilesum(ntiles);
+    F3M_LAUNCH((scan_tile_kernel<Tin, Tout>), ntiles, kScanBlock, 0, s, in, n, out, tilesum.get());
+    check_launch("scan_tile");
+    if (ntiles > 1) {
+        DBuf<Tout> tileoff((size_t)ntiles + 1);
+        exclusive_scan<Tout, Tout>(tilesum.get(), ntiles, tileoff.get(), s);
+        F3M_LAUNCH((scan_add_kernel<Tout>), ntiles, kScanBlock, 0, s, out, n1, tileoff.get());
+        check_launch("scan_add");
+    }
+}
+
+void exclusive_scan_i32(const int *in, long long n, int *out, hipStream_t s) { exclusive_scan<int, int>(in, n, out, s); }
+void exclusive_scan_i64(const long long *in, long long n, long long *out, hipStream_t s)
+{
+    exclusive_scan<long long, long long>(in, n, out, s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// bounding box (F3M_src/n_tree.cu:28-31,42-43: per-dimension min and max)
+
+constexpr int kBBGrid = 512;
+
+__global__ void minmax_kernel(const float *__restrict__ X, long long n, int d, float *__restrict__ part)
+{
+    __shared__ float sh[256];
+    float lo[kMaxD], hi[kMaxD];
+    for (int j = 0; j < kMaxD; j++) { lo[j] = INFINITY; hi[j] = -INFINITY; }
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        for (int j = 0; j < d; j++) {
+            float v = X[i * d + j];
+            lo[j] = fminf(lo[j], v);
+            hi[j] = fmaxf(hi[j], v);
+        }
+    for (int j = 0; j < d; j++)
+        for (int pass = 0; pass < 2; pass++) {
+            sh[threadIdx.x] = pass ? hi[j] : lo[j];
+            __syncthreads();
+            for (int off = 128; off > 0; off >>= 1) {
+                if ((int)threadIdx.x < off) {
+                    float a = sh[threadIdx.x], b = sh[threadIdx.x + off];
+                    sh[threadIdx.x] = pass ? fmaxf(a, b) : fminf(a, b);
+                }
+                __syncthreads();
+            }
+            if (threadIdx.x == 0) part[((long long)blockIdx.x * 2 + pass) * kMaxD + j] = sh[0];
+            __syncthreads();
+        }
+}
+
+void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s)
+{
+    unsigned grid = cdiv(n, 256);
+    if (grid > kBBGrid) grid = kBBGrid;
+    DBuf<float> part((size_t)grid * 2 * kMaxD);
+    F3M_LAUNCH(minmax_kernel, grid, 256, 0, s, X, n, d, part.get());
+    check_launch("minmax");
+    std::vector<float> h((size_t)grid * 2 * kMaxD);
+    d2h(h.data(), part.get(), h.size(), s);
+    for (int j = 0; j < d; j++) {
+        mn[j] = h[j];
+        mx[j] = h[kMaxD + j];
+        for (unsigned b = 1; b < grid; b++) {
+            mn[j] = fminf(mn[j], h[((size_t)b * 2) * kMaxD + j]);
+            mx[j] = fmaxf(mx[j], h[((size_t)b * 2 + 1) * kMaxD + j]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Morton keys.  Cell of a point at the key depth L, per dimension (F3M_src/1_d_conv.cu:1142-1144):
+//   g_j = (int) floor( (2^L * (x_j - origin_j)) / edge0 )
+// Scaling by a power of two commutes with rounding, so the cell at depth k <= L is g_j >> (L-k):
+// one key serves every level.  Key = child digits, coarsest level first; the digit of a level has
+// bit j set when the point lies in the upper half along dimension j (sign table of
+// F3M_src/1_d_conv.cu:895-897), which makes the natural child index of the reference the digit.
+
+__global__ void morton_kernel(const float *__restrict__ X, long long n, Geo g, uint32_t *__restrict__ keys, int *__restrict__ idx)
+{
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float side = (float)(1u << g.L);
+    const int top = (1 << g.L) - 1;
+    int cell[kMaxD];
+    for (int j = 0; j < g.d; j++) {
+        float a = X[i * g.d + j] - g.origin[j];
+        float q = side * a;
+        q = q / g.edge0;
+        int c = (int)floorf(q);
+        cell[j] = c < 0 ? 0 : (c > top ? top : c);
+    }
+    uint32_t key = 0;
+    for (int l = g.L - 1; l >= 0; l--) {
+        uint32_t digit = 0;
+        for (int j = 0; j < g.d; j++) digit |= (uint32_t)((cell[j] >> l) & 1) << j;
+        key = (key << g.d) | digit;
+    }
+    keys[i] = key;
+    idx[i] = (int)i;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Counting sort by 8-bit digits, least significant first; stable.  One wavefront per workgroup:
+// inside a round of 64 keys the rank of a key among equal digits comes from eight ballots, and
+// the running digit offsets live in LDS.
+
+constexpr int kSortRounds = 32;
+constexpr int kSortTile = kWave * kSortRounds;
+
+__global__ void __launch_bounds__(64) sort_hist_kernel(const uint32_t *__restrict__ keys, long long n, int shift,
+                                                         int *__restrict__ blockhist, int nblk)
+{
+    __shared__ int hist[256];
+    const int lane = threadIdx.x;
+    for (int b = lane; b < 256; b += kWave) hist[b] = 0;
+    __syncthreads();
+    const long long base = (long long)blockIdx.x * kSortTile;
+    for (int r = 0; r < kSortRounds; r++) {
+        long long i = base + r * kWave + lane;
+        if (i < n) atomicAdd(&hist[(keys[i] >> shift) & 255u], 1);
+    }
+    __syncthreads();
+    for (int b = lane; b < 256; b += kWave) blockhist[(long long)b * nblk + blockIdx.x] = hist[b];
+}
+
+__global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__restrict__ keys_in, const int *__restrict__ idx_in,
+                                                            uint32_t *__restrict__ keys_out, int *__restrict__ idx_out,
+                                                            long long n, int shift, const int *__restrict__ base, int nblk)
+{
+    __shared__ int run[256];
+    const int lane = threadIdx.x;
+    for (int b = lane; b < 256; b += kWave) run[b] = base[(long long)b * nblk + blockIdx.x];
+    __syncthreads();
+    const long long tile = (long long)blockIdx.x * kSortTile;
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    for (int r = 0; r < kSortRounds; r++) {
+        long long i = tile + r * kWave + lane;
+        bool valid = i < n;
+        uint32_t key = valid ? keys_in[i] : 0u;
+        int val = valid ? idx_in[i] : 0;
+        uint32_t digit = (key >> shift) & 255u;
+        unsigned long long same = wave_ballot(valid);
+#pragma unroll
+        for (int bit = 0; bit < 8; bit++) {
+            bool one = (digit >> bit) & 1u;
+            unsigned long long m = wave_ballot(one);
+            same &= one ? m : ~m;
+        }
+        int rank = __popcll(same & below);
+        int start = valid ? run[digit] : 0;
+        __syncthreads();
+        if (valid && rank == 0) run[digit] = start + __popcll(same);
+        __syncthreads();
+        if (valid) {
+            keys_out[start + rank] = key;
+            idx_out[start + rank] = val;
+        }
+    }
+}
+
+static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int bits, hipStream_t s)
+{
+    int nblk = (int)cdiv(n, kSortTile);
+    DBuf<uint32_t> keys2((size_t)n);
+    DBuf<int> idx2((size_t)n);
+    DBuf<int> hist((size_t)256 * nblk);
+    DBuf<int> base((size_t)256 * nblk + 1);
+    for (int shift = 0; shift < bits; shift += 8) {
+        F3M_LAUNCH(sort_hist_kernel, nblk, kWave, 0, s, keys.get(), n, shift, hist.get(), nblk);
+        check_launch("sort_hist");
+        exclusive_scan_i32(hist.get(), (long long)256 * nblk, base.get(), s);
+        F3M_LAUNCH(sort_scatter_kernel, nblk, kWave, 0, s, keys.get(), idx.get(), keys2.get(), idx2.get(), n, shift,
+                   base.get(), nblk);
+        check_launch("sort_scatter");
+        std::swap(keys, keys2);
+        std::swap(idx, idx2);
+    }
+}
+
+void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s)
+{
+    t.geo = geo;
+    t.n = n;
+    t.keys.reset((size_t)n);
+    t.perm.reset((size_t)n);
+    F3M_LAUNCH(morton_kernel, cdiv(n, 256), 256, 0, s, X, n, geo, t.keys.get(), t.perm.get());
+    check_launch("morton");
+    radix_sort(t.keys, t.perm, n, geo.d * geo.L, s);
+    t.pts.reset((size_t)n * geo.d);
+    gather_points(X, t.perm.get(), n, geo.d, t.pts.get(), s);
+    // root level (F3M_src/n_tree.cu:86-95)
+    t.lev.clear();
+    t.lev.reserve(40);
+    t.lev.emplace_back();
+    TreeLevel &r = t.lev[0];
+    r.depth = 0;
+    r.edge = geo.edge0;
+    r.nb = 1;
+    r.maxcount = (int)n;
+    r.off.reset(2);
+    r.prefix.reset(1);
+    r.ctr.reset(geo.d);
+    int off[2] = {0, (int)n};
+    uint32_t pf = 0;
+    float c[kMaxD];
+    float half = 0.5f * geo.edge0;
+    for (int j = 0; j < geo.d; j++) c[j] = geo.origin[j] + half;
+    h2d(r.off.get(), off, 2, s);
+    h2d(r.prefix.get(), &pf, 1, s);
+    h2d(r.ctr.get(), c, geo.d, s);
+}
+
+// ------------------------------------------------------------------------------------------------
+// One division (F3M_src/n_tree.cu:98-179).  Candidates are the 2^d children of every box, natural
+// index = parent*2^d + child; their point ranges are found by binary search in the sorted keys.
+
+__global__ void child_bounds_kernel(const uint32_t *__restrict__ keys, const uint32_t *__restrict__ prefix_prev,
+                                    const int *__restrict__ off_prev, long long ncand, int d, int shift, long long n,
+                                    int *__restrict__ natpos)
+{
+    long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (nat > ncand) return;
+    if (nat == ncand) { natpos[nat] = (int)n; return; }
+    int q = (int)(nat >> d);
+    uint32_t target = (prefix_prev[q] << d) | (uint32_t)(nat & ((1 << d) - 1));
+    int lo = off_prev[q], hi = off_prev[q + 1];
+    while (lo < hi) {
+        int mid = lo + ((hi - lo) >> 1);
+        if ((keys[mid] >> shift) < target) lo = mid + 1; else hi = mid;
+    }
+    natpos[nat] = lo;
+}
+
+__global__ void nonempty_kernel(const int *__restrict__ natpos, long long ncand, int *__restrict__ flag)
+{
+    long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (nat < ncand) flag[nat] = natpos[nat + 1] > natpos[nat] ? 1 : 0;
+}
+
+// stats[0] = number of non-empty children, stats[1] = largest count
+__global__ void build_level_kernel(const int *__restrict__ natpos, const int *__restrict__ cid, long long ncand, int d,
+                                   const uint32_t *__restrict__ prefix_prev, const float *__restrict__ ctr_prev,
+                                   float quarter, int *__restrict__ off, uint32_t *__restrict__ prefix,
+                                   float *__restrict__ ctr, int *__restrict__ childstart_prev, int *__restrict__ stats)
+{
+    long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (nat > ncand) return;
+    int id = cid[nat];
+    int q = (int)(nat >> d);
+    int child = (int)(nat & ((1 << d) - 1));
+    if (nat == ncand) {
+        off[id] = natpos[nat];
+        childstart_prev[q] = id;
+        stats[0] = id;
+        return;
+    }
+    if (child == 0) childstart_prev[q] = id;
+    int cnt = natpos[nat + 1] - natpos[nat];
+    if (cnt > 0) {
+        off[id] = natpos[nat];
+        prefix[id] = (prefix_prev[q] << d) | (uint32_t)child;
+        for (int j = 0; j < d; j++) {
+            float step = ((child >> j) & 1) ? quarter : -quarter;      // 0.25*edge*sign, exact
+            ctr[(long long)id * d + j] = ctr_prev[(long long)q * d + j] + step;
+        }
+        atomicMax(&stats[1], cnt);
+    }
+}
+
+bool divide_tree(Tree &t, hipStream_t s)
+{
+    const int d = t.geo.d;
+    const int k = (int)t.lev.size();   // depth being built
+    if (k > t.geo.L) return false;
+    TreeLevel &prev = t.lev[k - 1];
+    long long ncand = (long long)prev.nb << d;
+    F3M_REQUIRE(ncand < (1ll << 31) - 2, 20, "too many candidate boxes at depth %d (%lld)", k, ncand);
+    DBuf<int> natpos((size_t)ncand + 1), flag((size_t)ncand), cid((size_t)ncand + 1), stats(2);
+    int shift = d * (t.geo.L - k);
+    F3M_LAUNCH(child_bounds_kernel, cdiv(ncand + 1, 256), 256, 0, s, t.keys.get(), prev.prefix.get(), prev.off.get(), ncand,
+               d, shift, t.n, natpos.get());
+    check_launch("child_bounds");
+    F3M_LAUNCH(nonempty_kernel, cdiv(ncand, 256), 256, 0, s, natpos.get(), ncand, flag.get());
+    check_launch("nonempty");
+    exclusive_scan_i32(flag.get(), ncand, cid.get(), s);
+    size_t bound = (size_t)std::min<long long>(ncand, t.n);
+    TreeLevel cur;
+    cur.depth = k;
+    cur.off.reset(bound + 1);
+    cur.prefix.reset(bound);
+    cur.ctr.reset(bound * d);
+    prev.childstart.reset((size_t)prev.nb + 1);
+    F3M_HIP(hipMemsetAsync(stats.get(), 0, 2 * sizeof(int), s));
+    float quarter = 0.25f * prev.edge;
+    F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
+               prev.ctr.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), prev.childstart.get(), stats.get());
+    check_launch("build_level");
+    int h[2];
+    d2h(h, stats.get(), 2, s);
+    cur.nb = h[0];
+    cur.maxcount = h[1];
+    cur.edge = prev.edge * 0.5f;
+    t.lev.push_back(std::move(cur));
+    return true;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Interaction lists of depth k from the keep list of depth k-1
+// (F3M_src/n_tree.cu:594-641 expansion, 788-811 filter, 701-787 + F3M_src/1_d_conv.cu:903-1029 classes).
+// Children of a keep pair (x,y) are enumerated in the reference's order (x, child of x, y, child of
+// y); only non-empty children exist here, so the filter step is implicit.
+
+__global__ void keep_rows_kernel(const int *__restrict__ pairs, long long nk, const int *__restrict__ csy,
+                                 long long *__restrict__ wy, int *__restrict__ rowflag)
+{
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nk) return;
+    int y = pairs[2 * t + 1];
+    wy[t] = csy[y + 1] - csy[y];
+    rowflag[t] = (t == 0 || pairs[2 * t] != pairs[2 * (t - 1)]) ? 1 : 0;
+}
+
+__global__ void row_starts_kernel(const int *__restrict__ rowflag, const int *__restrict__ rowexcl, long long nk,
+                                  int *__restrict__ rowstart)
+{
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t > nk) return;
+    if (t == nk) { rowstart[rowexcl[nk]] = (int)nk; return; }
+    if (rowflag[t]) rowstart[rowexcl[t]] = (int)t;
+}
+
+__global__ void row_cand_kernel(const int *__restrict__ rowstart, const int *__restrict__ rowexcl, long long nk,
+                                const int *__restrict__ pairs, const int *__restrict__ csx, const long long *__restrict__ W,
+                                long long *__restrict__ rowcand)
+{
+    long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= nk) return;
+    int nrows = rowexcl[nk];
+    if (r >= nrows) { rowcand[r] = 0; return; }
+    int t0 = rowstart[r], t1 = rowstart[r + 1];
+    int x = pairs[2 * (long long)t0];
+    rowcand[r] = (long long)(csx[x + 1] - csx[x]) * (W[t1] - W[t0]);
+}
+
+// 0 small, 1 far, 2 keep, 3 dropped (F3M_src/1_d_conv.cu:927-952 and :983-1026)
+__device__ inline int classify_pair(const float *__restrict__ cx, const float *__restrict__ cy, int d, int size,
+                                    const ClassifyParams &cp)
+{
+    if (cp.do_init && size < 2 * cp.nr_interp) return 0;
+    float acc = 0.f;
+    for (int j = 0; j < d; j++) {
+        float dk = cy[j] - cx[j];
+        float sq = dk * dk;
+        acc = acc + sq;
+    }
+    float dist = sqrtf(acc);
+    float thr = cp.edge * 2.f;
+    if (dist >= thr) return cp.do_init ? 1 : 3;
+    if (cp.var_comp) {
+        float v = dist * dist;
+        v = v * cp.lcs;
+        if (cp.en_pair && (double)v <= 1e-2) return 1;
+        if (cp.en_all && dist <= cp.crit) return 1;
+    }
+    if (size < 2 * cp.small_limit) return 0;
+    return 2;
+}
+
+__global__ void expand_classify_kernel(long long T, const long long *__restrict__ B, const int *__restrict__ rowexcl,
+                                       long long nk, const int *__restrict__ rowstart, const int *__restrict__ pairs,
+                                       const long long *__restrict__ W, const int *__restrict__ csx,
+                                       const int *__restrict__ csy, const int *__restrict__ offx,
+                                       const int *__restrict__ offy, const float *__restrict__ ctrx,
+                                       const float *__restrict__ ctry, int d, ClassifyParams cp,
+                                       int *__restrict__ cand, unsigned char *__restrict__ cls)
+{
+    long long pos = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (pos >= T) return;
+    int nrows = rowexcl[nk];
+    // last row r with B[r] <= pos
+    int lo = 0, hi = nrows;
+    while (hi - lo > 1) {
+        int mid = lo + ((hi - lo) >> 1);
+        if (B[mid] <= pos) lo = mid; else hi = mid;
+    }
+    int r = lo;
+    long long rem = pos - B[r];
+    int t0 = rowstart[r], t1 = rowstart[r + 1];
+    long long w0 = W[t0];
+    long long R = W[t1] - w0;
+    int ci = (int)(rem / R);
+    long long rem2 = rem - (long long)ci * R;
+    int a = t0, b = t1;
+    while (b - a > 1) {
+        int mid = a + ((b - a) >> 1);
+        if (W[mid] - w0 <= rem2) a = mid; else b = mid;
+    }
+    int t = a;
+    int cj = (int)(rem2 - (W[t] - w0));
+    int x = pairs[2 * (long long)t], y = pairs[2 * (long long)t + 1];
+    int bx = csx[x] + ci, by = csy[y] + cj;
+    int size = (offx[bx + 1] - offx[bx]) + (offy[by + 1] - offy[by]);
+    cand[2 * pos] = bx;
+    cand[2 * pos + 1] = by;
+    cls[pos] = (unsigned char)classify_pair(ctrx + (long long)bx * d, ctry + (long long)by * d, d, size, cp);
+}
+
+// order-preserving three-way split
+constexpr int kSplitBlock = 256;
+constexpr int kSplitItems = 4;
+constexpr int kSplitTile = kSplitBlock * kSplitItems;
+
+__global__ void split_count_kernel(const unsigned char *__restrict__ cls, long long T, long long *__restrict__ blockcnt,
+                                   long long nblk)
+{
+    __shared__ int cnt[3];
+    if (threadIdx.x < 3) cnt[threadIdx.x] = 0;
+    __syncthreads();
+    long long base = (long long)blockIdx.x * kSplitTile + (long long)threadIdx.x * kSplitItems;
+    int c0 = 0, c1 = 0, c2 = 0;
+    for (int e = 0; e < kSplitItems; e++) {
+        long long i = base + e;
+        if (i < T) {
+            int c = cls[i];
+            c0 += c == 0; c1 += c == 1; c2 += c == 2;
+        }
+    }
+    if (c0) atomicAdd(&cnt[0], c0);
+    if (c1) atomicAdd(&cnt[1], c1);
+    if (c2) atomicAdd(&cnt[2], c2);
+    __syncthreads();
+    if (threadIdx.x < 3) blockcnt[(long long)threadIdx.x * nblk + blockIdx.x] = cnt[threadIdx.x];
+}
+
+__global__ void split_scatter_kernel(const unsigned char *__restrict__ cls, const int *__restrict__ cand, long long T,
+                                     const long long *__restrict__ off0, const long long *__restrict__ off1,
+                                     const long long *__restrict__ off2, int *__restrict__ out_small,
+                                     int *__restrict__ out_far, int *__restrict__ out_keep)
+{
+    // per-thread class counts packed 3 x 21 bits, scanned across the block
+    __shared__ unsigned long long sh[kSplitBlock];
+    const int tid = threadIdx.x;
+    long long base = (long long)blockIdx.x * kSplitTile + (long long)tid * kSplitItems;
+    int c[kSplitItems];
+    unsigned long long mine = 0;
+    for (int e = 0; e < kSplitItems; e++) {
+        long long i = base + e;
+        c[e] = (i < T) ? (int)cls[i] : 3;
+        if (c[e] < 3) mine += 1ull << (21 * c[e]);
+    }
+    sh[tid] = mine;
+    __syncthreads();
+    for (int off = 1; off < kSplitBlock; off <<= 1) {
+        unsigned long long t = (tid >= off) ? sh[tid - off] : 0ull;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    unsigned long long excl = sh[tid] - mine;
+    long long p0 = off0[blockIdx.x] + (long long)(excl & 0x1fffff);
+    long long p1 = off1[blockIdx.x] + (long long)((excl >> 21) & 0x1fffff);
+    long long p2 = off2[blockIdx.x] + (long long)((excl >> 42) & 0x1fffff);
+    for (int e = 0; e < kSplitItems; e++) {
+        long long i = base + e;
+        if (c[e] == 0) { out_small[2 * p0] = cand[2 * i]; out_small[2 * p0 + 1] = cand[2 * i + 1]; p0++; }
+        else if (c[e] == 1) { out_far[2 * p1] = cand[2 * i]; out_far[2 * p1 + 1] = cand[2 * i + 1]; p1++; }
+        else if (c[e] == 2) { out_keep[2 * p2] = cand[2 * i]; out_keep[2 * p2 + 1] = cand[2 * i + 1]; p2++; }
+    }
+}
+
+__global__ void rowptr_kernel(const int *__restrict__ pairs, long long n, int nbx, int *__restrict__ rowptr)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b > nbx) return;
+    long long lo = 0, hi = n;
+    while (lo < hi) {
+        long long mid = lo + ((hi - lo) >> 1);
+        if (pairs[2 * mid] < b) lo = mid + 1; else hi = mid;
+    }
+    rowptr[b] = (int)lo;
+}
+
+void build_rowptr(PairList &l, int nbx, hipStream_t s)
+{
+    l.rowptr.reset((size_t)nbx + 1);
+    F3M_LAUNCH(rowptr_kernel, cdiv((long long)nbx + 1, 256), 256, 0, s, l.pairs.get(), l.n, nbx, l.rowptr.get());
+    check_launch("rowptr");
+}
+
+void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+                  PlanLevel &out, hipStream_t s)
+{
+    const int d = tx.geo.d;
+    const long long nk = keep_prev.n;
+    const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
+    const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
+    out.far.n = out.small_.n = out.keep.n = 0;
+    if (nk == 0) return;
+    F3M_REQUIRE(nk < (1ll << 31) - 2, 21, "keep list too long (%lld)", nk);
+    DBuf<long long> wy((size_t)nk), W((size_t)nk + 1), rowcand((size_t)nk), B((size_t)nk + 1);
+    DBuf<int> rowflag((size_t)nk), rowexcl((size_t)nk + 1), rowstart((size_t)nk + 1);
+    F3M_LAUNCH(keep_rows_kernel, cdiv(nk, 256), 256, 0, s, keep_prev.pairs.get(), nk, py.childstart.get(), wy.get(),
+               rowflag.get());
+    check_launch("keep_rows");
+    exclusive_scan_i64(wy.get(), nk, W.get(), s);
+    exclusive_scan_i32(rowflag.get(), nk, rowexcl.get(), s);
+    F3M_LAUNCH(row_starts_kernel, cdiv(nk + 1, 256), 256, 0, s, rowflag.get(), rowexcl.get(), nk, rowstart.get());
+    check_launch("row_starts");
+    F3M_LAUNCH(row_cand_kernel, cdiv(nk, 256), 256, 0, s, rowstart.get(), rowexcl.get(), nk, keep_prev.pairs.get(),
+               px.childstart.get(), W.get(), rowcand.get());
+    check_launch("row_cand");
+    exclusive_scan_i64(rowcand.get(), nk, B.get(), s);
+    long long T = 0;
+    d2h(&T, B.get() + nk, 1, s);
+    if (T == 0) return;
+    F3M_REQUIRE(T < (1ll << 40), 22, "candidate list too long (%lld)", T);
+    DBuf<int> cand((size_t)T * 2);
+    DBuf<unsigned char> cls((size_t)T);
+    F3M_LAUNCH(expand_classify_kernel, cdiv(T, 256), 256, 0, s, T, B.get(), rowexcl.get(), nk, rowstart.get(),
+               keep_prev.pairs.get(), W.get(), px.childstart.get(), py.childstart.get(), lx.off.get(), ly.off.get(),
+               lx.ctr.get(), ly.ctr.get(), d, cp, cand.get(), cls.get());
+    check_launch("expand_classify");
+    long long nblk = (T + kSplitTile - 1) / kSplitTile;
+    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1);
+    F3M_LAUNCH(split_count_kernel, nblk, kSplitBlock, 0, s, cls.get(), T, blockcnt.get(), nblk);
+    check_launch("split_count");
+    exclusive_scan_i64(blockcnt.get(), nblk, off0.get(), s);
+    exclusive_scan_i64(blockcnt.get() + nblk, nblk, off1.get(), s);
+    exclusive_scan_i64(blockcnt.get() + 2 * nblk, nblk, off2.get(), s);
+    long long tot[3];
+    d2h(&tot[0], off0.get() + nblk, 1, s);
+    d2h(&tot[1], off1.get() + nblk, 1, s);
+    d2h(&tot[2], off2.get() + nblk, 1, s);
+    out.small_.n = tot[0];
+    out.far.n = tot[1];
+    out.keep.n = tot[2];
+    out.small_.pairs.reset((size_t)std::max<long long>(1, tot[0]) * 2);
+    out.far.pairs.reset((size_t)std::max<long long>(1, tot[1]) * 2);
+    out.keep.pairs.reset((size_t)std::max<long long>(1, tot[2]) * 2);
+    F3M_LAUNCH(split_scatter_kernel, nblk, kSplitBlock, 0, s, cls.get(), cand.get(), T, off0.get(), off1.get(), off2.get(),
+               out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get());
+    check_launch("split_scatter");
+    if (out.small_.n) build_rowptr(out.small_, lx.nb, s);
+    if (out.far.n) build_rowptr(out.far, lx.nb, s);
+    if (out.keep.n) build_rowptr(out.keep, lx.nb, s);
+    F3M_HIP(hipStreamSynchronize(s));   // temporaries above return to the pool only after their kernels ran
+}
+
+}  // namespace f3m

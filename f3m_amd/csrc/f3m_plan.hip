@@ -1,0 +1,546 @@
+// Host orchestration (the level loop of F3M_src/n_tree.cu:1056-1125) and the C ABI of include/f3m.h.
+#include "../../include/f3m.h"
+#include "f3m_engine.h"
+
+#include <cmath>
+#include <memory>
+
+namespace f3m {
+
+// ---- stage timing ----------------------------------------------------------------------------
+#ifndef F3M_CPU_EMU
+struct StageTimer {
+    bool enabled = false;
+    struct Span { int stage; hipEvent_t a, b; };
+    std::vector<Span> spans;
+    double t[kNumStages] = {0};
+    int n[kNumStages] = {0};
+    void begin(int stage, hipStream_t s)
+    {
+        if (!enabled) return;
+        Span sp{stage, nullptr, nullptr};
+        F3M_HIP(hipEventCreate(&sp.a));
+        F3M_HIP(hipEventCreate(&sp.b));
+        F3M_HIP(hipEventRecord(sp.a, s));
+        spans.push_back(sp);
+    }
+    void end(hipStream_t s)
+    {
+        if (!enabled || spans.empty()) return;
+        F3M_HIP(hipEventRecord(spans.back().b, s));
+    }
+    void reset()
+    {
+        for (auto &sp : spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
+        spans.clear();
+        for (int i = 0; i < kNumStages; i++) { t[i] = 0; n[i] = 0; }
+    }
+    void collect()
+    {
+        if (!enabled) return;
+        for (auto &sp : spans) {
+            float ms = 0.f;
+            if (hipEventSynchronize(sp.b) == hipSuccess && hipEventElapsedTime(&ms, sp.a, sp.b) == hipSuccess) {
+                t[sp.stage] += ms * 1e-3;
+                n[sp.stage] += 1;
+            }
+            (void)hipEventDestroy(sp.a);
+            (void)hipEventDestroy(sp.b);
+        }
+        spans.clear();
+    }
+};
+#else
+struct StageTimer {
+    bool enabled = false;
+    double t[kNumStages] = {0};
+    int n[kNumStages] = {0};
+    void begin(int, hipStream_t) {}
+    void end(hipStream_t) {}
+    void reset() {}
+    void collect() {}
+};
+#endif
+static thread_local StageTimer g_timer;
+static thread_local std::string g_error;
+
+struct Scope {
+    hipStream_t s;
+    Scope(int stage, hipStream_t st) : s(st) { g_timer.begin(stage, s); }
+    ~Scope() { g_timer.end(s); }
+};
+
+}  // namespace f3m
+
+using namespace f3m;
+
+struct f3m_plan {
+    int d = 0;
+    bool symmetric = true;
+    long long N = 0, M = 0;
+    f3m_params prm{};
+    float lcs = 0.f;
+    Tree tx, ty_;
+    Tree *ty = nullptr;
+    std::vector<PlanLevel> levels;         // levels[k-1] = depth k
+    std::map<int, std::unique_ptr<NodeSet>> nodes;
+    DBuf<float> Xraw, Yraw;                // row-major copies, only when no division happened
+    NodeSet &nodeset(int num_nodes, hipStream_t s)
+    {
+        auto it = nodes.find(num_nodes);
+        if (it == nodes.end()) {
+            std::unique_ptr<NodeSet> ns(new NodeSet());
+            make_nodes(*ns, d, num_nodes, s);
+            it = nodes.emplace(num_nodes, std::move(ns)).first;
+        }
+        return *it->second;
+    }
+};
+
+namespace f3m {
+
+static void check_params(int d, long long N, long long M, bool sym, const f3m_params *p)
+{
+    F3M_REQUIRE(p != nullptr, 1, "params is NULL");
+    F3M_REQUIRE(d >= 1 && d <= kMaxD, 2, "dimension must be 1..10 (got %d)", d);
+    F3M_REQUIRE(N >= 1, 3, "X has no rows");
+    F3M_REQUIRE(sym || M >= 1, 3, "Y has no rows");
+    F3M_REQUIRE(N < (1ll << 31) - 1 && M < (1ll << 31) - 1, 4, "at most 2^31-2 points per side");
+    F3M_REQUIRE(p->ls > 0.f && std::isfinite(p->ls), 5, "ls must be positive");
+    F3M_REQUIRE(p->nr_of_interpolation >= 1, 6, "nr_of_interpolation must be >= 1");
+    F3M_REQUIRE(p->small_field_points >= 0, 7, "small_field_points must be >= 0");
+}
+
+static void check_device_ptr(const void *p, const char *name)
+{
+    F3M_REQUIRE(p != nullptr, 8, "%s is NULL", name);
+#ifndef F3M_CPU_EMU
+    hipPointerAttribute_t a;
+    hipError_t e = hipPointerGetAttributes(&a, p);
+    if (e != hipSuccess) { (void)hipGetLastError(); throw Error(9, fmt("%s is not a device pointer", name)); }
+    F3M_REQUIRE(a.type == hipMemoryTypeDevice || a.type == hipMemoryTypeManaged, 9, "%s is not device memory", name);
+#endif
+}
+
+static float root_edge(const float *mn, const float *mx, int d)
+{
+    float e = mx[0] - mn[0];
+    for (int j = 1; j < d; j++) { float r = mx[j] - mn[j]; if (r > e) e = r; }
+    return e;
+}
+
+static ClassifyParams classify_params(const f3m_plan &P, float edge)
+{
+    ClassifyParams cp;
+    cp.nr_interp = P.prm.nr_of_interpolation;
+    cp.small_limit = P.prm.small_field_points;
+    cp.var_comp = P.prm.var_compression ? 1 : 0;
+    cp.lcs = P.lcs;
+    cp.edge = edge;
+    cp.do_init = 1; cp.en_pair = 0; cp.en_all = 0; cp.crit = 0.f;
+    if (cp.var_comp) {
+        // thresholds of F3M_src/n_tree.cu:728-743; the "ls" there is 1/(2 ls^2) (n_tree.cu:1083)
+        float sq = edge * edge * P.lcs;
+        float eff = P.prm.eff_var_limit;
+        cp.do_init = sq <= 5;
+        cp.en_pair = ((float)P.d * sq / 4) <= eff;
+        cp.en_all = ((float)P.d * sq / 4) <= (eff / 2);
+        cp.crit = sqrtf(eff * 2 / ((float)P.d * P.lcs));
+    }
+    return cp;
+}
+
+static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y, long long M, const f3m_params *prm,
+                             hipStream_t s)
+{
+    bool sym = (Y == nullptr || Y == X);
+    check_params(d, N, M, sym, prm);
+    check_device_ptr(X, "X");
+    if (!sym) check_device_ptr(Y, "Y");
+    std::unique_ptr<f3m_plan> P(new f3m_plan());
+    P->d = d; P->symmetric = sym; P->N = N; P->M = sym ? N : M; P->prm = *prm;
+    P->lcs = 1 / (2 * prm->ls * prm->ls);                        // F3M_src/n_tree.cu:1060
+    P->ty = sym ? &P->tx : &P->ty_;
+    Scope sc(kPlan, s);
+
+    // root geometry (F3M_src/n_tree.cu:25-46)
+    float xmn[kMaxD], xmx[kMaxD], ymn[kMaxD], ymx[kMaxD];
+    bounding_box(X, N, d, xmn, xmx, s);
+    float edge = root_edge(xmn, xmx, d);
+    if (!sym) {
+        bounding_box(Y, M, d, ymn, ymx, s);
+        float ye = root_edge(ymn, ymx, d);
+        if (ye > edge) edge = ye;
+    }
+    Geo gx;
+    memset(&gx, 0, sizeof(gx));
+    gx.d = d;
+    gx.edge0 = edge * 1.01f;
+    F3M_REQUIRE(gx.edge0 > 0.f && std::isfinite(gx.edge0), 10, "degenerate point cloud (edge %g)", (double)gx.edge0);
+    // key depth: past 31/d levels the reference's int32 grid keys overflow, past 16 its fp32 centres
+    // stop resolving cells; the tree is never deeper and what is left is summed exactly
+    gx.L = std::min(31 / d, 16);
+    Geo gy = gx;
+    for (int j = 0; j < d; j++) { gx.origin[j] = xmn[j]; gy.origin[j] = sym ? xmn[j] : ymn[j]; }
+    build_sorted_tree(P->tx, X, N, gx, s);
+    if (!sym) build_sorted_tree(P->ty_, Y, M, gy, s);
+
+    PairList root;
+    root.n = 1;
+    root.pairs.reset(2);
+    int zero2[2] = {0, 0};
+    h2d(root.pairs.get(), zero2, 2, s);
+    const PairList *keep = &root;
+    P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
+    // loop guard of F3M_src/n_tree.cu:1075 (symmetric) and :1099 (two trees)
+    while (keep->n > 0 && (float)P->tx.lev.back().maxcount > prm->min_points &&
+           (sym || (float)P->ty_.lev.back().maxcount > prm->min_points)) {
+        if ((int)P->tx.lev.size() > gx.L) break;
+        divide_tree(P->tx, s);
+        if (!sym) divide_tree(P->ty_, s);
+        int k = (int)P->tx.lev.size() - 1;
+        float e = P->tx.lev[k].edge;
+        P->levels.emplace_back();
+        PlanLevel &L = P->levels.back();
+        expand_lists(*keep, P->tx, *P->ty, k, classify_params(*P, e), L, s);
+        L.num_nodes = prm->nr_of_interpolation;
+        if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
+            L.num_nodes = std::min((int)pow(3, d), prm->nr_of_interpolation);
+        keep = &L.keep;
+    }
+    if (P->levels.empty()) {
+        P->Xraw.reset((size_t)N * d);
+        F3M_HIP(hipMemcpyAsync(P->Xraw.get(), X, sizeof(float) * (size_t)N * d, hipMemcpyDeviceToDevice, s));
+        if (!sym) {
+            P->Yraw.reset((size_t)M * d);
+            F3M_HIP(hipMemcpyAsync(P->Yraw.get(), Y, sizeof(float) * (size_t)M * d, hipMemcpyDeviceToDevice, s));
+        }
+    }
+    F3M_HIP(hipStreamSynchronize(s));
+    return P.release();
+}
+
+static void check_level(const f3m_plan *P, int level)
+{
+    F3M_REQUIRE(P != nullptr, 1, "plan is NULL");
+    F3M_REQUIRE(level >= 1 && level <= (int)P->levels.size(), 11, "level %d out of range 1..%d", level, (int)P->levels.size());
+}
+
+static void far_level(f3m_plan *P, int level, const float *bs, float *outs, float *mom, float *loc, hipStream_t s)
+{
+    PlanLevel &L = P->levels[level - 1];
+    if (L.far.n == 0) return;
+    NodeSet &ns = P->nodeset(L.num_nodes, s);
+    far_field(P->d, P->tx, P->tx.lev[level], *P->ty, P->ty->lev[level], L.far, ns, bs, outs, P->lcs, 0, mom, loc, s);
+}
+
+static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s)
+{
+    F3M_REQUIRE(P != nullptr, 1, "plan is NULL");
+    F3M_REQUIRE(c >= 1, 12, "b has no columns");
+    check_device_ptr(b, "b");
+    check_device_ptr(out, "out");
+    if (P->levels.empty()) {
+        const float *Yp = P->symmetric ? P->Xraw.get() : P->Yraw.get();
+        Scope sc(kNear, s);
+        exact_f32(P->d, P->Xraw.get(), P->N, Yp, P->M, b, c, P->prm.ls, false, out, s);
+        F3M_HIP(hipStreamSynchronize(s));
+        return;
+    }
+    DBuf<float> bs((size_t)P->M), outs((size_t)P->N);
+    const int depth = (int)P->levels.size();
+    for (int col = 0; col < c; col++) {
+        {
+            Scope sc(kPerm, s);
+            gather_column(b, P->ty->perm.get(), P->M, c, col, bs.get(), s);
+            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)P->N, s));
+        }
+        for (int k = 1; k <= depth; k++) {
+            PlanLevel &L = P->levels[k - 1];
+            // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
+            near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s);
+            far_level(P, k, bs.get(), outs.get(), nullptr, nullptr, s);
+        }
+        // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
+        near_field(P->d, P->tx, P->tx.lev[depth], *P->ty, P->ty->lev[depth], P->levels[depth - 1].keep, bs.get(),
+                   outs.get(), P->lcs, s);
+        {
+            Scope sc(kPerm, s);
+            scatter_column(outs.get(), P->tx.perm.get(), P->N, c, col, out, s);
+        }
+    }
+    F3M_HIP(hipStreamSynchronize(s));
+}
+
+template <typename F>
+static int guarded(F f)
+{
+    try {
+        f();
+        return 0;
+    } catch (const Error &e) {
+        g_error = e.what();
+        return e.code;
+    } catch (const std::exception &e) {
+        g_error = e.what();
+        return 99;
+    }
+}
+
+}  // namespace f3m
+
+// timing hooks used by f3m_field.hip
+namespace f3m {
+void timer_begin(int stage, hipStream_t s) { g_timer.begin(stage, s); }
+void timer_end(hipStream_t s) { g_timer.end(s); }
+}  // namespace f3m
+
+extern "C" {
+
+int f3m_kmvm_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c,
+                 const f3m_params *params, float *out, void *stream)
+{
+    return guarded([&] {
+        hipStream_t s = (hipStream_t)stream;
+        g_timer.reset();
+        std::unique_ptr<f3m_plan> P(plan_create(d, X, N, Y, M, params, s));
+        plan_apply(P.get(), b, c, out, s);
+        g_timer.collect();
+    });
+}
+
+int f3m_exact_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c, float ls,
+                  float *out, void *stream)
+{
+    return guarded([&] {
+        F3M_REQUIRE(d >= 1 && d <= kMaxD, 2, "dimension must be 1..10 (got %d)", d);
+        F3M_REQUIRE(N >= 0 && M >= 0 && c >= 1, 3, "bad shape");
+        F3M_REQUIRE(ls > 0.f, 5, "ls must be positive");
+        if (N == 0) return;
+        check_device_ptr(X, "X"); check_device_ptr(out, "out");
+        if (M > 0) { check_device_ptr(Y, "Y"); check_device_ptr(b, "b"); }
+        exact_f32(d, X, N, Y, M, b, c, ls, false, out, (hipStream_t)stream);
+        F3M_HIP(hipStreamSynchronize((hipStream_t)stream));
+    });
+}
+
+int f3m_exact_grad_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c, float ls,
+                       float *out, void *stream)
+{
+    return guarded([&] {
+        F3M_REQUIRE(d >= 1 && d <= kMaxD, 2, "dimension must be 1..10 (got %d)", d);
+        F3M_REQUIRE(N >= 0 && M >= 0 && c >= 1, 3, "bad shape");
+        F3M_REQUIRE(ls > 0.f, 5, "ls must be positive");
+        if (N == 0) return;
+        check_device_ptr(X, "X"); check_device_ptr(out, "out");
+        if (M > 0) { check_device_ptr(Y, "Y"); check_device_ptr(b, "b"); }
+        exact_f32(d, X, N, Y, M, b, c, ls, true, out, (hipStream_t)stream);
+        F3M_HIP(hipStreamSynchronize((hipStream_t)stream));
+    });
+}
+
+int f3m_exact_f64(int d, const double *X, int64_t N, const double *Y, int64_t M, const double *b, int c, double ls,
+                  double *out, void *stream)
+{
+    return guarded([&] {
+        F3M_REQUIRE(d >= 1 && d <= kMaxD, 2, "dimension must be 1..10 (got %d)", d);
+        F3M_REQUIRE(N >= 0 && M >= 0 && c >= 1, 3, "bad shape");
+        F3M_REQUIRE(ls > 0., 5, "ls must be positive");
+        if (N == 0) return;
+        check_device_ptr(X, "X"); check_device_ptr(out, "out");
+        if (M > 0) { check_device_ptr(Y, "Y"); check_device_ptr(b, "b"); }
+        exact_f64(d, X, N, Y, M, b, c, ls, out, (hipStream_t)stream);
+        F3M_HIP(hipStreamSynchronize((hipStream_t)stream));
+    });
+}
+
+int f3m_plan_create(int d, const float *X, int64_t N, const float *Y, int64_t M, const f3m_params *params, void *stream,
+                    f3m_plan **plan)
+{
+    return guarded([&] {
+        F3M_REQUIRE(plan != nullptr, 1, "plan is NULL");
+        *plan = nullptr;
+        g_timer.reset();
+        *plan = plan_create(d, X, N, Y, M, params, (hipStream_t)stream);
+        g_timer.collect();
+    });
+}
+
+int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stream)
+{
+    return guarded([&] {
+        g_timer.reset();
+        plan_apply(plan, b, c, out, (hipStream_t)stream);
+        g_timer.collect();
+    });
+}
+
+int f3m_plan_destroy(f3m_plan *plan)
+{
+    return guarded([&] { delete plan; });
+}
+
+int f3m_plan_depth(const f3m_plan *plan) { return plan ? (int)plan->levels.size() : -1; }
+int f3m_plan_symmetric(const f3m_plan *plan) { return plan ? (plan->symmetric ? 1 : 0) : -1; }
+
+int f3m_plan_level_sizes(const f3m_plan *plan, int level, int64_t *sizes, float *edge)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        const PlanLevel &L = plan->levels[level - 1];
+        sizes[0] = plan->tx.lev[level].nb;
+        sizes[1] = plan->ty->lev[level].nb;
+        sizes[2] = L.far.n;
+        sizes[3] = L.small_.n;
+        sizes[4] = L.keep.n;
+        sizes[5] = L.num_nodes;
+        sizes[6] = plan->tx.lev[level].maxcount;
+        sizes[7] = plan->ty->lev[level].maxcount;
+        if (edge) *edge = plan->tx.lev[level].edge;
+    });
+}
+
+int f3m_plan_level_copy(const f3m_plan *plan, int level, int which, void *dst, void *stream)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        F3M_REQUIRE(dst != nullptr, 1, "dst is NULL");
+        hipStream_t s = (hipStream_t)stream;
+        const PlanLevel &L = plan->levels[level - 1];
+        const TreeLevel &lx = plan->tx.lev[level], &ly = plan->ty->lev[level];
+        const int d = plan->d;
+        switch (which) {
+        case F3M_CENTERS_X: d2h((float *)dst, lx.ctr.get(), (size_t)lx.nb * d, s); break;
+        case F3M_CENTERS_Y: d2h((float *)dst, ly.ctr.get(), (size_t)ly.nb * d, s); break;
+        case F3M_OFFSETS_X: d2h((int *)dst, lx.off.get(), (size_t)lx.nb + 1, s); break;
+        case F3M_OFFSETS_Y: d2h((int *)dst, ly.off.get(), (size_t)ly.nb + 1, s); break;
+        case F3M_LIST_FAR: if (L.far.n) d2h((int *)dst, L.far.pairs.get(), (size_t)L.far.n * 2, s); break;
+        case F3M_LIST_SMALL: if (L.small_.n) d2h((int *)dst, L.small_.pairs.get(), (size_t)L.small_.n * 2, s); break;
+        case F3M_LIST_KEEP: if (L.keep.n) d2h((int *)dst, L.keep.pairs.get(), (size_t)L.keep.n * 2, s); break;
+        case F3M_PERM_X: d2h((int *)dst, plan->tx.perm.get(), (size_t)plan->N, s); break;
+        case F3M_PERM_Y: d2h((int *)dst, plan->ty->perm.get(), (size_t)plan->M, s); break;
+        default: throw Error(13, "unknown level array");
+        }
+    });
+}
+
+int f3m_plan_far_level(f3m_plan *plan, int level, const float *b, int c, float *out, float *mom, float *loc, void *stream)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        hipStream_t s = (hipStream_t)stream;
+        check_device_ptr(b, "b"); check_device_ptr(out, "out");
+        DBuf<float> bs((size_t)plan->M), outs((size_t)plan->N);
+        PlanLevel &L = plan->levels[level - 1];
+        int P = L.far.n ? plan->nodeset(L.num_nodes, s).P : 0;
+        for (int col = 0; col < c; col++) {
+            gather_column(b, plan->ty->perm.get(), plan->M, c, col, bs.get(), s);
+            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)plan->N, s));
+            far_level(plan, level, bs.get(), outs.get(),
+                      mom ? mom + (size_t)col * plan->ty->lev[level].nb * P : nullptr,
+                      loc ? loc + (size_t)col * plan->tx.lev[level].nb * P : nullptr, s);
+            scatter_column(outs.get(), plan->tx.perm.get(), plan->N, c, col, out, s);
+        }
+        F3M_HIP(hipStreamSynchronize(s));
+    });
+}
+
+int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, int c, float *out, void *stream)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        F3M_REQUIRE(which == F3M_LIST_SMALL || which == F3M_LIST_KEEP, 13, "which must be F3M_LIST_SMALL or F3M_LIST_KEEP");
+        hipStream_t s = (hipStream_t)stream;
+        check_device_ptr(b, "b"); check_device_ptr(out, "out");
+        DBuf<float> bs((size_t)plan->M), outs((size_t)plan->N);
+        PlanLevel &L = plan->levels[level - 1];
+        for (int col = 0; col < c; col++) {
+            gather_column(b, plan->ty->perm.get(), plan->M, c, col, bs.get(), s);
+            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)plan->N, s));
+            near_field(plan->d, plan->tx, plan->tx.lev[level], *plan->ty, plan->ty->lev[level],
+                       which == F3M_LIST_SMALL ? L.small_ : L.keep, bs.get(), outs.get(), plan->lcs, s);
+            scatter_column(outs.get(), plan->tx.perm.get(), plan->N, c, col, out, s);
+        }
+        F3M_HIP(hipStreamSynchronize(s));
+    });
+}
+
+int f3m_plan_work(const f3m_plan *plan, double *w)
+{
+    return guarded([&] {
+        F3M_REQUIRE(plan != nullptr && w != nullptr, 1, "NULL argument");
+        // computed on the host from copies of the lists and offsets
+        w[0] = w[1] = w[2] = w[3] = 0.0;
+        const int depth = (int)plan->levels.size();
+        if (depth == 0) { w[0] = (double)plan->N * (double)plan->M; return; }
+        hipStream_t s = nullptr;
+        for (int k = 1; k <= depth; k++) {
+            const PlanLevel &L = plan->levels[k - 1];
+            const TreeLevel &lx = plan->tx.lev[k], &ly = plan->ty->lev[k];
+            std::vector<int> ox((size_t)lx.nb + 1), oy((size_t)ly.nb + 1);
+            d2h(ox.data(), lx.off.get(), ox.size(), s);
+            d2h(oy.data(), ly.off.get(), oy.size(), s);
+            auto pair_sum = [&](const PairList &l) {
+                double acc = 0;
+                if (!l.n) return acc;
+                std::vector<int> h((size_t)l.n * 2);
+                d2h(h.data(), l.pairs.get(), h.size(), s);
+                for (long long t = 0; t < l.n; t++)
+                    acc += (double)(ox[h[2 * t] + 1] - ox[h[2 * t]]) * (double)(oy[h[2 * t + 1] + 1] - oy[h[2 * t + 1]]);
+                return acc;
+            };
+            w[0] += pair_sum(L.small_);
+            if (k == depth) w[0] += pair_sum(L.keep);
+            w[1] += (double)L.far.n;
+            if (L.far.n) {
+                std::vector<int> h((size_t)L.far.n * 2);
+                d2h(h.data(), L.far.pairs.get(), h.size(), s);
+                std::vector<char> ux(lx.nb, 0), uy(ly.nb, 0);
+                for (long long t = 0; t < L.far.n; t++) { ux[h[2 * t]] = 1; uy[h[2 * t + 1]] = 1; }
+                for (int bx = 0; bx < lx.nb; bx++) if (ux[bx]) w[2] += ox[bx + 1] - ox[bx];
+                for (int by = 0; by < ly.nb; by++) if (uy[by]) w[2] += oy[by + 1] - oy[by];
+                int P = 1;
+                {
+                    NodeSet tmp;
+                    // node count of the level without touching the device
+                    float ref_val = (float)pow((double)L.num_nodes, 1.0 / (double)(float)plan->d);
+                    int hi = (int)std::ceil(ref_val), lo = (int)std::floor(ref_val), acc = 1;
+                    for (int i = 0; i < plan->d; i++) {
+                        int fut = (int)((double)acc * pow((double)lo, (double)(plan->d - (i + 1))) * (double)hi);
+                        int pick = fut <= L.num_nodes ? hi : lo;
+                        if (pick < 1) pick = 1;
+                        acc *= pick;
+                    }
+                    P = acc;
+                }
+                w[3] += (double)L.far.n * (double)P * (double)P;
+            }
+        }
+    });
+}
+
+int f3m_set_timing(int enabled)
+{
+    g_timer.enabled = enabled != 0;
+    return 0;
+}
+
+int f3m_get_timing(double *t, int *n)
+{
+    for (int i = 0; i < kNumStages; i++) {
+        if (t) t[i] = g_timer.t[i];
+        if (n) n[i] = g_timer.n[i];
+    }
+    return 0;
+}
+
+const char *f3m_last_error(void) { return g_error.c_str(); }
+
+int f3m_release_cache(void)
+{
+    return guarded([&] { Pool::get().release_cached(); });
+}
+
+const char *f3m_version(void) { return "f3m-gfx950 0.1"; }
+
+}  // extern "C"

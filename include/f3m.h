@@ -1,0 +1,108 @@
+/*
+ * C ABI of the MI355X (gfx950) F3M kernel-matrix-vector-product engine.
+ *
+ * Every pointer named X, Y, b, out is DEVICE memory (fp32 row-major unless stated), borrowed for
+ * the duration of the call and never modified except `out`.  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  Every function returns 0 on success or a positive error
+ * code; f3m_last_error() then returns a message for the calling thread.  Calls are synchronous:
+ * the stream is idle when they return.  One call at a time per device (the engine keeps a cache of
+ * device buffers that concurrent calls would share).
+ *
+ * The citations name the interface of the upstream reference (repository MrHuff/F3M) that each
+ * entry point replaces.
+ */
+#ifndef F3M_H
+#define F3M_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct f3m_plan f3m_plan;
+
+/* Problem parameters = the scalar arguments of FFM_XY<float,nd>
+ * (F3M_src/n_tree.cu:1056-1059; Python defaults experiments/FFM_classes.py:9-19). */
+typedef struct f3m_params {
+    float ls;                   /* lengthscale: K = exp(-r^2 / (2 ls^2)) */
+    float min_points;           /* divide while the fullest box holds more points than this */
+    int nr_of_interpolation;    /* interpolation nodes per box (upper bound of the tensor grid) */
+    int var_compression;        /* 0/1: extra far-field shortcuts of 1_d_conv.cu:955-1029 */
+    float eff_var_limit;        /* threshold used by var_compression */
+    int small_field_points;     /* box pairs with fewer points than 2*this are summed exactly */
+} f3m_params;
+
+/* out(N,c) = K(X,Y) b.  Replaces FFM_XY_FLOAT_{1..10} (F3M_src/pybinder_setup.cu:17-36, C++ body
+ * F3M_src/n_tree.cu:1056-1125).  d = columns of X and Y (1..10).  Y == NULL or Y == X selects the
+ * symmetric case (the reference tests X.data_ptr()==Y.data_ptr(), n_tree.cu:1072); M is then ignored.
+ * b is (M,c).  If no division happens (N <= min_points) the exact product is returned, where the
+ * reference reads undefined tensors. */
+int f3m_kmvm_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c,
+                 const f3m_params *params, float *out, void *stream);
+
+/* Exact dense products.  Replace rbf_float_{1..10}, rbf_float_{1..10}_grad and rbf_double_{1..10}
+ * (F3M_src/pybinder_setup.cu:40-72, bodies F3M_src/n_tree.cu:185-241).  The _grad form returns
+ * sum_j exp(-r^2/(2 ls^2)) r^2 b_j / ls^3. */
+int f3m_exact_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c,
+                  float ls, float *out, void *stream);
+int f3m_exact_grad_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, const float *b, int c,
+                       float ls, float *out, void *stream);
+int f3m_exact_f64(int d, const double *X, int64_t N, const double *Y, int64_t M, const double *b, int c,
+                  double ls, double *out, void *stream);
+
+/* Plan = box division + interaction lists of (X, Y, params), i.e. everything FFM_XY computes that
+ * does not depend on b (F3M_src/n_tree.cu:105-179 divide, :903-969 get_field).  f3m_kmvm_f32 is
+ * create + apply + destroy; callers that multiply many vectors by the same kernel matrix (the
+ * conjugate-gradient drivers, conjugate_gradient/custom_conjugate_gradient_falkon.py:144-160) keep
+ * the plan.  The plan holds its own sorted copy of the points: X and Y may be freed after create. */
+int f3m_plan_create(int d, const float *X, int64_t N, const float *Y, int64_t M, const f3m_params *params,
+                    void *stream, f3m_plan **plan);
+int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stream);
+int f3m_plan_destroy(f3m_plan *plan);
+
+/* Introspection for parity tests (no counterpart is exported by the reference; the data are its
+ * n_tree_cuda members, F3M_src/n_tree.cu:51-78, and the three lists of separate_interactions,
+ * :701-787).  Levels are numbered 1..depth. */
+int f3m_plan_depth(const f3m_plan *plan);                 /* number of divisions performed */
+int f3m_plan_symmetric(const f3m_plan *plan);
+/* sizes[0..7] = boxes of X tree, boxes of Y tree, |far|, |small|, |keep|, nodes used, max count X, max count Y */
+int f3m_plan_level_sizes(const f3m_plan *plan, int level, int64_t *sizes, float *edge);
+enum f3m_level_array {
+    F3M_CENTERS_X = 0,   /* float (nbx,d) */
+    F3M_CENTERS_Y = 1,
+    F3M_OFFSETS_X = 2,   /* int32 nbx+1: point ranges of the boxes in sorted order */
+    F3M_OFFSETS_Y = 3,
+    F3M_LIST_FAR = 4,    /* int32 (n,2) */
+    F3M_LIST_SMALL = 5,
+    F3M_LIST_KEEP = 6,
+    F3M_PERM_X = 7,      /* int32 N: sorted position -> row of X (same at every level) */
+    F3M_PERM_Y = 8
+};
+/* copies one array of a level to HOST memory `dst` (caller sizes it from f3m_plan_level_sizes) */
+int f3m_plan_level_copy(const f3m_plan *plan, int level, int which, void *dst, void *stream);
+/* far field of one level only: out(N,c) receives its contribution; mom (nby*P*c) and loc (nbx*P*c),
+ * device pointers or NULL, receive the moments and local expansions, column-major over c */
+int f3m_plan_far_level(f3m_plan *plan, int level, const float *b, int c, float *out, float *mom, float *loc,
+                       void *stream);
+/* near field of one list of one level: which = F3M_LIST_SMALL or F3M_LIST_KEEP */
+int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, int c, float *out, void *stream);
+/* work model of the plan: w[0] = point pairs summed exactly, w[1] = far box pairs, w[2] = points
+ * interpolated (P2M + L2P passes), w[3] = sum over levels of far pairs * P^2 */
+int f3m_plan_work(const f3m_plan *plan, double *w);
+
+/* seconds spent by the last f3m_plan_apply / f3m_kmvm_f32 of this thread in each stage, measured
+ * with HIP events on the call's stream when timing is enabled: t[0] plan, t[1] near, t[2] P2M,
+ * t[3] M2L, t[4] L2P, t[5] permutations; n[] = kernel launches per stage */
+int f3m_set_timing(int enabled);
+int f3m_get_timing(double *t, int *n);
+
+const char *f3m_last_error(void);
+/* frees the cached device buffers */
+int f3m_release_cache(void);
+const char *f3m_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,222 @@
+// TEST INFRASTRUCTURE ONLY: a minimal single-OS-thread emulation of the HIP execution model, so
+// that the engine's kernel sources can be compiled with g++ and run on a CPU for logic tests and
+// for debugging with gdb / sanitizers.  The product never links this; the Python package loads only
+// the gfx950 library and fails if it is missing.
+//
+// Model: blocks run one after another; the threads of a block are fibers (ucontext) scheduled
+// round-robin; __syncthreads and wave-level operations are generation barriers that yield.
+// Wave size is 64.  Only 1-D grids and blocks.
+#pragma once
+#include <ucontext.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <functional>
+#include <vector>
+
+#define __global__
+#define __device__
+#define __host__
+#define __forceinline__ inline
+#define __shared__ static
+#define __launch_bounds__(...)
+
+struct dim3 {
+    unsigned x, y, z;
+    dim3(unsigned x_ = 1, unsigned y_ = 1, unsigned z_ = 1) : x(x_), y(y_), z(z_) {}
+};
+
+typedef int hipError_t;
+typedef void *hipStream_t;
+enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2 };
+enum hipMemcpyKind { hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
+
+inline hipError_t hipMalloc(void **p, size_t n) { *p = malloc(n ? n : 1); return *p ? hipSuccess : hipErrorOutOfMemory; }
+inline hipError_t hipFree(void *p) { free(p); return hipSuccess; }
+inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { memcpy(d, s, n); return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void *d, const void *s, size_t n, hipMemcpyKind, hipStream_t) { memcpy(d, s, n); return hipSuccess; }
+inline hipError_t hipMemsetAsync(void *d, int v, size_t n, hipStream_t) { memset(d, v, n); return hipSuccess; }
+inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
+inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
+inline hipError_t hipGetLastError() { return hipSuccess; }
+inline const char *hipGetErrorString(hipError_t) { return "emu"; }
+inline hipError_t hipGetDevice(int *d) { *d = 0; return hipSuccess; }
+
+namespace emu {
+
+constexpr int WAVE = 64;
+constexpr size_t STACK = 256 * 1024;
+
+struct Wave {
+    uint64_t bits[2];
+    uint32_t vals[2][WAVE];
+    int arrived, gen, alive;
+};
+
+struct Fiber {
+    ucontext_t ctx;
+    unsigned tid;
+    bool done;
+};
+
+struct State {
+    ucontext_t main_ctx;
+    std::vector<Fiber> fibers;
+    std::vector<char *> stacks;
+    std::vector<Wave> waves;
+    Fiber *cur = nullptr;
+    unsigned block = 0, bdim = 1, gdim = 1;
+    int bar_arrived = 0, bar_gen = 0, alive = 0;
+    std::function<void()> body;
+    std::vector<char> dynshared;
+};
+
+inline State &S() { static State s; return s; }
+
+inline void yield() { State &s = S(); swapcontext(&s.cur->ctx, &s.main_ctx); }
+
+inline void trampoline()
+{
+    State &s = S();
+    s.body();
+    Fiber *f = s.cur;
+    f->done = true;
+    // leaving threads stop counting towards barriers
+    s.alive--;
+    if (s.alive > 0 && s.bar_arrived == s.alive) { s.bar_arrived = 0; s.bar_gen++; }
+    Wave &w = s.waves[f->tid / WAVE];
+    w.alive--;
+    if (w.alive > 0 && w.arrived == w.alive) { w.arrived = 0; w.bits[(w.gen & 1) ^ 1] = 0; w.gen++; }
+    swapcontext(&f->ctx, &s.main_ctx);
+}
+
+inline void launch(unsigned grid, unsigned block, size_t shmem, std::function<void()> body)
+{
+    State &s = S();
+    if (block == 0 || grid == 0) return;
+    if (s.fibers.size() < block) {
+        size_t old = s.fibers.size();
+        s.fibers.resize(block);
+        s.stacks.resize(block, nullptr);
+        for (size_t i = old; i < block; i++) s.stacks[i] = (char *)malloc(STACK);
+    }
+    s.dynshared.assign(shmem + 16, 0);
+    s.body = body;
+    s.bdim = block; s.gdim = grid;
+    unsigned nw = (block + WAVE - 1) / WAVE;
+    s.waves.resize(nw);
+    for (unsigned b = 0; b < grid; b++) {
+        s.block = b;
+        s.bar_arrived = 0; s.bar_gen = 0; s.alive = (int)block;
+        for (unsigned w = 0; w < nw; w++) {
+            Wave &W = s.waves[w];
+            memset(&W, 0, sizeof(W));
+            W.alive = (int)std::min<unsigned>(WAVE, block - w * WAVE);
+        }
+        for (unsigned t = 0; t < block; t++) {
+            Fiber &f = s.fibers[t];
+            f.tid = t; f.done = false;
+            getcontext(&f.ctx);
+            f.ctx.uc_stack.ss_sp = s.stacks[t];
+            f.ctx.uc_stack.ss_size = STACK;
+            f.ctx.uc_link = &s.main_ctx;
+            makecontext(&f.ctx, (void (*)())trampoline, 0);
+        }
+        int remaining = (int)block;
+        long sweeps = 0;
+        while (remaining > 0) {
+            remaining = 0;
+            for (unsigned t = 0; t < block; t++) {
+                Fiber &f = s.fibers[t];
+                if (f.done) continue;
+                s.cur = &f;
+                swapcontext(&s.main_ctx, &f.ctx);
+                if (!f.done) remaining++;
+            }
+            if (++sweeps > 100000000L) { fprintf(stderr, "emu: kernel does not terminate (deadlocked barrier?)\n"); abort(); }
+        }
+    }
+    s.cur = nullptr;
+}
+
+inline void syncthreads()
+{
+    State &s = S();
+    int my = s.bar_gen;
+    if (++s.bar_arrived == s.alive) { s.bar_arrived = 0; s.bar_gen++; }
+    else while (s.bar_gen == my) yield();
+}
+
+inline Wave &wave() { State &s = S(); return s.waves[s.cur->tid / WAVE]; }
+
+inline void wave_barrier(Wave &w)
+{
+    int my = w.gen;
+    if (++w.arrived == w.alive) { w.arrived = 0; w.bits[(w.gen & 1) ^ 1] = 0; w.gen++; }
+    else while (w.gen == my) yield();
+}
+
+inline uint64_t ballot(bool pred)
+{
+    Wave &w = wave();
+    int slot = w.gen & 1;
+    unsigned lane = S().cur->tid % WAVE;
+    if (pred) w.bits[slot] |= 1ull << lane;
+    wave_barrier(w);
+    return w.bits[slot];
+}
+
+inline uint32_t shfl_bits(uint32_t v, int src)
+{
+    Wave &w = wave();
+    int slot = w.gen & 1;
+    unsigned lane = S().cur->tid % WAVE;
+    w.vals[slot][lane] = v;
+    wave_barrier(w);
+    return w.vals[slot][src & (WAVE - 1)];
+}
+
+struct Idx { unsigned x; };
+struct TidProxy { struct X { operator unsigned() const { return S().cur->tid; } } x; };
+struct BidProxy { struct X { operator unsigned() const { return S().block; } } x; };
+struct BdimProxy { struct X { operator unsigned() const { return S().bdim; } } x; };
+struct GdimProxy { struct X { operator unsigned() const { return S().gdim; } } x; };
+
+}  // namespace emu
+
+static emu::TidProxy threadIdx;
+static emu::BidProxy blockIdx;
+static emu::BdimProxy blockDim;
+static emu::GdimProxy gridDim;
+
+inline void __syncthreads() { emu::syncthreads(); }
+
+template <typename T> inline T atomicAdd(T *p, T v) { T o = *p; *p = o + v; return o; }
+template <typename T> inline T atomicMax(T *p, T v) { T o = *p; if (v > o) *p = v; return o; }
+template <typename T> inline T atomicMin(T *p, T v) { T o = *p; if (v < o) *p = v; return o; }
+template <typename T> inline T atomicCAS(T *p, T cmp, T v) { T o = *p; if (o == cmp) *p = v; return o; }
+template <typename T> inline T atomicOr(T *p, T v) { T o = *p; *p = o | v; return o; }
+
+inline int __popcll(unsigned long long v) { return __builtin_popcountll(v); }
+inline int __popc(unsigned v) { return __builtin_popcount(v); }
+inline int __ffsll(unsigned long long v) { return __builtin_ffsll((long long)v); }
+inline int __clz(unsigned v) { return v ? __builtin_clz(v) : 32; }
+
+namespace emu {
+template <typename K, typename... A>
+inline void launch_k(unsigned grid, unsigned block, size_t shmem, K kernel, A... args)
+{
+    launch(grid, block, shmem, [=]() { kernel(args...); });
+}
+}  // namespace emu
+#define F3M_EMU_LAUNCH(kernel, grid, block, shmem, stream, ...) \
+    emu::launch_k((unsigned)(grid), (unsigned)(block), (size_t)(shmem), kernel, __VA_ARGS__)
+
+struct float4 { float x, y, z, w; };
+inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }
+using std::max;
+using std::min;

@@ -1,0 +1,114 @@
+"""Runs the engine's real kernel sources, compiled for the CPU by tests/cpu_emu, against the oracle
+on small inputs: box division and lists bit-exact, every numeric stage within tolerance.  These are
+logic tests of the HIP code (indexing, barriers, ballots); numerics on the device are covered by
+the -m gpu tests."""
+import numpy as np
+import pytest
+
+import emu_engine as ee
+from parity_checks import assert_plan_matches_oracle, rel_l2
+
+f32 = np.float32
+
+
+def _cloud(name, rng):
+    if name == "uniform3":
+        return rng.random((3000, 3), dtype=f32), None
+    if name == "normal2":
+        return rng.standard_normal((2500, 2)).astype(f32), None
+    if name == "uniform1":
+        return rng.random((1200, 1), dtype=f32), None
+    if name == "uniform4":
+        return rng.random((3000, 4), dtype=f32), None
+    if name == "asym3":
+        X = rng.standard_normal((2500, 3)).astype(f32)
+        Y = (rng.random((1800, 3)) * 5 - 2.5).astype(f32)
+        return X, Y
+    if name == "dups_faces":
+        g = (np.stack(np.meshgrid(*[np.arange(9)] * 3, indexing="ij"), -1).reshape(-1, 3) / 8.0).astype(f32)
+        return np.concatenate([g, g[::-1], g[::3]]), None
+    raise KeyError(name)
+
+
+PRM = dict(ls=0.6, min_points=60, nr_of_interpolation=27, small_field_points=40)
+
+
+@pytest.mark.parametrize("name", ["uniform3", "normal2", "uniform1", "uniform4", "asym3", "dups_faces"])
+def test_tree_and_lists_bit_exact(oracle, name):
+    X, Y = _cloud(name, np.random.default_rng(21))
+    eng = ee.Plan(X, Y, **PRM)
+    ora = oracle.Plan(X, Y, **PRM)
+    assert_plan_matches_oracle(eng, ora)
+    w = eng.work()
+    assert w[0] == ora.work_near_pairs and w[1] == ora.work_far_pairs and w[2] == ora.work_interp_pts
+
+
+def test_var_compression_lists_bit_exact(oracle):
+    X, _ = _cloud("uniform3", np.random.default_rng(3))
+    prm = dict(PRM, var_compression=True, eff_var_limit=0.3, ls=2.0)
+    assert_plan_matches_oracle(ee.Plan(X, None, **prm), oracle.Plan(X, None, **prm))
+
+
+def test_exact_kernels(oracle):
+    rng = np.random.default_rng(0)
+    for d in (1, 3, 5):
+        X = rng.standard_normal((300, d)).astype(f32)
+        Y = rng.standard_normal((700, d)).astype(f32)
+        b = rng.standard_normal((700, 2)).astype(f32)
+        ref = oracle.exact_f64(X, Y, b, 0.8)
+        assert rel_l2(ee.exact("f3m_exact_f32", X, Y, b, 0.8), ref) < 1e-5
+        assert rel_l2(ee.exact("f3m_exact_f64", X, Y, b, 0.8, np.float64), ref) < 1e-12
+        assert rel_l2(ee.exact("f3m_exact_grad_f32", X, Y, b, 0.8), oracle.exact_grad_f32(X, Y, b, 0.8)) < 1e-5
+
+
+@pytest.mark.parametrize("name,P", [("uniform3", 27), ("normal2", 16), ("asym3", 64), ("uniform4", 16)])
+def test_stages_and_product(oracle, name, P):
+    rng = np.random.default_rng(8)
+    X, Y = _cloud(name, rng)
+    M = X.shape[0] if Y is None else Y.shape[0]
+    b = rng.standard_normal((M, 2)).astype(f32)
+    prm = dict(PRM, nr_of_interpolation=P)
+    eng = ee.Plan(X, Y, **prm)
+    ora = oracle.Plan(X, Y, **prm)
+    nodes = int(np.prod(oracle.node_counts(X.shape[1], P)))
+    did_far = False
+    for k in range(1, eng.depth + 1):
+        sz = eng.level_sizes(k)
+        if sz["nsmall"]:
+            assert rel_l2(eng.near_level(k, "small", b), ora.near_level(k - 1, "small", b)) < 1e-5
+        if sz["nfar"]:
+            did_far = True
+            out, mom, loc = eng.far_level(k, b, nodes)
+            o_out, o_mom, o_loc = ora.far_level(k - 1, b)
+            assert rel_l2(mom, np.moveaxis(o_mom, 2, 0)) < 1e-4
+            assert rel_l2(loc, np.moveaxis(o_loc, 2, 0)) < 1e-4
+            assert rel_l2(out, o_out) < 1e-4
+    assert did_far
+    if eng.level_sizes(eng.depth)["nkeep"]:
+        assert rel_l2(eng.near_level(eng.depth, "keep", b), ora.near_level(eng.depth - 1, "keep", b)) < 1e-5
+    got = eng.apply(b)
+    assert rel_l2(got, ora.apply(b)) < 1e-5
+    exact = oracle.exact_f64(X, X if Y is None else Y, b, prm["ls"])
+    assert rel_l2(got, exact) <= 1.5 * rel_l2(ora.apply(b), exact) + 1e-6
+    assert rel_l2(ee.kmvm(X, Y, b, **prm), got) == 0.0
+
+
+def test_no_division_returns_exact_product(oracle):
+    rng = np.random.default_rng(2)
+    X = rng.random((200, 3), dtype=f32)
+    b = rng.standard_normal((200, 1)).astype(f32)
+    out = ee.kmvm(X, None, b, ls=0.5, min_points=1000)
+    assert rel_l2(out, oracle.exact_f64(X, X, b, 0.5)) < 1e-5
+
+
+def test_error_paths():
+    rng = np.random.default_rng(2)
+    X = rng.random((50, 3), dtype=f32)
+    b = rng.standard_normal((50, 1)).astype(f32)
+    from f3m_amd.capi import F3MError
+    with pytest.raises(F3MError):
+        ee.kmvm(X, None, b, ls=-1.0)
+    with pytest.raises(F3MError):
+        ee.kmvm(np.zeros((50, 11), f32), None, b)
+    with pytest.raises(F3MError):
+        ee.kmvm(np.ones((50, 3), f32), None, b, min_points=10)      # all points identical: zero edge
