@@ -1,0 +1,127 @@
+#!/usr/bin/env python3
+"""Benchmark of the F3M kernel-matrix-vector product on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--dist uniform|normal] [--ls LS]
+
+A step is one complete product out = K(X,X) b through the C ABI (box division + interaction lists +
+near field + far field), inputs resident in HBM, like one `FFM(X) @ b` of the reference
+(experiments/experiments.py:72-77).  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3      # MI355X vector fp32 peak (packed); the near field is VALU work
+
+
+def cpu_baseline(X, b, ls, budget_s=15.0):
+    """Exact tiled PyTorch product on the host cores for a bounded number of target rows against all
+    sources (the checker's code, timed only here)."""
+    import torch
+    from oracle import f3m_oracle as fo
+    Xc, bc = X.cpu(), b.cpu()
+    rows = 64
+    t0 = time.perf_counter()
+    fo.exact_tiled_torch(Xc[:rows], Xc, bc, ls, row_tile=rows, col_tile=1 << 18)
+    t1 = time.perf_counter() - t0
+    rows2 = int(max(64, min(20000, rows * budget_s / max(t1, 1e-3)))) // 64 * 64
+    t0 = time.perf_counter()
+    fo.exact_tiled_torch(Xc[:rows2], Xc, bc, ls, row_tile=min(rows2, 256), col_tile=1 << 18)
+    t2 = time.perf_counter() - t0
+    return {"value": rows2 / t2, "unit": "points/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": "%d target rows x all %d sources, exact tiled torch fp32, %.1f s; implied full product %.0f s"
+                      % (rows2, Xc.shape[0], t2, Xc.shape[0] / (rows2 / t2)),
+            "host_cpu_count": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--n", type=int, default=10_000_000)
+    ap.add_argument("--d", type=int, default=3)
+    ap.add_argument("--dist", default="uniform", choices=["uniform", "normal"])
+    ap.add_argument("--ls", type=float, default=1.0)
+    ap.add_argument("--nodes", type=int, default=64)
+    ap.add_argument("--subsample", type=int, default=100_000)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-accuracy", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported. "
+              "Run with --gpus 1." % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from f3m_amd import engine
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    g = torch.Generator().manual_seed(1)
+    N, d = args.n, args.d
+    X = (torch.rand(N, d, generator=g) if args.dist == "uniform" else torch.randn(N, d, generator=g)).cuda()
+    b = torch.randn(N, 1, generator=g).cuda()
+    prm = dict(ls=args.ls, min_points=1000, nr_of_interpolation=args.nodes, small_field_points=1000)
+
+    engine.set_timing(True)
+    for _ in range(args.warmup):
+        out = engine.kmvm(X, None, b, **prm)
+    torch.cuda.synchronize()
+    near_t, near_n, stage = 0.0, 0, {}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = engine.kmvm(X, None, b, **prm)
+        tm = engine.get_timing()
+        near_t += tm["near"][0]
+        near_n += tm["near"][1]
+        for k, v in tm.items():
+            stage[k] = stage.get(k, 0.0) + v[0]
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms = dt / args.steps * 1e3
+
+    plan = engine.Plan(X, None, **prm)
+    work = plan.work()
+    depth = plan.depth
+    plan.close()
+    F = 3 * d + 3                                  # flops per kernel evaluation (d sub, d mul, d-1 add, scale, exp, fma)
+    near_flops = F * work["near_pairs"]
+    near_per_launch_s = near_t / max(near_n, 1)
+    achieved = near_flops * args.steps / max(near_t, 1e-12) / 1e12
+    roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None, "kernel": "near_kernel<%d,1>" % d,
+                "note": "fp32 vector ALU kernel priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
+                        "%.3e kernel evaluations/step x %d flops" % (near_n // max(args.steps, 1), near_per_launch_s * 1e3,
+                                                                     work["near_pairs"], F)}
+    res = {
+        "metric": "KMVM points/sec at N=1e7 3D Gaussian (1 GPU); rel-L2 error vs fp64 exact",
+        "value": N / (dt / args.steps), "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "3D Gaussian KMVM X=Y, N=%d %s, b~N(0,1) (N,1), ls=%g, %d nodes/box, cutoff 1000 "
+                               "(BASELINE.json configs[1])" % (N, "uniform [0,1]^%d" % d if args.dist == "uniform" else "N(0,I)", args.ls, args.nodes),
+                   "N": N, "d": d, "ls": args.ls, "nodes": args.nodes, "tree_depth": depth},
+        "roofline": roofline,
+        "stage_ms_per_step": {k: v / args.steps * 1e3 for k, v in stage.items()},
+        "work": work,
+    }
+    if not args.no_accuracy:
+        rows = torch.from_numpy(np.random.default_rng(1).choice(N, min(args.subsample, N), replace=False)).cuda()
+        exact = engine.exact_f64(X[rows].double(), X.double(), b.double(), args.ls)
+        diff = (out[rows].double() - exact)
+        res["rel_l2_error"] = float(diff.norm() / exact.norm())
+        res["rel_l2_rows"] = int(rows.numel())
+    if not args.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(X, b, args.ls)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

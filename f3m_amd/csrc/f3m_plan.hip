@@ -470,7 +470,7 @@ int f3m_plan_work(const f3m_plan *plan, double *w)
     return guarded([&] {
         F3M_REQUIRE(plan != nullptr && w != nullptr, 1, "NULL argument");
         // computed on the host from copies of the lists and offsets
-        w[0] = w[1] = w[2] = w[3] = 0.0;
+        w[0] = w[1] = w[2] = w[3] = w[4] = 0.0;
         const int depth = (int)plan->levels.size();
         if (depth == 0) { w[0] = (double)plan->N * (double)plan->M; return; }
         hipStream_t s = nullptr;
@@ -492,6 +492,7 @@ int f3m_plan_work(const f3m_plan *plan, double *w)
             w[0] += pair_sum(L.small_);
             if (k == depth) w[0] += pair_sum(L.keep);
             w[1] += (double)L.far.n;
+            w[4] += pair_sum(L.far);
             if (L.far.n) {
                 std::vector<int> h((size_t)L.far.n * 2);
                 d2h(h.data(), L.far.pairs.get(), h.size(), s);

@@ -192,10 +192,11 @@ class Plan:
 
     def work(self):
         """Work model: point pairs summed exactly, far box pairs, interpolated points, far pairs * P^2."""
-        w = (C.c_double * 4)()
+        w = (C.c_double * 5)()
         with torch.cuda.device(self.device):
             capi.check(self._lib, self._lib.f3m_plan_work(self._h, w))
-        return {"near_pairs": w[0], "far_pairs": w[1], "interp_points": w[2], "m2l_evals": w[3]}
+        return {"near_pairs": w[0], "far_pairs": w[1], "interp_points": w[2], "m2l_evals": w[3],
+                "far_point_pairs": w[4]}
 
 
 def node_counts(d, max_nodes):

@@ -88,7 +88,8 @@ int f3m_plan_far_level(f3m_plan *plan, int level, const float *b, int c, float *
 /* near field of one list of one level: which = F3M_LIST_SMALL or F3M_LIST_KEEP */
 int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, int c, float *out, void *stream);
 /* work model of the plan: w[0] = point pairs summed exactly, w[1] = far box pairs, w[2] = points
- * interpolated (P2M + L2P passes), w[3] = sum over levels of far pairs * P^2 */
+ * interpolated (P2M + L2P passes), w[3] = sum over levels of far pairs * P^2, w[4] = point pairs
+ * covered by far box pairs (w[0] + w[4] = N*M: every point pair is handled exactly once) */
 int f3m_plan_work(const f3m_plan *plan, double *w);
 
 /* seconds spent by the last f3m_plan_apply / f3m_kmvm_f32 of this thread in each stage, measured

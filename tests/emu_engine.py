@@ -115,6 +115,6 @@ class Plan:
         return out
 
     def work(self):
-        w = (C.c_double * 4)()
+        w = (C.c_double * 5)()
         capi.check(lib(), lib().f3m_plan_work(self._h, w))
         return list(w)

@@ -1,0 +1,205 @@
+"""GPU parity tests: the gfx950 library, called through its C ABI, against the CPU oracle on the
+same seeded inputs.  Box division and interaction lists are compared bit for bit; floating-point
+stages with the tolerance written at each assert (north star: rel-L2 <= 1e-3 against an fp64 exact
+product and no worse than 1.5x the oracle algorithm's own error)."""
+import numpy as np
+import pytest
+
+from parity_checks import assert_plan_matches_oracle, rel_l2
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def eng():
+    import torch
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    from f3m_amd import engine
+    engine._lib.get()          # fails loudly if the gfx950 library is not built
+    return engine
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def clouds(name, rng):
+    if name == "C1_uniform3":        # config 1: N=1e5 uniform, ls=1, 64 nodes, cutoff 1000
+        return rng.random((100000, 3), dtype=f32), None, dict(ls=1.0)
+    if name == "normal3":
+        return rng.standard_normal((60000, 3)).astype(f32), None, dict(ls=0.5)
+    if name == "clustered_xy":       # config 3 in miniature
+        mu, sd = rng.random((50, 3)) * 10, 0.05 + 0.45 * rng.random((50, 3))
+        X = np.concatenate([rng.normal(m, s, (1500, 3)) for m, s in zip(mu, sd)]).astype(f32)
+        Y = (X.min(0) + (X.max(0) - X.min(0)) * rng.random((30000, 3))).astype(f32)
+        return X, Y, dict(ls=0.5)
+    if name == "uniform4":
+        return rng.random((60000, 4), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=81)
+    if name == "uniform5":
+        return rng.random((60000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=32, min_points=100,
+                                                              small_field_points=40)
+    if name == "uniform2":
+        return rng.random((80000, 2), dtype=f32), None, dict(ls=0.2)
+    if name == "uniform1":
+        return rng.random((50000, 1), dtype=f32), None, dict(ls=0.05, nr_of_interpolation=8)
+    if name == "lattice_faces_dups":
+        g = (np.stack(np.meshgrid(*[np.arange(33)] * 3, indexing="ij"), -1).reshape(-1, 3) / 32.0).astype(f32)
+        return np.concatenate([g, g[::-1], g[::2]]), None, dict(ls=0.3, min_points=200, small_field_points=100)
+    raise KeyError(name)
+
+
+NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "uniform2", "uniform1", "lattice_faces_dups"]
+
+
+@pytest.mark.parametrize("name", NAMES)
+def test_box_division_and_lists_bit_exact(eng, oracle, name):
+    print("case", name, flush=True)
+    X, Y, prm = clouds(name, np.random.default_rng(100))
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    ora = oracle.Plan(X, Y, **prm)
+    assert ora.nlevels >= 1
+    assert_plan_matches_oracle(plan, ora)
+    w = plan.work()
+    assert w["near_pairs"] == ora.work_near_pairs and w["far_pairs"] == ora.work_far_pairs
+    assert w["interp_points"] == ora.work_interp_pts
+    M = X.shape[0] if Y is None else Y.shape[0]
+    assert w["near_pairs"] + w["far_point_pairs"] == float(X.shape[0]) * M      # every pair exactly once
+
+
+@pytest.mark.parametrize("d", [1, 2, 3, 5, 10])
+def test_exact_kernels(eng, oracle, d):
+    print("case exact d=%d" % d, flush=True)
+    rng = np.random.default_rng(d)
+    X = rng.standard_normal((1500, d)).astype(f32)
+    Y = rng.standard_normal((2300, d)).astype(f32)
+    b = rng.standard_normal((2300, 3)).astype(f32)
+    ls = 0.9 * np.sqrt(d)
+    ref = oracle.exact_f64(X, Y, b, ls)
+    assert rel_l2(eng.exact_f32(dev(X), dev(Y), dev(b), ls).cpu().numpy(), ref) < 1e-5
+    assert rel_l2(eng.exact_f64(dev(X.astype(np.float64)), dev(Y.astype(np.float64)), dev(b.astype(np.float64)), ls).cpu().numpy(), ref) < 1e-12
+    assert rel_l2(eng.exact_grad_f32(dev(X), dev(Y), dev(b), ls).cpu().numpy(), oracle.exact_grad_f32(X, Y, b, ls)) < 1e-5
+
+
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5"])
+def test_stages_against_oracle(eng, oracle, name):
+    print("case stages", name, flush=True)
+    rng = np.random.default_rng(7)
+    X, Y, prm = clouds(name, rng)
+    X = X[:30000]
+    Y = None if Y is None else Y[:12000]
+    M = X.shape[0] if Y is None else Y.shape[0]
+    b = rng.standard_normal((M, 2)).astype(f32)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    ora = oracle.Plan(X, Y, **prm)
+    assert_plan_matches_oracle(plan, ora)
+    did_far = False
+    for k in range(1, plan.depth + 1):
+        sz = plan.level_sizes(k)
+        if sz["nsmall"]:
+            got = plan.near_level(k, "small", dev(b)).cpu().numpy()
+            assert rel_l2(got, ora.near_level(k - 1, "small", b)) < 1e-5          # fp32 summation order only
+        if sz["nfar"]:
+            did_far = True
+            out, mom, loc = plan.far_level(k, dev(b), want_expansions=True)
+            o_out, o_mom, o_loc = ora.far_level(k - 1, b)
+            assert rel_l2(mom.cpu().numpy(), np.moveaxis(o_mom, 2, 0)) < 1e-4     # P2M
+            assert rel_l2(loc.cpu().numpy(), np.moveaxis(o_loc, 2, 0)) < 1e-4     # M2L
+            assert rel_l2(out.cpu().numpy(), o_out) < 1e-4                        # L2P
+    assert did_far or name == "uniform5"
+    if plan.level_sizes(plan.depth)["nkeep"]:
+        got = plan.near_level(plan.depth, "keep", dev(b)).cpu().numpy()
+        assert rel_l2(got, ora.near_level(plan.depth - 1, "keep", b)) < 1e-5
+    got = plan.apply(dev(b)).cpu().numpy()
+    assert rel_l2(got, ora.apply(b)) < 1e-5
+
+
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform4"])
+def test_product_error_vs_fp64_exact(eng, oracle, name):
+    print("case product", name, flush=True)
+    rng = np.random.default_rng(9)
+    X, Y, prm = clouds(name, rng)
+    M = X.shape[0] if Y is None else Y.shape[0]
+    b = rng.standard_normal((M, 1)).astype(f32)
+    Xd, Yd, bd = dev(X), (None if Y is None else dev(Y)), dev(b)
+    got = eng.kmvm(Xd, Yd, bd, **prm).cpu().numpy()
+    Ys = X if Y is None else Y
+    exact = eng.exact_f64(dev(X.astype(np.float64)), dev(Ys.astype(np.float64)), dev(b.astype(np.float64)), prm["ls"]).cpu().numpy()
+    err = rel_l2(got, exact)
+    err_oracle = rel_l2(oracle.kmvm(X, Y, b, **prm), exact)
+    print("rel-L2 engine %.3e oracle %.3e" % (err, err_oracle), flush=True)
+    assert err <= 1e-3                                   # north-star tolerance
+    assert err <= 1.5 * err_oracle + 1e-7                # no worse than 1.5x the reference algorithm
+
+
+def test_columns_linearity_and_plan_reuse(eng, oracle):
+    rng = np.random.default_rng(11)
+    X = rng.random((40000, 3), dtype=f32)
+    b = rng.standard_normal((40000, 3)).astype(f32)
+    plan = eng.Plan(dev(X), None, ls=0.4)
+    o = plan.apply(dev(b)).cpu().numpy()
+    for col in range(3):
+        assert np.array_equal(plan.apply(dev(b[:, col:col + 1])).cpu().numpy(), o[:, col:col + 1])
+    comb = plan.apply(dev((2 * b[:, :1] - b[:, 1:2]).astype(f32))).cpu().numpy()
+    assert rel_l2(comb, 2.0 * o[:, :1] - o[:, 1:2]) < 1e-5
+    one_shot = eng.kmvm(dev(X), None, dev(b), ls=0.4).cpu().numpy()
+    assert np.array_equal(one_shot, o)                   # deterministic: no float atomics anywhere
+
+
+def test_edge_cases(eng, oracle):
+    import torch
+    from f3m_amd.capi import F3MError
+    rng = np.random.default_rng(12)
+    X = rng.random((600, 3), dtype=f32)
+    b = rng.standard_normal((600, 2)).astype(f32)
+    # N <= min_points: no division, exact product
+    out = eng.kmvm(dev(X), None, dev(b), ls=0.5).cpu().numpy()
+    assert rel_l2(out, oracle.exact_f64(X, X, b, 0.5)) < 1e-5
+    # nothing far: reduces to the dense product
+    X2 = rng.random((3000, 3), dtype=f32)
+    b2 = rng.standard_normal((3000, 1)).astype(f32)
+    out = eng.kmvm(dev(X2), None, dev(b2), ls=0.5, small_field_points=10000).cpu().numpy()
+    assert rel_l2(out, oracle.exact_f64(X2, X2, b2, 0.5)) < 1e-5
+    # tiny and ragged
+    Xt = rng.random((1, 3), dtype=f32)
+    assert np.allclose(eng.kmvm(dev(Xt), None, dev(np.ones((1, 1), f32)), ls=1.0).cpu().numpy(), 1.0)
+    Y3 = rng.random((2001, 3), dtype=f32)
+    out = eng.kmvm(dev(X2[:1777]), dev(Y3), dev(rng.standard_normal((2001, 1)).astype(f32)), ls=0.3, min_points=100,
+                   small_field_points=50, nr_of_interpolation=27)
+    assert out.shape == (1777, 1) and torch.isfinite(out).all()
+    with pytest.raises(F3MError):
+        eng.kmvm(dev(X), None, dev(b), ls=0.0)
+    with pytest.raises(F3MError):
+        eng.kmvm(dev(np.ones((2000, 3), f32)), None, dev(np.ones((2000, 1), f32)))     # zero-size cloud
+    with pytest.raises(RuntimeError):
+        eng.kmvm(torch.from_numpy(X), None, torch.from_numpy(b))                      # host tensors
+    with pytest.raises(AssertionError):
+        eng.kmvm(dev(X), None, dev(b[:100]))
+
+
+def test_reference_operator_classes(eng, oracle):
+    import torch
+    from f3m_amd import ffm_3d_float
+    from f3m_amd.FFM_classes import FFM, benchmark_matmul, benchmark_matmul_double, block_FFM_matmul
+    assert len(ffm_3d_float.__all__) == 40
+    rng = np.random.default_rng(13)
+    X = rng.random((30000, 3), dtype=f32)
+    Y = rng.random((9000, 3), dtype=f32)
+    b = rng.standard_normal((30000, 1)).astype(f32)
+    by = rng.standard_normal((9000, 1)).astype(f32)
+    Xt, Yt, bt, byt = (torch.from_numpy(v) for v in (X, Y, b, by))
+    ref = (benchmark_matmul_double(Xt, ls=0.5) @ bt).cpu().numpy()
+    assert rel_l2(ref[:500], oracle.exact_f64(X[:500], X, b, 0.5)) < 1e-12
+    assert rel_l2((FFM(Xt, ls=0.5) @ bt).cpu().numpy(), ref) < 1e-3
+    assert rel_l2((benchmark_matmul(Xt, ls=0.5) @ bt).cpu().numpy(), ref) < 1e-5
+    ffm = FFM(Xt, Yt, ls=0.5)
+    refxy = (benchmark_matmul_double(Xt, Yt, ls=0.5) @ byt).cpu().numpy()
+    assert rel_l2((ffm @ byt).cpu().numpy(), refxy) < 1e-3
+    assert rel_l2(ffm.chunk_forward_example(byt, chunks=3).cpu().numpy(), refxy) < 1e-3
+    refT = (benchmark_matmul_double(Yt, Xt, ls=0.5) @ bt).cpu().numpy()
+    assert rel_l2(ffm.chunk_forward_transpose(bt, chunks=3).cpu().numpy(), refT) < 1e-3
+    blk = block_FFM_matmul(Xt, ls=0.5, blocks_X=2) @ bt
+    assert rel_l2(blk.numpy(), ref) < 1e-3
+    g = ffm.grad(byt).cpu().numpy()
+    assert rel_l2(g, oracle.exact_grad_f32(X, Y, by, 0.5)) < 1e-5
