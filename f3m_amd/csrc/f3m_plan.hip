@@ -163,27 +163,38 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     P->ty = sym ? &P->tx : &P->ty_;
     Scope sc(kPlan, s);
 
-    // root geometry (F3M_src/n_tree.cu:25-46)
-    float xmn[kMaxD], xmx[kMaxD], ymn[kMaxD], ymx[kMaxD];
-    bounding_box(X, N, d, xmn, xmx, s);
-    float edge = root_edge(xmn, xmx, d);
-    if (!sym) {
-        bounding_box(Y, M, d, ymn, ymx, s);
-        float ye = root_edge(ymn, ymx, d);
-        if (ye > edge) edge = ye;
-    }
+    // The loop of F3M_src/n_tree.cu:1075/:1099 divides only while the fullest box holds more than
+    // min_points points, and depth 0 is one box with every point.  A cloud whose points all coincide
+    // cannot be divided either (the reference would compute 0/0 cell indices).  Both cases take the
+    // exact product and need no tree.
+    bool need_tree = (float)N > prm->min_points && (sym || (float)M > prm->min_points);
     Geo gx;
     memset(&gx, 0, sizeof(gx));
-    gx.d = d;
-    gx.edge0 = edge * 1.01f;
-    F3M_REQUIRE(gx.edge0 > 0.f && std::isfinite(gx.edge0), 10, "degenerate point cloud (edge %g)", (double)gx.edge0);
-    // key depth: past 31/d levels the reference's int32 grid keys overflow, past 16 its fp32 centres
-    // stop resolving cells; the tree is never deeper and what is left is summed exactly
-    gx.L = std::min(31 / d, 16);
-    Geo gy = gx;
-    for (int j = 0; j < d; j++) { gx.origin[j] = xmn[j]; gy.origin[j] = sym ? xmn[j] : ymn[j]; }
-    build_sorted_tree(P->tx, X, N, gx, s);
-    if (!sym) build_sorted_tree(P->ty_, Y, M, gy, s);
+    if (need_tree) {
+        // root geometry (F3M_src/n_tree.cu:25-46)
+        float xmn[kMaxD], xmx[kMaxD], ymn[kMaxD], ymx[kMaxD];
+        bounding_box(X, N, d, xmn, xmx, s);
+        float edge = root_edge(xmn, xmx, d);
+        if (!sym) {
+            bounding_box(Y, M, d, ymn, ymx, s);
+            float ye = root_edge(ymn, ymx, d);
+            if (ye > edge) edge = ye;
+        }
+        gx.d = d;
+        gx.edge0 = edge * 1.01f;
+        F3M_REQUIRE(std::isfinite(gx.edge0), 10, "point coordinates are not finite");
+        // key depth: past 31/d levels the reference's int32 grid keys overflow, past 16 its fp32
+        // centres stop resolving cells; the tree is never deeper and what is left is summed exactly
+        gx.L = std::min(31 / d, 16);
+        if (gx.edge0 > 0.f) {
+            Geo gy = gx;
+            for (int j = 0; j < d; j++) { gx.origin[j] = xmn[j]; gy.origin[j] = sym ? xmn[j] : ymn[j]; }
+            build_sorted_tree(P->tx, X, N, gx, s);
+            if (!sym) build_sorted_tree(P->ty_, Y, M, gy, s);
+        } else {
+            need_tree = false;
+        }
+    }
 
     PairList root;
     root.n = 1;
@@ -193,7 +204,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     const PairList *keep = &root;
     P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
     // loop guard of F3M_src/n_tree.cu:1075 (symmetric) and :1099 (two trees)
-    while (keep->n > 0 && (float)P->tx.lev.back().maxcount > prm->min_points &&
+    while (need_tree && keep->n > 0 && (float)P->tx.lev.back().maxcount > prm->min_points &&
            (sym || (float)P->ty_.lev.back().maxcount > prm->min_points)) {
         if ((int)P->tx.lev.size() > gx.L) break;
         divide_tree(P->tx, s);
