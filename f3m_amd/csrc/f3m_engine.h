@@ -23,6 +23,7 @@ struct TreeLevel {
     DBuf<int> off;       // nb+1 offsets into the Morton-sorted point order
     DBuf<uint32_t> prefix;  // nb Morton prefixes (depth*d bits)
     DBuf<float> ctr;     // nb*d box centres, row-major
+    DBuf<int> cell;      // nb*d integer cell coordinates of the box at its depth
     DBuf<int> childstart;   // nb+1: compact id at depth+1 of each box's first child (set by the next level)
 };
 

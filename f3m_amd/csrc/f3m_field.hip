@@ -502,6 +502,81 @@ __global__ void __launch_bounds__(1024) m2l_direct_kernel(const float *__restric
 }
 
 // ------------------------------------------------------------------------------------------------
+// M2L, separable form.  Box centres sit on the regular grid of their depth, so the centre offset of
+// a far pair is (integer cell offset)*edge + (origin_y - origin_x), and the Gaussian factorises over
+// dimensions: K[(a_0..a_{d-1}),(m_0..m_{d-1})] = prod_j E_j[o_j][a_j][m_j] with
+// E_j[o][a][m] = exp(-lcs ((t_a - t_m) edge/2 - (o edge + delta_j))^2).  Applying the d small
+// factors one dimension at a time costs sum_j n_j multiply-adds per node and far pair instead of P.
+// The tables (a few KB, built on the host in fp64) live in LDS; the moment vector ping-pongs between
+// two LDS buffers.  Same sums as m2l_direct_kernel up to rounding.
+
+constexpr int kM2LOffsets = 13;   // cell offsets per dimension that a far pair can have (|dc| < 5 edge)
+
+struct SepMeta {
+    int omin[kMaxD];
+    int NT;      // row length of a table (largest per-dimension node count)
+};
+
+template <int D>
+__global__ void __launch_bounds__(1024) m2l_sep_kernel(const float *__restrict__ tables, int ntab, NodeMeta nm, SepMeta sm,
+                                                        const int *__restrict__ cellx, const int *__restrict__ celly,
+                                                        const int *__restrict__ pairs, const int *__restrict__ rowptr,
+                                                        const float *__restrict__ mom, float *__restrict__ loc)
+{
+    F3M_DYN_SHARED(float, smem);
+    float *tab = smem;                 // ntab
+    float *bufA = smem + ntab;         // P
+    float *bufB = bufA + nm.P;         // P
+    const int bx = blockIdx.x, tid = threadIdx.x, BD = blockDim.x, P = nm.P;
+    const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    if (m0 == m1) return;              // uniform over the workgroup
+    for (int e = tid; e < ntab; e += BD) tab[e] = tables[e];
+    // digit of this lane's node along every dimension, and the flat index with that digit cleared
+    int dig[D], base[D], stride[D];
+    {
+        int st = 1;
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            stride[j] = st;
+            dig[j] = (tid / st) % nm.n[j];
+            base[j] = tid - dig[j] * st;
+            st *= nm.n[j];
+        }
+    }
+    int cx[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) cx[j] = cellx[(long long)bx * D + j] + sm.omin[j];
+    const bool live = tid < P;
+    float acc = 0.f;
+    for (int m = m0; m < m1; m++) {
+        const int by = pairs[2 * (long long)m + 1];
+        __syncthreads();
+        if (live) bufA[tid] = mom[(long long)by * P + tid];
+        __syncthreads();
+        float *in = bufA, *out = bufB;
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            int oi = celly[(long long)by * D + j] - cx[j];
+            oi = oi < 0 ? 0 : (oi >= kM2LOffsets ? kM2LOffsets - 1 : oi);
+            float sum = 0.f;
+            if (live) {
+                const float *row = tab + ((j * kM2LOffsets + oi) * sm.NT + dig[j]) * sm.NT;
+                const float *src = in + base[j];
+                for (int q = 0; q < nm.n[j]; q++) sum = fmaf(row[q], src[q * stride[j]], sum);
+            }
+            if (j == D - 1) {
+                acc += sum;
+            } else {
+                if (live) out[tid] = sum;
+                __syncthreads();
+                float *t = in; in = out; out = t;
+            }
+        }
+    }
+    if (live) loc[(long long)bx * P + tid] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
 // L2P (F3M_src/1_d_conv.cu:554-659): out_i += sum_m L_m(x_i) Loc[box][m].  One lane per point; the
 // product over dimensions >= 1 is reused along dimension 0.
 
@@ -574,7 +649,6 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     if (far.n == 0) return;
     const int P = ns.P;
     F3M_REQUIRE(P <= 1024, 30, "at most 1024 interpolation nodes per box are supported (got %d)", P);
-    (void)m2l_mode;
     set_node_offsets(ns, lx.edge, s);
     NodeMeta nm = meta_of(ns);
     const float factor = 2 / lx.edge;                  // F3M_src/1_d_conv.cu:473
@@ -613,21 +687,63 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 
     // M2L
     F3M_HIP(hipMemsetAsync(loc.get(), 0, sizeof(float) * (size_t)lx.nb * P, s));
-    size_t shm = sizeof(float) * (size_t)P * (d + 1);
-    timer_begin(kM2L, s);
+    int NT = 1;
+    for (int j = 0; j < d; j++) NT = std::max(NT, ns.n[j]);
+    const int ntab = d * kM2LOffsets * NT * NT;
+    const bool separable = m2l_mode == 2 || (m2l_mode == 0 && (size_t)(ntab + 2 * P) * sizeof(float) <= 48 * 1024);
+    if (separable) {
+        F3M_REQUIRE((size_t)(ntab + 2 * P) * sizeof(float) <= 64 * 1024, 31, "separable M2L tables do not fit in LDS");
+        SepMeta sm;
+        sm.NT = NT;
+        std::vector<float> tab((size_t)ntab, 0.f);
+        const double edge = (double)lx.edge, h = edge / 2, lc = (double)lcs;
+        for (int j = 0; j < kMaxD; j++) sm.omin[j] = 0;
+        for (int j = 0; j < d; j++) {
+            const double delta = (double)ty.geo.origin[j] - (double)tx.geo.origin[j];
+            sm.omin[j] = (int)std::floor(-5.0 - delta / edge) - 1;
+            for (int oi = 0; oi < kM2LOffsets; oi++) {
+                const double shift = (double)(sm.omin[j] + oi) * edge + delta;     // c_y - c_x along j
+                for (int a = 0; a < ns.n[j]; a++)
+                    for (int q = 0; q < ns.n[j]; q++) {
+                        double diff = ((double)ns.t[ns.start[j] + a] - (double)ns.t[ns.start[j] + q]) * h - shift;
+                        tab[(((size_t)j * kM2LOffsets + oi) * NT + a) * NT + q] = (float)std::exp(-lc * diff * diff);
+                    }
+            }
+        }
+        DBuf<float> dtab((size_t)ntab);
+        h2d(dtab.get(), tab.data(), tab.size(), s);
+        size_t shs = sizeof(float) * ((size_t)ntab + 2 * (size_t)P);
+        timer_begin(kM2L, s);
+#define F3M_CASE(DD)                                                                                                   \
+    case DD:                                                                                                           \
+        F3M_LAUNCH((m2l_sep_kernel<DD>), lx.nb, bdp, shs, s, dtab.get(), ntab, nm, sm, lx.cell.get(), ly.cell.get(),   \
+                   far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());                                           \
+        break;
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
+#undef F3M_CASE
+        timer_end(s);
+        check_launch("m2l_sep");
+    } else {
+        size_t shm = sizeof(float) * (size_t)P * (d + 1);
+        timer_begin(kM2L, s);
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((m2l_direct_kernel<DD>), lx.nb, bdp, shm, s, ns.noff.get(), P, lx.ctr.get(), ly.ctr.get(),          \
                    far.pairs.get(), far.rowptr.get(), mom.get(), lcs * kLog2e, loc.get());                             \
         break;
-    switch (d) {
-        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
-        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
-    default: throw Error(2, "dimension must be 1..10");
-    }
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
 #undef F3M_CASE
-    timer_end(s);
-    check_launch("m2l");
+        timer_end(s);
+        check_launch("m2l");
+    }
 
     // L2P
     DBuf<int> tilex;

@@ -268,6 +268,8 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     r.off.reset(2);
     r.prefix.reset(1);
     r.ctr.reset(geo.d);
+    r.cell.reset(geo.d);
+    F3M_HIP(hipMemsetAsync(r.cell.get(), 0, sizeof(int) * geo.d, s));
     int off[2] = {0, (int)n};
     uint32_t pf = 0;
     float c[kMaxD];
@@ -308,8 +310,9 @@ __global__ void nonempty_kernel(const int *__restrict__ natpos, long long ncand,
 // stats[0] = number of non-empty children, stats[1] = largest count
 __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__restrict__ cid, long long ncand, int d,
                                    const uint32_t *__restrict__ prefix_prev, const float *__restrict__ ctr_prev,
-                                   float quarter, int *__restrict__ off, uint32_t *__restrict__ prefix,
-                                   float *__restrict__ ctr, int *__restrict__ childstart_prev, int *__restrict__ stats)
+                                   const int *__restrict__ cell_prev, float quarter, int *__restrict__ off,
+                                   uint32_t *__restrict__ prefix, float *__restrict__ ctr, int *__restrict__ cell,
+                                   int *__restrict__ childstart_prev, int *__restrict__ stats)
 {
     long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (nat > ncand) return;
@@ -330,6 +333,7 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
         for (int j = 0; j < d; j++) {
             float step = ((child >> j) & 1) ? quarter : -quarter;      // 0.25*edge*sign, exact
             ctr[(long long)id * d + j] = ctr_prev[(long long)q * d + j] + step;
+            cell[(long long)id * d + j] = 2 * cell_prev[(long long)q * d + j] + ((child >> j) & 1);
         }
         atomicMax(&stats[1], cnt);
     }
@@ -357,11 +361,13 @@ bool divide_tree(Tree &t, hipStream_t s)
     cur.off.reset(bound + 1);
     cur.prefix.reset(bound);
     cur.ctr.reset(bound * d);
+    cur.cell.reset(bound * d);
     prev.childstart.reset((size_t)prev.nb + 1);
     F3M_HIP(hipMemsetAsync(stats.get(), 0, 2 * sizeof(int), s));
     float quarter = 0.25f * prev.edge;
     F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
-               prev.ctr.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), prev.childstart.get(), stats.get());
+               prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
+               prev.childstart.get(), stats.get());
     check_launch("build_level");
     int h[2];
     d2h(h, stats.get(), 2, s);

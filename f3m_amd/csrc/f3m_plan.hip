@@ -3,6 +3,7 @@
 #include "f3m_engine.h"
 
 #include <cmath>
+#include <cstdlib>
 #include <memory>
 
 namespace f3m {
@@ -242,7 +243,10 @@ static void far_level(f3m_plan *P, int level, const float *bs, float *outs, floa
     PlanLevel &L = P->levels[level - 1];
     if (L.far.n == 0) return;
     NodeSet &ns = P->nodeset(L.num_nodes, s);
-    far_field(P->d, P->tx, P->tx.lev[level], *P->ty, P->ty->lev[level], L.far, ns, bs, outs, P->lcs, 0, mom, loc, s);
+    // F3M_M2L=direct|separable forces one form of the M2L kernel (default: separable when its tables fit)
+    int mode = 0;
+    if (const char *e = getenv("F3M_M2L")) mode = !strcmp(e, "direct") ? 1 : (!strcmp(e, "separable") ? 2 : 0);
+    far_field(P->d, P->tx, P->tx.lev[level], *P->ty, P->ty->lev[level], L.far, ns, bs, outs, P->lcs, mode, mom, loc, s);
 }
 
 static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s)
