@@ -3,6 +3,8 @@
 #include "f3m_engine.h"
 
 #include <cmath>
+#include <cstdlib>
+#include <cstring>
 
 namespace f3m {
 
@@ -270,34 +272,226 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
     }
 }
 
+// Near field with the exponent on the matrix pipe.  The exponent of a pair,
+//   t = 2x'.y' - |y'|^2 - |x'|^2   (x', y' shifted to the x-box centre and scaled by sqrt(lcs log2 e)),
+// is an inner product over the D+1 components (2y'_k, -|y'|^2) . (x'_k, 1) plus a per-target constant.
+// Every fp32 operand is split into two f16 values, v = hi + lo (|v - hi - lo| <= 2^-22 |v|), and the
+// products hi.hi + hi.lo + lo.hi of all components fill the 16 inner slots of one
+// v_mfma_f32_32x32x16_f16 (two instructions for D >= 5), accumulated in fp32 on top of C = -|x'|^2.
+// The f16 matrix pipe runs beside the vector ALU, which is left with one exp2 and one fused
+// multiply-add per pair.  A wavefront owns two tiles of 32 targets (lanes l and l+32 hold the same
+// target and different source rows; their partial sums are combined once at the end), a workgroup
+// of four wavefronts 256 targets.  Sources of a y box are staged through LDS as ready-made matrix
+// operands, padded with zero-weight sources to a multiple of 32.
+// Valid while |x'|, |y'| stay small enough for the split (the host checks the box size against the
+// lengthscale and otherwise launches near_kernel).
+
+constexpr int kNearTPW = 2;                         // target tiles (of 32) per wavefront
+constexpr int kNearMfmaBlock = 256;                 // lanes per workgroup
+constexpr int kNearMfmaTargets = (kNearMfmaBlock / kWave) * kNearTPW * 32;
+
+// inner slot s of the matrix product: component s/3; s%3 = 0: hi.hi, 1: (source hi).(target lo), 2: (source lo).(target hi)
+template <int D>
+__device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, int hh, bool source)
+{
+    h8 v;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        const int slot = 16 * n + 8 * hh + e;
+        if (slot < 3 * (D + 1)) {
+            const int c = slot / 3, tau = slot % 3;
+            v[e] = source ? (tau == 2 ? lo[c] : hi[c]) : (tau == 1 ? lo[c] : hi[c]);
+        } else {
+            v[e] = to_half(0.f);
+        }
+    }
+    return v;
+}
+
+template <int D>
+__global__ void __launch_bounds__(kNearMfmaBlock, 2) near_h_kernel(
+    const float *__restrict__ xs, long long N, const float *__restrict__ ys, long long M, const float *__restrict__ bs,
+    float *__restrict__ outs, const int *__restrict__ offx, const int *__restrict__ offy, const float *__restrict__ ctrx,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc)
+{
+    constexpr int C = D + 1;
+    constexpr int NS = (3 * C + 15) / 16;           // matrix instructions per tile
+    __shared__ h8 aop[NS][2][kNearCap];
+    __shared__ __align__(16) float sb[kNearCap];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+    const int bx = find_box(tileoff, nbx, blockIdx.x);
+    const int tile = blockIdx.x - tileoff[bx];
+    const int x0 = offx[bx] + tile * kNearMfmaTargets, x1 = offx[bx + 1];
+    float cx[D];
+#pragma unroll
+    for (int k = 0; k < D; k++) cx[k] = ctrx[(long long)bx * D + k];
+    h8 bop[kNearTPW][NS];
+    f32x16 cinit[kNearTPW];
+    float acc[kNearTPW];
+    bool live[kNearTPW];
+#pragma unroll
+    for (int q = 0; q < kNearTPW; q++) {
+        const int t0 = x0 + (wave * kNearTPW + q) * 32;
+        const int i = t0 + col;
+        live[q] = t0 < x1;
+        half_t hi[C], lo[C];
+        float nx2 = 0.f;
+#pragma unroll
+        for (int k = 0; k < C; k++) {
+            float v = 1.f;
+            if (k < D) {
+                v = (i < x1) ? sc * (xs[(long long)k * N + i] - cx[k]) : 0.f;
+                nx2 -= v * v;
+            }
+            hi[k] = to_half(v);
+            lo[k] = to_half(v - half_to_float(hi[k]));
+        }
+#pragma unroll
+        for (int n = 0; n < NS; n++) {
+            h8 v0 = split_operand<D>(hi, lo, n, 0, false), v1 = split_operand<D>(hi, lo, n, 1, false);
+            bop[q][n] = half ? v1 : v0;
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r++) cinit[q][r] = nx2;
+        acc[q] = 0.f;
+    }
+    const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    for (int m = m0; m < m1; m++) {
+        const int by = pairs[2 * (long long)m + 1];
+        const int s0 = offy[by], s1 = offy[by + 1];
+        for (int base = s0; base < s1; base += kNearCap) {
+            const int cnt = (s1 - base) < kNearCap ? (s1 - base) : kNearCap;
+            const int cntp = (cnt + 31) & ~31;
+            __syncthreads();
+            for (int jj = tid; jj < cntp; jj += kNearMfmaBlock) {
+                half_t hi[C], lo[C];
+                float ny2 = 0.f;
+#pragma unroll
+                for (int k = 0; k < C; k++) {
+                    float v;
+                    if (k < D) {
+                        float y = (jj < cnt) ? sc * (ys[(long long)k * M + base + jj] - cx[k]) : 0.f;
+                        ny2 -= y * y;
+                        v = 2.f * y;
+                    } else {
+                        v = ny2;
+                    }
+                    hi[k] = to_half(v);
+                    lo[k] = to_half(v - half_to_float(hi[k]));
+                }
+#pragma unroll
+                for (int n = 0; n < NS; n++) {
+                    aop[n][0][jj] = split_operand<D>(hi, lo, n, 0, true);
+                    aop[n][1][jj] = split_operand<D>(hi, lo, n, 1, true);
+                }
+                sb[jj] = (jj < cnt) ? bs[base + jj] : 0.f;
+            }
+            __syncthreads();
+            if (!live[0]) continue;                 // uniform per wavefront
+            for (int j0 = 0; j0 < cntp; j0 += 32) {
+                h8 a[NS];
+#pragma unroll
+                for (int n = 0; n < NS; n++) a[n] = aop[n][half][j0 + col];
+                float4 bq[4];
+#pragma unroll
+                for (int g = 0; g < 4; g++) bq[g] = *reinterpret_cast<const float4 *>(&sb[j0 + 8 * g + 4 * half]);
+                f32x16 t0 = cinit[0];
+#pragma unroll
+                for (int n = 0; n < NS; n++) t0 = mfma_32x32x16_f16(a[n], bop[0][n], t0);
+                if (live[1]) {                      // uniform per wavefront
+                    f32x16 t1 = cinit[1];
+#pragma unroll
+                    for (int n = 0; n < NS; n++) t1 = mfma_32x32x16_f16(a[n], bop[1][n], t1);
+                    float s0a = acc[0], s1a = acc[1];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        s0a = fmaf(fast_exp2(t0[4 * g + 0]), bq[g].x, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 1]), bq[g].y, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 2]), bq[g].z, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 3]), bq[g].w, s0a);
+                    }
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        s1a = fmaf(fast_exp2(t1[4 * g + 0]), bq[g].x, s1a);
+                        s1a = fmaf(fast_exp2(t1[4 * g + 1]), bq[g].y, s1a);
+                        s1a = fmaf(fast_exp2(t1[4 * g + 2]), bq[g].z, s1a);
+                        s1a = fmaf(fast_exp2(t1[4 * g + 3]), bq[g].w, s1a);
+                    }
+                    acc[0] = s0a;
+                    acc[1] = s1a;
+                } else {
+                    float s0a = acc[0];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        s0a = fmaf(fast_exp2(t0[4 * g + 0]), bq[g].x, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 1]), bq[g].y, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 2]), bq[g].z, s0a);
+                        s0a = fmaf(fast_exp2(t0[4 * g + 3]), bq[g].w, s0a);
+                    }
+                    acc[0] = s0a;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < kNearTPW; q++) {
+        if (!live[q]) continue;
+        float total = acc[q] + wave_shfl_xor_f(acc[q], 32);
+        const int i = x0 + (wave * kNearTPW + q) * 32 + col;
+        if (half == 0 && i < x1) outs[i] += total;
+    }
+}
+
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s)
 {
     if (list.n == 0) return;
+    // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to
+    // ~2^-22 |y'|^2; it is used while the farthest listed source stays within |y'| <= 20 of the x-box
+    // centre in scaled units (box edge at most ~2 lengthscales), otherwise the all-vector kernel.
+    // F3M_NEAR=valu|mfma overrides the choice.
+    const float sc_edge = sqrtf(lcs * kLog2e) * lx.edge;
+    bool use_mfma = sc_edge * 5.5f * sqrtf((float)d) <= 20.f;
+    if (const char *env = getenv("F3M_NEAR")) use_mfma = !strcmp(env, "mfma") ? true : (!strcmp(env, "valu") ? false : use_mfma);
     constexpr int T = 1;
-    // workgroup size: whole boxes where possible (multiple of the wave size, at most 512 lanes)
+    // all-vector kernel: whole boxes per workgroup where possible (multiple of the wave size, <= 512 lanes)
     int bd = ((lx.maxcount + kWave - 1) / kWave) * kWave;
     if (bd > 512) bd = 256;
     if (bd < kWave) bd = kWave;
     DBuf<int> flag((size_t)lx.nb), tileoff;
     F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
     check_launch("mark_rows");
-    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, bd * T, tileoff, s);
+    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, use_mfma ? kNearMfmaTargets : bd * T, tileoff, s);
     if (ntiles == 0) return;
     float sc = sqrtf(lcs * kLog2e);
     timer_begin(kNear, s);
+    if (use_mfma) {
+#define F3M_CASE(DD)                                                                                                  \
+    case DD:                                                                                                          \
+        F3M_LAUNCH((near_h_kernel<DD>), ntiles, kNearMfmaBlock, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs,  \
+                   outs, lx.off.get(), ly.off.get(), lx.ctr.get(), list.pairs.get(), list.rowptr.get(),               \
+                   tileoff.get(), lx.nb, sc);                                                                         \
+        break;
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
+#undef F3M_CASE
+    } else {
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
         F3M_LAUNCH((near_kernel<DD, T>), ntiles, bd, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs, outs,          \
                    lx.off.get(), ly.off.get(), lx.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
                    lx.nb, sc);                                                                                        \
         break;
-    switch (d) {
-        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
-        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
-    default: throw Error(2, "dimension must be 1..10");
-    }
+        switch (d) {
+            F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+            F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+        default: throw Error(2, "dimension must be 1..10");
+        }
 #undef F3M_CASE
+    }
     timer_end(s);
     check_launch("near_field");
 }

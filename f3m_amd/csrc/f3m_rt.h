@@ -167,11 +167,136 @@ __device__ inline unsigned long long wave_ballot(bool p) { return emu::ballot(p)
 __device__ inline unsigned lane_id() { return emu::S().cur->tid % 64; }
 __device__ inline float fast_exp2(float x) { return exp2f(x); }
 __device__ inline int wave_shfl_i(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }
+__device__ inline float wave_shfl_xor_f(float v, int mask)
+{
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    u = emu::shfl_bits(u, (int)(lane_id() ^ (unsigned)mask));
+    memcpy(&v, &u, 4);
+    return v;
+}
+struct f32x16 {
+    float v[16];
+    float &operator[](int i) { return v[i]; }
+    const float &operator[](int i) const { return v[i]; }
+};
+// D = A(32x2) B(2x32) + C on one wavefront: lane l supplies A[l%32][l/32] and B[l/32][l%32] and
+// holds D[8(r/4) + 4(l/32) + r%4][l%32] in element r
+__device__ inline f32x16 mfma_32x32x2(float a, float b, f32x16 c)
+{
+    uint32_t A[64], B[64];
+    uint32_t ua, ub;
+    memcpy(&ua, &a, 4);
+    memcpy(&ub, &b, 4);
+    emu::gather_bits(ua, A);
+    emu::gather_bits(ub, B);
+    const unsigned l = lane_id(), j = l & 31, h = l >> 5;
+    for (int r = 0; r < 16; r++) {
+        unsigned i = 8 * (r / 4) + 4 * h + (r % 4);
+        float a0, a1, b0, b1;
+        memcpy(&a0, &A[i], 4); memcpy(&a1, &A[i + 32], 4);
+        memcpy(&b0, &B[j], 4); memcpy(&b1, &B[j + 32], 4);
+        c.v[r] = fmaf(a1, b1, fmaf(a0, b0, c.v[r]));
+    }
+    return c;
+}
+// IEEE binary16 stand-ins for the CPU build (round to nearest even, subnormals kept)
+struct half_t { uint16_t bits; };
+__device__ inline half_t to_half(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint32_t sign = (x >> 16) & 0x8000u, mant = x & 0x7fffffu;
+    int exp = (int)((x >> 23) & 0xff) - 127 + 15;
+    uint16_t h;
+    if (((x >> 23) & 0xff) == 0xff) h = (uint16_t)(sign | 0x7c00u | (mant ? 0x200u : 0));
+    else if (exp >= 31) h = (uint16_t)(sign | 0x7c00u);
+    else if (exp <= 0) {
+        if (exp < -10) h = (uint16_t)sign;
+        else {
+            mant |= 0x800000u;
+            int shift = 14 - exp;
+            uint32_t hm = mant >> shift, rem = mant & ((1u << shift) - 1), halfway = 1u << (shift - 1);
+            if (rem > halfway || (rem == halfway && (hm & 1))) hm++;
+            h = (uint16_t)(sign | hm);
+        }
+    } else {
+        uint32_t hm = mant >> 13, rem = mant & 0x1fffu;
+        uint32_t v = ((uint32_t)exp << 10) | hm;
+        if (rem > 0x1000u || (rem == 0x1000u && (hm & 1))) v++;
+        h = (uint16_t)(sign | v);
+    }
+    return half_t{h};
+}
+__device__ inline float half_to_float(half_t hv)
+{
+    uint32_t h = hv.bits, sign = (h & 0x8000u) << 16, exp = (h >> 10) & 0x1f, mant = h & 0x3ffu, x;
+    if (exp == 0) {
+        if (mant == 0) x = sign;
+        else {
+            int e = -1;
+            do { e++; mant <<= 1; } while (!(mant & 0x400u));
+            x = sign | ((uint32_t)(127 - 15 - e) << 23) | ((mant & 0x3ffu) << 13);
+        }
+    } else if (exp == 31) x = sign | 0x7f800000u | (mant << 13);
+    else x = sign | ((exp - 15 + 127) << 23) | (mant << 13);
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+struct h8 {
+    half_t v[8];
+    half_t &operator[](int i) { return v[i]; }
+    const half_t &operator[](int i) const { return v[i]; }
+};
+// D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation: lane l supplies row l%32 of A and
+// column l%32 of B for the eight inner indices of its half-wave; the output layout is that of
+// mfma_32x32x2
+__device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
+{
+    uint32_t A[4][64], B[4][64];
+    uint32_t wa[4], wb[4];
+    memcpy(wa, &a, 16);
+    memcpy(wb, &b, 16);
+    for (int w = 0; w < 4; w++) { emu::gather_bits(wa[w], A[w]); emu::gather_bits(wb[w], B[w]); }
+    const unsigned l = lane_id(), j = l & 31, h = l >> 5;
+    for (int r = 0; r < 16; r++) {
+        unsigned i = 8 * (r / 4) + 4 * h + (r % 4);
+        double acc = c.v[r];
+        for (int hh = 0; hh < 2; hh++)
+            for (int e = 0; e < 8; e++) {
+                uint32_t aw = A[e / 2][i + 32 * hh], bw = B[e / 2][j + 32 * hh];
+                half_t ah{(uint16_t)((e & 1) ? (aw >> 16) : (aw & 0xffff))}, bh{(uint16_t)((e & 1) ? (bw >> 16) : (bw & 0xffff))};
+                acc += (double)half_to_float(ah) * (double)half_to_float(bh);
+            }
+        c.v[r] = (float)acc;
+    }
+    return c;
+}
 #else
 __device__ __forceinline__ unsigned long long wave_ballot(bool p) { return __ballot(p); }
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ int wave_shfl_i(int v, int src) { return __shfl(v, src, 64); }
+__device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+// D = A(32x2) B(2x32) + C on the matrix pipe (v_mfma_f32_32x32x2_f32): lane l supplies A[l%32][l/32]
+// and B[l/32][l%32] and holds D[8(r/4) + 4(l/32) + r%4][l%32] in element r
+__device__ __forceinline__ f32x16 mfma_32x32x2(float a, float b, f32x16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+typedef _Float16 half_t;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ half_t to_half(float f) { return (_Float16)f; }
+__device__ __forceinline__ float half_to_float(half_t h) { return (float)h; }
+// D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation (v_mfma_f32_32x32x16_f16): lane l
+// supplies row l%32 of A and column l%32 of B for the eight inner indices of its half-wave; the
+// output layout is that of mfma_32x32x2
+__device__ __forceinline__ f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
 #endif
 
 }  // namespace f3m

@@ -24,6 +24,7 @@
 #define __forceinline__ inline
 #define __shared__ static
 #define __launch_bounds__(...)
+#define __align__(n) alignas(n)
 
 struct dim3 {
     unsigned x, y, z;
@@ -178,6 +179,17 @@ inline uint32_t shfl_bits(uint32_t v, int src)
     w.vals[slot][lane] = v;
     wave_barrier(w);
     return w.vals[slot][src & (WAVE - 1)];
+}
+
+// every lane's value of the wave (exited lanes keep their last deposit)
+inline void gather_bits(uint32_t v, uint32_t *out)
+{
+    Wave &w = wave();
+    int slot = w.gen & 1;
+    unsigned lane = S().cur->tid % WAVE;
+    w.vals[slot][lane] = v;
+    wave_barrier(w);
+    memcpy(out, w.vals[slot], sizeof(uint32_t) * WAVE);
 }
 
 struct Idx { unsigned x; };

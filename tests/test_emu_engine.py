@@ -33,6 +33,13 @@ def _cloud(name, rng):
 PRM = dict(ls=0.6, min_points=60, nr_of_interpolation=27, small_field_points=40)
 
 
+@pytest.fixture(autouse=True)
+def _vector_near_kernel(monkeypatch):
+    # the emulated matrix instruction costs two fiber barriers per call; the bulk of these tests
+    # therefore runs the all-vector near-field kernel and test_mfma_near_field covers the other one
+    monkeypatch.setenv("F3M_NEAR", "valu")
+
+
 @pytest.mark.parametrize("name", ["uniform3", "normal2", "uniform1", "uniform4", "asym3", "dups_faces"])
 def test_tree_and_lists_bit_exact(oracle, name):
     X, Y = _cloud(name, np.random.default_rng(21))
@@ -91,6 +98,27 @@ def test_stages_and_product(oracle, name, P):
     exact = oracle.exact_f64(X, X if Y is None else Y, b, prm["ls"])
     assert rel_l2(got, exact) <= 1.5 * rel_l2(ora.apply(b), exact) + 1e-6
     assert rel_l2(ee.kmvm(X, Y, b, **prm), got) == 0.0
+
+
+def test_mfma_near_field(oracle, monkeypatch):
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    rng = np.random.default_rng(5)
+    for d, n in ((3, 700), (2, 500), (4, 600)):
+        X = rng.random((n, d), dtype=f32)
+        Y = (rng.random((n - 123, d)) * 1.1).astype(f32)
+        b = rng.standard_normal((n - 123, 1)).astype(f32)
+        prm = dict(ls=0.4, min_points=50, nr_of_interpolation=8, small_field_points=30)
+        eng = ee.Plan(X, Y, **prm)
+        ora = oracle.Plan(X, Y, **prm)
+        checked = 0
+        for k in range(1, eng.depth + 1):
+            sz = eng.level_sizes(k)
+            for which in ("small", "keep"):
+                if sz["n" + which] and (which == "small" or k == eng.depth):
+                    assert rel_l2(eng.near_level(k, which, b), ora.near_level(k - 1, which, b)) < 1e-5
+                    checked += 1
+        assert checked > 0
+        assert rel_l2(eng.apply(b), ora.apply(b)) < 1e-5
 
 
 def test_no_division_returns_exact_product(oracle):
