@@ -76,8 +76,7 @@ struct NodeSet {
     int d = 0, P = 0, S1 = 0;
     int n[kMaxD] = {0};
     int start[kMaxD] = {0};
-    std::vector<float> t, w;        // concatenated 1-D nodes and barycentric weights (host)
-    DBuf<float> dt, dw;             // device copies
+    DBuf<float> dt, dw;             // concatenated 1-D nodes and barycentric weights
     DBuf<float> noff;               // (P,d) node offsets of a box of the current level
 };
 void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s);

@@ -155,17 +155,19 @@ __global__ void mark_cols_kernel(const int *__restrict__ pairs, long long n, int
     if (t < n) flag[pairs[2 * t + 1]] = 1;
 }
 
-// tileoff (nb+1) = exclusive scan of tiles per box; returns the total number of tiles
-static int build_tiles(const int *off, const int *flag, int nb, int tile, DBuf<int> &tileoff, hipStream_t s)
+// tileoff (nb+1) = exclusive scan of tiles per box.  Returns an upper bound of the number of tiles
+// (nb + npoints/tile) to launch with; workgroups past tileoff[nb] exit at once, so the host never
+// waits for the exact count.
+static int build_tiles(const int *off, const int *flag, int nb, long long npoints, int tile, DBuf<int> &tileoff, hipStream_t s)
 {
     DBuf<int> nt((size_t)nb);
     tileoff.reset((size_t)nb + 1);
     F3M_LAUNCH(tiles_per_box_kernel, cdiv(nb, 256), 256, 0, s, off, flag, nb, tile, nt.get());
     check_launch("tiles_per_box");
     exclusive_scan_i32(nt.get(), nb, tileoff.get(), s);
-    int total = 0;
-    d2h(&total, tileoff.get() + nb, 1, s);
-    return total;
+    long long bound = (long long)nb + npoints / tile;
+    F3M_REQUIRE(bound < (1ll << 31) - 1, 32, "too many work items");
+    return (int)bound;
 }
 
 __device__ inline int find_box(const int *__restrict__ tileoff, int nb, int tileid)
@@ -199,6 +201,7 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
     __shared__ float4 sv[NV][kNearCap];
     __shared__ float sb[kNearCap];
     const int tid = threadIdx.x, BD = blockDim.x;
+    if ((int)blockIdx.x >= tileoff[nbx]) return;    // launched with an upper bound of the tile count
     const int bx = find_box(tileoff, nbx, blockIdx.x);
     const int tile = blockIdx.x - tileoff[bx];
     const int x0 = offx[bx] + tile * BD * T, x1 = offx[bx + 1];
@@ -319,6 +322,7 @@ __global__ void __launch_bounds__(kNearMfmaBlock, 2) near_h_kernel(
     __shared__ h8 aop[NS][2][kNearCap];
     __shared__ __align__(16) float sb[kNearCap];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
+    if ((int)blockIdx.x >= tileoff[nbx]) return;    // launched with an upper bound of the tile count
     const int bx = find_box(tileoff, nbx, blockIdx.x);
     const int tile = blockIdx.x - tileoff[bx];
     const int x0 = offx[bx] + tile * kNearMfmaTargets, x1 = offx[bx + 1];
@@ -461,8 +465,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     DBuf<int> flag((size_t)lx.nb), tileoff;
     F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
     check_launch("mark_rows");
-    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, use_mfma ? kNearMfmaTargets : bd * T, tileoff, s);
-    if (ntiles == 0) return;
+    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? kNearMfmaTargets : bd * T, tileoff, s);
     float sc = sqrtf(lcs * kLog2e);
     timer_begin(kNear, s);
     if (use_mfma) {
@@ -499,6 +502,74 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 // ------------------------------------------------------------------------------------------------
 // interpolation nodes (F3M_src/n_tree.cu:265-349, F3M_src/1_d_conv.cu:850-884)
 
+struct NodeMeta {
+    int n[kMaxD];
+    int start[kMaxD];
+    int S1, P;
+};
+
+static NodeMeta meta_of(const NodeSet &ns)
+{
+    NodeMeta nm;
+    for (int k = 0; k < kMaxD; k++) { nm.n[k] = ns.n[k] > 0 ? ns.n[k] : 1; nm.start[k] = ns.start[k]; }
+    nm.S1 = ns.S1;
+    nm.P = ns.P;
+    return nm;
+}
+
+// 1-D first-kind Chebyshev nodes t_i = cos((2i+1)pi/(2n)) and barycentric weights
+// w_i = (-1)^i sin((2i+1)pi/(2n)) of every dimension, pi as a float (F3M_src/n_tree.cu:265-285)
+__global__ void nodes_kernel(NodeMeta nm, int d, float *__restrict__ t, float *__restrict__ w)
+{
+    int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= nm.S1) return;
+    int j = 0;
+    while (j + 1 < d && e >= nm.start[j + 1]) j++;
+    const int i = e - nm.start[j], n = nm.n[j];
+    const float PI = 3.14159274101257324f;
+    float a = (float)i;
+    a = a * 2.0f;
+    a = a + 1.0f;
+    a = a * PI;
+    a = a / (float)(2 * (n - 1) + 2);
+    t[e] = cosf(a);
+    double sg = (i % 2 == 0) ? 1.0 : -1.0;
+    w[e] = (float)(sg * sin(((2. * (double)i + 1.) * (double)PI) / (2. * (double)(n - 1) + 2.)));
+}
+
+// node position inside a box relative to its centre: cheb*edge/2 + edge/2 (F3M_src/n_tree.cu:510)
+__global__ void node_offsets_kernel(NodeMeta nm, int d, const float *__restrict__ t, float edge, float *__restrict__ noff)
+{
+    int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= nm.P * d) return;
+    int m = e / d, j = e % d, cum = 1;
+    for (int k = 0; k < j; k++) cum *= nm.n[k];
+    int a = (m / cum) % nm.n[j];
+    float v = t[nm.start[j] + a] * edge;
+    v = v / 2.f;
+    noff[e] = v + edge / 2.f;
+}
+
+// tables of the separable M2L: E_j[o][a][q] = exp(-lcs ((t_a - t_q) edge/2 - ((omin_j+o) edge + delta_j))^2)
+struct SepGeo {
+    double delta[kMaxD];
+    int omin[kMaxD];
+};
+__global__ void sep_tables_kernel(NodeMeta nm, int d, int NT, int noffsets, const float *__restrict__ t, double edge, double lcs,
+                                  SepGeo g, float *__restrict__ tab)
+{
+    int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= d * noffsets * NT * NT) return;
+    int q = e % NT, a = (e / NT) % NT, oi = (e / (NT * NT)) % noffsets, j = e / (NT * NT * noffsets);
+    float v = 0.f;
+    if (a < nm.n[j] && q < nm.n[j]) {
+        double shift = (double)(g.omin[j] + oi) * edge + g.delta[j];
+        double diff = ((double)t[nm.start[j] + a] - (double)t[nm.start[j] + q]) * (edge / 2) - shift;
+        v = (float)exp(-lcs * diff * diff);
+    }
+    tab[e] = v;
+}
+
 void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s)
 {
     ns.d = d;
@@ -519,50 +590,21 @@ void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s)
         ns.S1 += pick;
         ns.P *= pick;
     }
-    ns.t.assign(ns.S1, 0.f);
-    ns.w.assign(ns.S1, 0.f);
-    const float PI = (float)(atan(1.) * 4.);
-    for (int j = 0; j < d; j++)
-        for (int i = 0; i < ns.n[j]; i++) {
-            float a = (float)i;
-            a = a * 2.0f;
-            a = a + 1.0f;
-            a = a * PI;
-            a = a / (float)(2 * (ns.n[j] - 1) + 2);
-            ns.t[ns.start[j] + i] = cosf(a);
-            double sgn = (i % 2 == 0) ? 1.0 : -1.0;
-            ns.w[ns.start[j] + i] =
-                (float)(sgn * sin(((2. * (double)(float)i + 1.) * (double)PI) / (2. * (double)(float)(ns.n[j] - 1.0) + 2.)));
-        }
     ns.dt.reset(ns.S1);
     ns.dw.reset(ns.S1);
-    h2d(ns.dt.get(), ns.t.data(), ns.S1, s);
-    h2d(ns.dw.get(), ns.w.data(), ns.S1, s);
+    NodeMeta nm = meta_of(ns);
+    F3M_LAUNCH(nodes_kernel, cdiv(ns.S1, 64), 64, 0, s, nm, d, ns.dt.get(), ns.dw.get());
+    check_launch("nodes");
     ns.noff.reset((size_t)ns.P * d);
 }
 
 void set_node_offsets(NodeSet &ns, float edge, hipStream_t s)
 {
-    // node position inside a box relative to its centre: cheb*edge/2 + edge/2 (n_tree.cu:510)
-    std::vector<float> h((size_t)ns.P * ns.d);
-    int cum = 1;
-    for (int j = 0; j < ns.d; j++) {
-        for (int m = 0; m < ns.P; m++) {
-            int a = (m / cum) % ns.n[j];
-            float v = ns.t[ns.start[j] + a] * edge;
-            v = v / 2.f;
-            h[(size_t)m * ns.d + j] = v + edge / 2.f;
-        }
-        cum *= ns.n[j];
-    }
-    h2d(ns.noff.get(), h.data(), h.size(), s);
+    NodeMeta nm = meta_of(ns);
+    F3M_LAUNCH(node_offsets_kernel, cdiv((long long)ns.P * ns.d, 256), 256, 0, s, nm, ns.d, ns.dt.get(), edge, ns.noff.get());
+    check_launch("node_offsets");
 }
 
-struct NodeMeta {
-    int n[kMaxD];
-    int start[kMaxD];
-    int S1, P;
-};
 
 // 1-D barycentric basis values of one coordinate (F3M_src/1_d_conv.cu:418-448 and :217-238):
 // l_a = (w_a/(t-t_a)) / sum_l w_l/(t-t_l), or the unit vector when t hits a node exactly.
@@ -604,6 +646,7 @@ __global__ void __launch_bounds__(1024) p2m_kernel(const float *__restrict__ ys,
     float *snw = smem + nm.S1;               // S1
     float *sl = smem + 2 * nm.S1;            // kP2MSub * S1: per point, per dimension basis values
     const int tid = threadIdx.x, BD = blockDim.x;
+    if ((int)blockIdx.x >= tileoff[nb]) return;     // launched with an upper bound of the chunk count
     const int box = find_box(tileoff, nb, blockIdx.x);
     const int chunk = blockIdx.x - tileoff[box];
     const int p0 = off[box] + chunk * kP2MChunk;
@@ -790,6 +833,7 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict_
     float *sloc = smem + 2 * nm.S1;          // P
     float *sl = sloc + nm.P;                 // kL2PBlock * S1p
     const int tid = threadIdx.x;
+    if ((int)blockIdx.x >= tileoff[nb]) return;     // launched with an upper bound of the chunk count
     const int box = find_box(tileoff, nb, blockIdx.x);
     const int chunk = blockIdx.x - tileoff[box];
     const int i = off[box] + chunk * kL2PBlock + tid;
@@ -827,15 +871,6 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict_
     outs[i] += acc;
 }
 
-static NodeMeta meta_of(const NodeSet &ns)
-{
-    NodeMeta nm;
-    for (int k = 0; k < kMaxD; k++) { nm.n[k] = ns.n[k] > 0 ? ns.n[k] : 1; nm.start[k] = ns.start[k]; }
-    nm.S1 = ns.S1;
-    nm.P = ns.P;
-    return nm;
-}
-
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode, float *mom_out, float *loc_out,
                hipStream_t s)
@@ -843,7 +878,6 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     if (far.n == 0) return;
     const int P = ns.P;
     F3M_REQUIRE(P <= 1024, 30, "at most 1024 interpolation nodes per box are supported (got %d)", P);
-    set_node_offsets(ns, lx.edge, s);
     NodeMeta nm = meta_of(ns);
     const float factor = 2 / lx.edge;                  // F3M_src/1_d_conv.cu:473
     // participating boxes: x boxes with a non-empty far row, y boxes that occur in the far list
@@ -856,7 +890,7 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 
     // P2M
     DBuf<int> tiley;
-    int nty = build_tiles(ly.off.get(), fy.get(), ly.nb, kP2MChunk, tiley, s);
+    int nty = build_tiles(ly.off.get(), fy.get(), ly.nb, ty.n, kP2MChunk, tiley, s);
     DBuf<float> partial((size_t)std::max(1, nty) * P), mom((size_t)ly.nb * P), loc((size_t)lx.nb * P);
     int bdp = ((P + kWave - 1) / kWave) * kWave;
     size_t shp = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)kP2MSub * ns.S1);
@@ -889,23 +923,17 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         F3M_REQUIRE((size_t)(ntab + 2 * P) * sizeof(float) <= 64 * 1024, 31, "separable M2L tables do not fit in LDS");
         SepMeta sm;
         sm.NT = NT;
-        std::vector<float> tab((size_t)ntab, 0.f);
-        const double edge = (double)lx.edge, h = edge / 2, lc = (double)lcs;
-        for (int j = 0; j < kMaxD; j++) sm.omin[j] = 0;
+        SepGeo sg;
+        const double edge = (double)lx.edge;
+        for (int j = 0; j < kMaxD; j++) { sm.omin[j] = 0; sg.omin[j] = 0; sg.delta[j] = 0; }
         for (int j = 0; j < d; j++) {
-            const double delta = (double)ty.geo.origin[j] - (double)tx.geo.origin[j];
-            sm.omin[j] = (int)std::floor(-5.0 - delta / edge) - 1;
-            for (int oi = 0; oi < kM2LOffsets; oi++) {
-                const double shift = (double)(sm.omin[j] + oi) * edge + delta;     // c_y - c_x along j
-                for (int a = 0; a < ns.n[j]; a++)
-                    for (int q = 0; q < ns.n[j]; q++) {
-                        double diff = ((double)ns.t[ns.start[j] + a] - (double)ns.t[ns.start[j] + q]) * h - shift;
-                        tab[(((size_t)j * kM2LOffsets + oi) * NT + a) * NT + q] = (float)std::exp(-lc * diff * diff);
-                    }
-            }
+            sg.delta[j] = (double)ty.geo.origin[j] - (double)tx.geo.origin[j];
+            sm.omin[j] = sg.omin[j] = (int)std::floor(-5.0 - sg.delta[j] / edge) - 1;
         }
         DBuf<float> dtab((size_t)ntab);
-        h2d(dtab.get(), tab.data(), tab.size(), s);
+        F3M_LAUNCH(sep_tables_kernel, cdiv(ntab, 256), 256, 0, s, nm, d, NT, kM2LOffsets, ns.dt.get(), edge, (double)lcs, sg,
+                   dtab.get());
+        check_launch("sep_tables");
         size_t shs = sizeof(float) * ((size_t)ntab + 2 * (size_t)P);
         timer_begin(kM2L, s);
 #define F3M_CASE(DD)                                                                                                   \
@@ -922,6 +950,7 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         timer_end(s);
         check_launch("m2l_sep");
     } else {
+        set_node_offsets(ns, lx.edge, s);
         size_t shm = sizeof(float) * (size_t)P * (d + 1);
         timer_begin(kM2L, s);
 #define F3M_CASE(DD)                                                                                                   \
@@ -941,7 +970,7 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 
     // L2P
     DBuf<int> tilex;
-    int ntx = build_tiles(lx.off.get(), fx.get(), lx.nb, kL2PBlock, tilex, s);
+    int ntx = build_tiles(lx.off.get(), fx.get(), lx.nb, tx.n, kL2PBlock, tilex, s);
     size_t shl = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)P + (size_t)kL2PBlock * (ns.S1 | 1));
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \

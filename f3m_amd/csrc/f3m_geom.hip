@@ -245,6 +245,19 @@ static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int bi
     }
 }
 
+// depth 0: one box with every point, centred at origin + edge0/2 (F3M_src/n_tree.cu:86-95)
+__global__ void root_level_kernel(Geo g, int n, int *__restrict__ off, uint32_t *__restrict__ prefix, float *__restrict__ ctr,
+                                  int *__restrict__ cell)
+{
+    int j = threadIdx.x;
+    if (j == 0) { off[0] = 0; off[1] = n; prefix[0] = 0u; }
+    if (j < g.d) {
+        float half = 0.5f * g.edge0;
+        ctr[j] = g.origin[j] + half;
+        cell[j] = 0;
+    }
+}
+
 void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s)
 {
     t.geo = geo;
@@ -269,15 +282,8 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     r.prefix.reset(1);
     r.ctr.reset(geo.d);
     r.cell.reset(geo.d);
-    F3M_HIP(hipMemsetAsync(r.cell.get(), 0, sizeof(int) * geo.d, s));
-    int off[2] = {0, (int)n};
-    uint32_t pf = 0;
-    float c[kMaxD];
-    float half = 0.5f * geo.edge0;
-    for (int j = 0; j < geo.d; j++) c[j] = geo.origin[j] + half;
-    h2d(r.off.get(), off, 2, s);
-    h2d(r.prefix.get(), &pf, 1, s);
-    h2d(r.ctr.get(), c, geo.d, s);
+    F3M_LAUNCH(root_level_kernel, 1, 64, 0, s, geo, (int)n, r.off.get(), r.prefix.get(), r.ctr.get(), r.cell.get());
+    check_launch("root_level");
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -451,6 +457,7 @@ __global__ void expand_classify_kernel(long long T, const long long *__restrict_
     long long pos = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (pos >= T) return;
     int nrows = rowexcl[nk];
+    if (pos >= B[nrows]) { cls[pos] = 3; return; }   // T may be an upper bound of the candidate count
     // last row r with B[r] <= pos
     int lo = 0, hi = nrows;
     while (hi - lo > 1) {
@@ -542,6 +549,11 @@ __global__ void split_scatter_kernel(const unsigned char *__restrict__ cls, cons
     }
 }
 
+__global__ void gather3_kernel(const long long *a, const long long *b, const long long *c, long long *out)
+{
+    if (threadIdx.x == 0) { out[0] = *a; out[1] = *b; out[2] = *c; }
+}
+
 __global__ void rowptr_kernel(const int *__restrict__ pairs, long long n, int nbx, int *__restrict__ rowptr)
 {
     int b = blockIdx.x * blockDim.x + threadIdx.x;
@@ -584,9 +596,14 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                px.childstart.get(), W.get(), rowcand.get());
     check_launch("row_cand");
     exclusive_scan_i64(rowcand.get(), nk, B.get(), s);
-    long long T = 0;
-    d2h(&T, B.get() + nk, 1, s);
-    if (T == 0) return;
+    // Candidate storage: every keep pair has at most 4^d child pairs.  When that bound is affordable
+    // the exact count is not fetched first (one host round-trip less per level).
+    const long long p2 = 1ll << (2 * d);
+    long long T = nk * p2;
+    if (T > (1ll << 28)) {
+        d2h(&T, B.get() + nk, 1, s);
+        if (T == 0) return;
+    }
     F3M_REQUIRE(T < (1ll << 40), 22, "candidate list too long (%lld)", T);
     DBuf<int> cand((size_t)T * 2);
     DBuf<unsigned char> cls((size_t)T);
@@ -595,16 +612,16 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                lx.ctr.get(), ly.ctr.get(), d, cp, cand.get(), cls.get());
     check_launch("expand_classify");
     long long nblk = (T + kSplitTile - 1) / kSplitTile;
-    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1);
+    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1), dtot(3);
     F3M_LAUNCH(split_count_kernel, nblk, kSplitBlock, 0, s, cls.get(), T, blockcnt.get(), nblk);
     check_launch("split_count");
     exclusive_scan_i64(blockcnt.get(), nblk, off0.get(), s);
     exclusive_scan_i64(blockcnt.get() + nblk, nblk, off1.get(), s);
     exclusive_scan_i64(blockcnt.get() + 2 * nblk, nblk, off2.get(), s);
+    F3M_LAUNCH(gather3_kernel, 1, 64, 0, s, off0.get() + nblk, off1.get() + nblk, off2.get() + nblk, dtot.get());
+    check_launch("gather3");
     long long tot[3];
-    d2h(&tot[0], off0.get() + nblk, 1, s);
-    d2h(&tot[1], off1.get() + nblk, 1, s);
-    d2h(&tot[2], off2.get() + nblk, 1, s);
+    d2h(tot, dtot.get(), 3, s);
     out.small_.n = tot[0];
     out.far.n = tot[1];
     out.keep.n = tot[2];
@@ -617,7 +634,6 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     if (out.small_.n) build_rowptr(out.small_, lx.nb, s);
     if (out.far.n) build_rowptr(out.far, lx.nb, s);
     if (out.keep.n) build_rowptr(out.keep, lx.nb, s);
-    F3M_HIP(hipStreamSynchronize(s));   // temporaries above return to the pool only after their kernels ran
 }
 
 }  // namespace f3m

@@ -200,8 +200,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     PairList root;
     root.n = 1;
     root.pairs.reset(2);
-    int zero2[2] = {0, 0};
-    h2d(root.pairs.get(), zero2, 2, s);
+    F3M_HIP(hipMemsetAsync(root.pairs.get(), 0, 2 * sizeof(int), s));     // the root pair (0,0)
     const PairList *keep = &root;
     P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
     // loop guard of F3M_src/n_tree.cu:1075 (symmetric) and :1099 (two trees)
