@@ -16,7 +16,10 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK_FP32_TFLOPS = 157.3      # MI355X vector fp32 peak (packed); the near field is VALU work
+PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak
+# HBM bytes moved by one near-field launch of the default workload, from the rocprofv3 FETCH_SIZE and
+# WRITE_SIZE counter runs summarised in profiles/ (None until measured)
+NEAR_TRAFFIC_BYTES = 1.909e9
 
 
 def cpu_baseline(X, b, ls, budget_s=15.0):
@@ -52,6 +55,8 @@ def main():
     ap.add_argument("--subsample", type=int, default=100_000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-accuracy", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run one plain 1 GiB device copy (a kernel of known HBM traffic, to scale rocprof counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on ONE GPU (no sharding, no collectives); --gpus %d is not supported. "
@@ -69,6 +74,14 @@ def main():
     X = (torch.rand(N, d, generator=g) if args.dist == "uniform" else torch.randn(N, d, generator=g)).cuda()
     b = torch.randn(N, 1, generator=g).cuda()
     prm = dict(ls=args.ls, min_points=1000, nr_of_interpolation=args.nodes, small_field_points=1000)
+
+    if args.copy_probe:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
+        src.fill_(1.0)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     engine.set_timing(True)
     for _ in range(args.warmup):
@@ -96,10 +109,13 @@ def main():
     near_per_launch_s = near_t / max(near_n, 1)
     achieved = near_flops * args.steps / max(near_t, 1e-12) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP32_TFLOPS, "traffic": None, "kernel": "near_kernel<%d,1>" % d,
-                "note": "fp32 vector ALU kernel priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
-                        "%.3e kernel evaluations/step x %d flops" % (near_n // max(args.steps, 1), near_per_launch_s * 1e3,
-                                                                     work["near_pairs"], F)}
+                "frac": achieved / PEAK_FP32_TFLOPS, "traffic": NEAR_TRAFFIC_BYTES if (N == 10_000_000 and d == 3) else None,
+                "kernel": "near_h_kernel<%d>" % d,
+                "note": "near field: exponents on the f16 matrix pipe (hi/lo-split operands, fp32 accumulate), exp2 + FMA on "
+                        "the fp32 vector ALU; priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
+                        "%.3e kernel evaluations/step x %d flops; traffic = HBM bytes per launch from rocprofv3 "
+                        "FETCH_SIZE + WRITE_SIZE (profiles/)" % (near_n // max(args.steps, 1), near_per_launch_s * 1e3,
+                                                               work["near_pairs"], F)}
     res = {
         "metric": "KMVM points/sec at N=1e7 3D Gaussian (1 GPU); rel-L2 error vs fp64 exact",
         "value": N / (dt / args.steps), "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
