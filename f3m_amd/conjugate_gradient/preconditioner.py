@@ -1,0 +1,59 @@
+"""The FALKON preconditioner (Rudi, Carratino, Rosasco 2017, Alg. 1), in PyTorch on the GPU.
+
+The reference calls ``falkon.preconditioner.FalkonPreconditioner`` (conjugate_gradient/custom_falkon.py:
+195-199, used through invA/invT/invTt/invAt/apply/apply_t at custom_conjugate_gradient_falkon.py:149-159,
+181-182 and custom_falkon.py:241).  With K_MM the kernel matrix of the M Nystrom centres:
+
+    T = chol(K_MM + eps M I)          upper triangular,  T^T T = K_MM + eps M I
+    A = chol(T T^T / M + lambda I)    upper triangular
+
+``apply(v) = T^-1 A^-1 v`` maps the preconditioned solution beta to the Nystrom coefficients alpha and
+``apply_t(v) = A^-T T^-T v`` is its transpose."""
+import torch
+
+
+class FalkonPreconditioner:
+    def __init__(self, penalty, kernel, opt):
+        self.penalty = float(penalty)
+        self.kernel = kernel
+        self.params = opt
+        self.T = None
+        self.A = None
+
+    def init(self, ny_points, weight_vec=None):
+        if weight_vec is not None:
+            raise NotImplementedError("weighted FALKON is not provided")
+        dt = self.params.pc_dtype
+        M = ny_points.shape[0]
+        K = self.kernel(ny_points, ny_points).to(dt)
+        eps = self.params.pc_epsilon(ny_points.dtype)
+        K.diagonal().add_(eps * M)
+        T = torch.linalg.cholesky(K, upper=True)
+        del K
+        A = (T @ T.T).div_(M)
+        A.diagonal().add_(self.penalty)
+        self.A = torch.linalg.cholesky(A, upper=True)
+        self.T = T
+        return self
+
+    def _solve(self, tri, v, transpose):
+        out = torch.linalg.solve_triangular(tri.T if transpose else tri, v.to(tri.dtype), upper=not transpose)
+        return out.to(v.dtype)
+
+    def invA(self, v):
+        return self._solve(self.A, v, False)
+
+    def invAt(self, v):
+        return self._solve(self.A, v, True)
+
+    def invT(self, v):
+        return self._solve(self.T, v, False)
+
+    def invTt(self, v):
+        return self._solve(self.T, v, True)
+
+    def apply(self, v):
+        return self.invT(self.invA(v))
+
+    def apply_t(self, v):
+        return self.invAt(self.invTt(v))

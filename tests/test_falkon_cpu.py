@@ -1,0 +1,65 @@
+"""Pins the FALKON preconditioner and conjugate-gradient drivers (no engine involved: the K_nm matrix is
+passed densely, the branch the reference takes when K_nm fits in memory,
+conjugate_gradient/custom_falkon.py:229-232) against the closed form of the system they solve."""
+import pytest
+
+torch = pytest.importorskip("torch")
+
+
+class DenseGaussian:
+    def __init__(self, sigma):
+        self.sigma = sigma
+
+    def __call__(self, A, B, opt=None):
+        return torch.exp(-torch.cdist(A.double(), B.double()) ** 2 / (2 * self.sigma ** 2))
+
+
+def test_preconditioned_cg_converges_to_closed_form():
+    from f3m_amd.conjugate_gradient.custom_conjugate_gradient_falkon import FalkonConjugateGradient_custom
+    from f3m_amd.conjugate_gradient.options import FalkonOptions
+    from f3m_amd.conjugate_gradient.preconditioner import FalkonPreconditioner
+    torch.manual_seed(0)
+    n, M, lam, sigma, eps = 3000, 150, 1e-6, 0.5, 1e-5
+    X = 2 * torch.rand(n, 3) - 1
+    y = (torch.sin(3 * X[:, 0]) * torch.cos(2 * X[:, 1]) + X[:, 2] ** 2 + 0.1 * torch.randn(n))[:, None].double()
+    k = DenseGaussian(sigma)
+    C = X[torch.randperm(n)[:M]]
+    opt = FalkonOptions(cg_tolerance=1e-13, pc_epsilon_32=eps)
+    pc = FalkonPreconditioner(lam, k, opt).init(C)
+    Knm = k(X, C)
+    # triangular factors: T^T T = K_mm + eps M I,  A^T A = T T^T / M + lambda I
+    Kmm_j = k(C, C) + eps * M * torch.eye(M, dtype=torch.float64)
+    assert torch.allclose(pc.T.T @ pc.T, Kmm_j, atol=1e-10)
+    assert torch.allclose(pc.A.T @ pc.A, pc.T @ pc.T.T / M + lam * torch.eye(M, dtype=torch.float64), atol=1e-10)
+    v = torch.randn(M, 2, dtype=torch.float64)
+    assert torch.allclose(pc.T @ pc.A @ pc.apply(v), v, atol=1e-6) or torch.allclose(pc.A @ (pc.T @ pc.apply(v)), v, atol=1e-6)
+    assert torch.allclose(pc.apply_t(v), torch.linalg.solve(pc.A.T, torch.linalg.solve(pc.T.T, v)), atol=1e-8)
+    # closed form of the system FALKON solves (the jitter of the preconditioner is part of it)
+    H = Knm.T @ Knm + lam * n * Kmm_j
+    pred_ref = Knm @ torch.linalg.solve(H, Knm.T @ y)
+    errs = []
+    for its in (10, 30, 100):
+        cg = FalkonConjugateGradient_custom(k, pc, opt)
+        beta = cg.solve(Knm, None, y, lam, None, its)
+        pred = Knm @ pc.apply(beta)
+        errs.append(float((pred - pred_ref).norm() / pred_ref.norm()))
+    assert errs[0] > errs[1] > errs[2] and errs[1] < 5e-3 and errs[2] < 1e-7, errs
+
+
+def test_options_defaults_are_documented_values():
+    from f3m_amd.conjugate_gradient import ConjugateGradientOptions, FalkonOptions
+    o = FalkonOptions()
+    assert (o.cg_epsilon(torch.float32), o.cg_tolerance, o.cg_full_gradient_every) == (1e-7, 1e-7, 10)
+    assert isinstance(o.get_conjgrad_options(), ConjugateGradientOptions)
+
+
+def test_conjugate_gradient_solves_spd_system():
+    from f3m_amd.conjugate_gradient import ConjugateGradient, ConjugateGradientOptions
+    g = torch.Generator().manual_seed(0)
+    A = torch.randn(60, 60, generator=g, dtype=torch.float64)
+    A = A @ A.T + 60 * torch.eye(60, dtype=torch.float64)
+    B = torch.randn(60, 3, generator=g, dtype=torch.float64)
+    cg = ConjugateGradient(ConjugateGradientOptions(cg_tolerance=1e-9))
+    X = cg.solve(None, B, lambda v: A @ v, max_iter=200)
+    assert torch.allclose(A @ X, B, atol=1e-7)
+    assert cg.iterations_ <= 70             # exact in about dim steps; stops at the tolerance
