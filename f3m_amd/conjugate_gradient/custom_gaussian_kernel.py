@@ -30,10 +30,10 @@ class custom_GaussianKernel:
         self._plan_key = None
 
     # dense kernel matrix, used for the M x M preconditioner only
-    def __call__(self, X1, X2, opt=None):
+    def __call__(self, X1, X2, opt=None, dtype=torch.float64):
         X1 = X1.to(self.device, torch.float64)
         X2 = X2.to(self.device, torch.float64)
-        out = torch.empty(X1.shape[0], X2.shape[0], dtype=torch.float64, device=self.device)
+        out = torch.empty(X1.shape[0], X2.shape[0], dtype=dtype, device=self.device)
         step = max(1, (1 << 26) // max(1, X2.shape[0]))
         for i in range(0, X1.shape[0], step):
             out[i:i + step] = torch.exp_(torch.cdist(X1[i:i + step], X2).pow_(2).mul_(-0.5 / (self.sigma ** 2)))

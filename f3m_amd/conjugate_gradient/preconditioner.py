@@ -13,6 +13,8 @@ import torch
 
 
 class FalkonPreconditioner:
+    MAX_MATRIX_BYTES = 8 * 2 ** 30
+
     def __init__(self, penalty, kernel, opt):
         self.penalty = float(penalty)
         self.kernel = kernel
@@ -25,14 +27,24 @@ class FalkonPreconditioner:
             raise NotImplementedError("weighted FALKON is not provided")
         dt = self.params.pc_dtype
         M = ny_points.shape[0]
-        K = self.kernel(ny_points, ny_points).to(dt)
+        nbytes = M * M * torch.empty((), dtype=dt).element_size()
+        if nbytes > self.MAX_MATRIX_BYTES:
+            # A run with two 80 GB fp64 factors (M = 1e5) aborted inside the BLAS library on the
+            # development machines and could not be diagnosed; sizes beyond what has been validated
+            # are refused rather than attempted.
+            raise NotImplementedError("preconditioner matrices of %.1f GiB exceed the validated limit of %.0f GiB "
+                                      "(M = %d, %s); use fewer centres or pc_dtype=torch.float32"
+                                      % (nbytes / 2 ** 30, self.MAX_MATRIX_BYTES / 2 ** 30, M, dt))
+        # every factorisation is done in place: at M = 1e5 one fp64 M x M matrix is 80 GB
+        K = self.kernel(ny_points, ny_points, dtype=dt)
         eps = self.params.pc_epsilon(ny_points.dtype)
         K.diagonal().add_(eps * M)
-        T = torch.linalg.cholesky(K, upper=True)
-        del K
-        A = (T @ T.T).div_(M)
+        T = torch.linalg.cholesky(K, upper=True, out=K)
+        A = torch.empty_like(T)
+        torch.mm(T, T.T, out=A)
+        A.div_(M)
         A.diagonal().add_(self.penalty)
-        self.A = torch.linalg.cholesky(A, upper=True)
+        self.A = torch.linalg.cholesky(A, upper=True, out=A)
         self.T = T
         return self
 

@@ -24,7 +24,9 @@ def main():
     ap.add_argument("--maxiter", type=int, default=20)
     ap.add_argument("--nodes", type=int, default=64)
     ap.add_argument("--var-compression", action="store_true")
-    ap.add_argument("--pc-dtype", default="float32", choices=["float32", "float64"])
+    ap.add_argument("--pc-dtype", default="float64", choices=["float32", "float64"])
+    ap.add_argument("--products-only", action="store_true",
+                    help="time only the two engine products of one CG iteration (no preconditioner, no solve)")
     args = ap.parse_args()
     n, m = int(args.n), int(args.m)
     g = torch.Generator().manual_seed(1)
@@ -33,6 +35,23 @@ def main():
     X, Y = X.cuda(), y[:, None].cuda()
     opt = FalkonOptions(pc_dtype=getattr(torch, args.pc_dtype))
     kernel = custom_GaussianKernel(args.ls, opt=opt, var_compression=args.var_compression, interpolation_nr=args.nodes)
+    if args.products_only:
+        C = X[torch.randperm(n, generator=g)[:m].cuda()].contiguous()
+        v = torch.randn(m, 1, generator=g).cuda()
+        torch.cuda.synchronize()
+        t0 = time.time()
+        kernel.dmmv(X, C, v, None)             # builds both plans, then K_nm v and K_nm^T (.)
+        torch.cuda.synchronize()
+        t_first = time.time() - t0
+        times = []
+        for _ in range(5):
+            t0 = time.time()
+            out = kernel.dmmv(X, C, v, None)
+            torch.cuda.synchronize()
+            times.append(time.time() - t0)
+        print(json.dumps({"n": n, "m": m, "ls": args.ls, "first_dmmv_with_plans_s": t_first,
+                          "dmmv_s": [round(t, 4) for t in times], "finite": bool(torch.isfinite(out).all())}))
+        return
     model = custom_Falkon(kernel, args.penalty, m, maxiter=args.maxiter, seed=1, options=opt)
     torch.cuda.synchronize()
     t0 = time.time()

@@ -10,8 +10,8 @@ class DenseGaussian:
     def __init__(self, sigma):
         self.sigma = sigma
 
-    def __call__(self, A, B, opt=None):
-        return torch.exp(-torch.cdist(A.double(), B.double()) ** 2 / (2 * self.sigma ** 2))
+    def __call__(self, A, B, opt=None, dtype=torch.float64):
+        return torch.exp(-torch.cdist(A.double(), B.double()) ** 2 / (2 * self.sigma ** 2)).to(dtype)
 
 
 def test_preconditioned_cg_converges_to_closed_form():
