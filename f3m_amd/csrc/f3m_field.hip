@@ -289,19 +289,16 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 // Valid while |x'|, |y'| stay small enough for the split (the host checks the box size against the
 // lengthscale and otherwise launches near_kernel).
 
-constexpr int kNearTPW = 2;                         // target tiles (of 32) per wavefront
-constexpr int kNearMfmaBlock = 256;                 // lanes per workgroup
-constexpr int kNearMfmaTargets = (kNearMfmaBlock / kWave) * kNearTPW * 32;
 
 // inner slot s of the matrix product: component s/3; s%3 = 0: hi.hi, 1: (source hi).(target lo), 2: (source lo).(target hi)
-template <int D>
+template <int C>
 __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, int hh, bool source)
 {
     h8 v;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const int slot = 16 * n + 8 * hh + e;
-        if (slot < 3 * (D + 1)) {
+        if (slot < 3 * C) {
             const int c = slot / 3, tau = slot % 3;
             v[e] = source ? (tau == 2 ? lo[c] : hi[c]) : (tau == 1 ? lo[c] : hi[c]);
         } else {
@@ -311,137 +308,152 @@ __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, in
     return v;
 }
 
+// Source operands, once per tree level: point i of box b, shifted to the centre of b and scaled,
+// as the rows (2y', -|y'|^2) of the matrix product in split-f16 form.  Layout: ops[(n*2 + h)*stride + i]
+// = the eight inner slots of half-wave h of instruction n; stride = npoints + 32 (the tail is zero so
+// that a wavefront may read one padded tile past the end).
 template <int D>
-__global__ void __launch_bounds__(kNearMfmaBlock, 2) near_h_kernel(
-    const float *__restrict__ xs, long long N, const float *__restrict__ ys, long long M, const float *__restrict__ bs,
-    float *__restrict__ outs, const int *__restrict__ offx, const int *__restrict__ offy, const float *__restrict__ ctrx,
-    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc)
+__global__ void near_operands_kernel(const float *__restrict__ ys, long long M, const int *__restrict__ off, int nb,
+                                     const float *__restrict__ ctr, float sc, long long stride, h8 *__restrict__ ops)
 {
-    constexpr int C = D + 1;
-    constexpr int NS = (3 * C + 15) / 16;           // matrix instructions per tile
-    __shared__ h8 aop[NS][2][kNearCap];
-    __shared__ __align__(16) float sb[kNearCap];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, col = lane & 31;
-    if ((int)blockIdx.x >= tileoff[nbx]) return;    // launched with an upper bound of the tile count
-    const int bx = find_box(tileoff, nbx, blockIdx.x);
-    const int tile = blockIdx.x - tileoff[bx];
-    const int x0 = offx[bx] + tile * kNearMfmaTargets, x1 = offx[bx + 1];
-    float cx[D];
-#pragma unroll
-    for (int k = 0; k < D; k++) cx[k] = ctrx[(long long)bx * D + k];
-    h8 bop[kNearTPW][NS];
-    f32x16 cinit[kNearTPW];
-    float acc[kNearTPW];
-    bool live[kNearTPW];
-#pragma unroll
-    for (int q = 0; q < kNearTPW; q++) {
-        const int t0 = x0 + (wave * kNearTPW + q) * 32;
-        const int i = t0 + col;
-        live[q] = t0 < x1;
-        half_t hi[C], lo[C];
-        float nx2 = 0.f;
+    constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
+    constexpr int NS = (3 * C + 15) / 16;
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= stride) return;
+    half_t hi[C], lo[C];
+    if (i < M) {
+        const int box = find_box(off, nb, (int)i);
+        float ny2 = 0.f;
 #pragma unroll
         for (int k = 0; k < C; k++) {
-            float v = 1.f;
+            float v;
             if (k < D) {
-                v = (i < x1) ? sc * (xs[(long long)k * N + i] - cx[k]) : 0.f;
-                nx2 -= v * v;
+                float y = sc * (ys[(long long)k * M + i] - ctr[(long long)box * D + k]);
+                ny2 -= y * y;
+                v = 2.f * y;
+            } else if (k == D) {
+                v = ny2;
+            } else {
+                v = 1.f;
             }
             hi[k] = to_half(v);
             lo[k] = to_half(v - half_to_float(hi[k]));
         }
+    } else {
 #pragma unroll
-        for (int n = 0; n < NS; n++) {
-            h8 v0 = split_operand<D>(hi, lo, n, 0, false), v1 = split_operand<D>(hi, lo, n, 1, false);
-            bop[q][n] = half ? v1 : v0;
-        }
-#pragma unroll
-        for (int r = 0; r < 16; r++) cinit[q][r] = nx2;
-        acc[q] = 0.f;
+        for (int k = 0; k < C; k++) { hi[k] = to_half(0.f); lo[k] = to_half(0.f); }
     }
+#pragma unroll
+    for (int n = 0; n < NS; n++) {
+        ops[(long long)(n * 2 + 0) * stride + i] = split_operand<C>(hi, lo, n, 0, true);
+        ops[(long long)(n * 2 + 1) * stride + i] = split_operand<C>(hi, lo, n, 1, true);
+    }
+}
+
+// Near field, matrix-pipe form.  One wavefront per TPW*32 targets of an x box (TPW tiles of 32; lanes
+// l and l+32 hold the same target and different source rows).  For every listed y box the targets are
+// re-expressed relative to the centre of that y box (x'' = sc (x - c_y)) and split into f16 pairs; the
+// per-target constant -|x''|^2 rides in two spare inner slots (against a source-side 1), so the
+// accumulator starts from zero.  The source operands come ready-made from near_operands_kernel and
+// are streamed from global memory / L2 in 32-source tiles, together with their weights.  No LDS and
+// no barriers: wavefronts are independent.  Rows past the end of a box are neutralised by a zero
+// weight (the exponent of any two vectors is -|x''-y'|^2 <= 0, so exp2 stays finite).
+constexpr int kNearWavesPerBlock = 2;
+struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floats at any 4-byte boundary
+
+template <int D, int TPW>
+__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
+    const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
+    float *__restrict__ outs, const int *__restrict__ offx, const int *__restrict__ offy, const float *__restrict__ ctry,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc)
+{
+    constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
+    constexpr int NS = (3 * C + 15) / 16;
+    const int lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
+    const int wid = blockIdx.x * kNearWavesPerBlock + (threadIdx.x >> 6);      // work item: TPW*32 targets of one box
+    if (wid >= tileoff[nbx]) return;
+    const int bx = find_box(tileoff, nbx, wid);
+    const int x0 = offx[bx] + (wid - tileoff[bx]) * (TPW * 32), x1 = offx[bx + 1];
+    int nlive = (x1 - x0 + 31) / 32;                 // tiles with targets (uniform per wavefront)
+    if (nlive > TPW) nlive = TPW;
+    float xr[TPW][D];
+#pragma unroll
+    for (int q = 0; q < TPW; q++) {
+        const int i = x0 + q * 32 + col;
+#pragma unroll
+        for (int k = 0; k < D; k++) xr[q][k] = (i < x1) ? xs[(long long)k * N + i] : 0.f;
+    }
+    float acc[TPW];
+#pragma unroll
+    for (int q = 0; q < TPW; q++) acc[q] = 0.f;
     const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
     for (int m = m0; m < m1; m++) {
         const int by = pairs[2 * (long long)m + 1];
         const int s0 = offy[by], s1 = offy[by + 1];
-        for (int base = s0; base < s1; base += kNearCap) {
-            const int cnt = (s1 - base) < kNearCap ? (s1 - base) : kNearCap;
-            const int cntp = (cnt + 31) & ~31;
-            __syncthreads();
-            for (int jj = tid; jj < cntp; jj += kNearMfmaBlock) {
-                half_t hi[C], lo[C];
-                float ny2 = 0.f;
+        float cy[D];
 #pragma unroll
-                for (int k = 0; k < C; k++) {
-                    float v;
-                    if (k < D) {
-                        float y = (jj < cnt) ? sc * (ys[(long long)k * M + base + jj] - cx[k]) : 0.f;
-                        ny2 -= y * y;
-                        v = 2.f * y;
-                    } else {
-                        v = ny2;
-                    }
-                    hi[k] = to_half(v);
-                    lo[k] = to_half(v - half_to_float(hi[k]));
-                }
+        for (int k = 0; k < D; k++) cy[k] = ctry[(long long)by * D + k];
+        // target operands relative to the centre of this y box
+        h8 bop[TPW][NS];
 #pragma unroll
-                for (int n = 0; n < NS; n++) {
-                    aop[n][0][jj] = split_operand<D>(hi, lo, n, 0, true);
-                    aop[n][1][jj] = split_operand<D>(hi, lo, n, 1, true);
+        for (int q = 0; q < TPW; q++) {
+            const bool ok = x0 + q * 32 + col < x1;
+            half_t hi[C], lo[C];
+            float nx2 = 0.f;
+#pragma unroll
+            for (int k = 0; k < C; k++) {
+                float v = 1.f;
+                if (k < D) {
+                    v = ok ? sc * (xr[q][k] - cy[k]) : 0.f;
+                    nx2 -= v * v;
+                } else if (k == D + 1) {
+                    v = nx2;
                 }
-                sb[jj] = (jj < cnt) ? bs[base + jj] : 0.f;
+                hi[k] = to_half(v);
+                lo[k] = to_half(v - half_to_float(hi[k]));
             }
-            __syncthreads();
-            if (!live[0]) continue;                 // uniform per wavefront
-            for (int j0 = 0; j0 < cntp; j0 += 32) {
-                h8 a[NS];
 #pragma unroll
-                for (int n = 0; n < NS; n++) a[n] = aop[n][half][j0 + col];
-                float4 bq[4];
+            for (int n = 0; n < NS; n++) {
+                h8 v0 = split_operand<C>(hi, lo, n, 0, false), v1 = split_operand<C>(hi, lo, n, 1, false);
+                bop[q][n] = half ? v1 : v0;
+            }
+        }
+        for (int j0 = s0; j0 < s1; j0 += 32) {
+            h8 a[NS];
 #pragma unroll
-                for (int g = 0; g < 4; g++) bq[g] = *reinterpret_cast<const float4 *>(&sb[j0 + 8 * g + 4 * half]);
-                f32x16 t0 = cinit[0];
+            for (int n = 0; n < NS; n++) a[n] = ops[(long long)(n * 2 + half) * stride + j0 + col];
+            // weights of the 16 source rows this lane sees: rows 8g + 4 half + e of the tile (bs is
+            // padded by one tile, so the loads stay in bounds; rows past the box get weight zero)
+            float bq[16];
 #pragma unroll
-                for (int n = 0; n < NS; n++) t0 = mfma_32x32x16_f16(a[n], bop[0][n], t0);
-                if (live[1]) {                      // uniform per wavefront
-                    f32x16 t1 = cinit[1];
+            for (int g = 0; g < 4; g++) {
+                const float4u f = *reinterpret_cast<const float4u *>(bs + j0 + 8 * g + 4 * half);
+                bq[4 * g + 0] = f.x; bq[4 * g + 1] = f.y; bq[4 * g + 2] = f.z; bq[4 * g + 3] = f.w;
+            }
+            if (j0 + 32 > s1) {
 #pragma unroll
-                    for (int n = 0; n < NS; n++) t1 = mfma_32x32x16_f16(a[n], bop[1][n], t1);
-                    float s0a = acc[0], s1a = acc[1];
+                for (int r = 0; r < 16; r++) bq[r] = (j0 + 8 * (r / 4) + 4 * half + (r % 4) < s1) ? bq[r] : 0.f;
+            }
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        s0a = fmaf(fast_exp2(t0[4 * g + 0]), bq[g].x, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 1]), bq[g].y, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 2]), bq[g].z, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 3]), bq[g].w, s0a);
-                    }
+            for (int q = 0; q < TPW; q++) {
+                if (q < nlive) {                     // uniform per wavefront
+                    f32x16 t;
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        s1a = fmaf(fast_exp2(t1[4 * g + 0]), bq[g].x, s1a);
-                        s1a = fmaf(fast_exp2(t1[4 * g + 1]), bq[g].y, s1a);
-                        s1a = fmaf(fast_exp2(t1[4 * g + 2]), bq[g].z, s1a);
-                        s1a = fmaf(fast_exp2(t1[4 * g + 3]), bq[g].w, s1a);
-                    }
-                    acc[0] = s0a;
-                    acc[1] = s1a;
-                } else {
-                    float s0a = acc[0];
+                    for (int r = 0; r < 16; r++) t[r] = 0.f;
 #pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        s0a = fmaf(fast_exp2(t0[4 * g + 0]), bq[g].x, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 1]), bq[g].y, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 2]), bq[g].z, s0a);
-                        s0a = fmaf(fast_exp2(t0[4 * g + 3]), bq[g].w, s0a);
-                    }
-                    acc[0] = s0a;
+                    for (int n = 0; n < NS; n++) t = mfma_32x32x16_f16(a[n], bop[q][n], t);
+                    float sum = acc[q];
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sum = fmaf(fast_exp2(t[r]), bq[r], sum);
+                    acc[q] = sum;
                 }
             }
         }
     }
 #pragma unroll
-    for (int q = 0; q < kNearTPW; q++) {
-        if (!live[q]) continue;
+    for (int q = 0; q < TPW; q++) {
         float total = acc[q] + wave_shfl_xor_f(acc[q], 32);
-        const int i = x0 + (wave * kNearTPW + q) * 32 + col;
+        const int i = x0 + q * 32 + col;
         if (half == 0 && i < x1) outs[i] += total;
     }
 }
@@ -450,12 +462,13 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                 const float *bs, float *outs, float lcs, hipStream_t s)
 {
     if (list.n == 0) return;
-    // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to
-    // ~2^-22 |y'|^2; it is used while the farthest listed source stays within |y'| <= 20 of the x-box
-    // centre in scaled units (box edge at most ~2 lengthscales), otherwise the all-vector kernel.
+    // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to about
+    // 2^-22 times the largest term, |x''|^2 <= 30 d (sc edge)^2 (listed targets lie within 5.5 edges per
+    // dimension of the source box centre); it is used while that bound stays below 1e-4 (box edge up to
+    // ~2 lengthscales in 3-D), otherwise the all-vector kernel.
     // F3M_NEAR=valu|mfma overrides the choice.
     const float sc_edge = sqrtf(lcs * kLog2e) * lx.edge;
-    bool use_mfma = sc_edge * 5.5f * sqrtf((float)d) <= 20.f;
+    bool use_mfma = 30.f * (float)d * sc_edge * sc_edge <= 400.f;
     if (const char *env = getenv("F3M_NEAR")) use_mfma = !strcmp(env, "mfma") ? true : (!strcmp(env, "valu") ? false : use_mfma);
     constexpr int T = 1;
     // all-vector kernel: whole boxes per workgroup where possible (multiple of the wave size, <= 512 lanes)
@@ -465,15 +478,35 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     DBuf<int> flag((size_t)lx.nb), tileoff;
     F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
     check_launch("mark_rows");
-    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? kNearMfmaTargets : bd * T, tileoff, s);
+    constexpr int tpw = 4;      // target tiles of 32 per wavefront (2: 10.2 ms, 4: 9.2 ms, 8: 9.4 ms at N=1e7, d=3)
+    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? tpw * 32 : bd * T, tileoff, s);
     float sc = sqrtf(lcs * kLog2e);
-    timer_begin(kNear, s);
     if (use_mfma) {
+        const int C = d + 2, NS = (3 * C + 15) / 16;
+        const long long stride = ty.n + 32;
+        if (ly.nearops.size() == 0 || ly.nearops_sc != sc) {
+            ly.nearops.reset((size_t)NS * 2 * stride * 16);
+            ly.nearops_sc = sc;
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_h_kernel<DD>), ntiles, kNearMfmaBlock, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs,  \
-                   outs, lx.off.get(), ly.off.get(), lx.ctr.get(), list.pairs.get(), list.rowptr.get(),               \
-                   tileoff.get(), lx.nb, sc);                                                                         \
+        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, 256), 256, 0, s, ty.pts.get(), ty.n, ly.off.get(), ly.nb, \
+                   ly.ctr.get(), sc, stride, reinterpret_cast<h8 *>(ly.nearops.get()));                               \
+        break;
+            switch (d) {
+                F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+                F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+            default: throw Error(2, "dimension must be 1..10");
+            }
+#undef F3M_CASE
+            check_launch("near_operands");
+        }
+        timer_begin(kNear, s);
+#define F3M_CASE(DD)                                                                                                  \
+    case DD:                                                                                                          \
+        F3M_LAUNCH((near_g_kernel<DD, tpw>), cdiv(ntiles, kNearWavesPerBlock), kNearWavesPerBlock * 64, 0, s,         \
+                   tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, outs,              \
+                   lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
+                   lx.nb, sc);                                                                                        \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -482,6 +515,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         }
 #undef F3M_CASE
     } else {
+        timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
         F3M_LAUNCH((near_kernel<DD, T>), ntiles, bd, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs, outs,          \

@@ -261,7 +261,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         F3M_HIP(hipStreamSynchronize(s));
         return;
     }
-    DBuf<float> bs((size_t)P->M), outs((size_t)P->N);
+    DBuf<float> bs((size_t)P->M + 32), outs((size_t)P->N);   // bs padded: near_g_kernel reads whole tiles
     const int depth = (int)P->levels.size();
     for (int col = 0; col < c; col++) {
         {
@@ -444,7 +444,7 @@ int f3m_plan_far_level(f3m_plan *plan, int level, const float *b, int c, float *
         check_level(plan, level);
         hipStream_t s = (hipStream_t)stream;
         check_device_ptr(b, "b"); check_device_ptr(out, "out");
-        DBuf<float> bs((size_t)plan->M), outs((size_t)plan->N);
+        DBuf<float> bs((size_t)plan->M + 32), outs((size_t)plan->N);
         PlanLevel &L = plan->levels[level - 1];
         int P = L.far.n ? plan->nodeset(L.num_nodes, s).P : 0;
         for (int col = 0; col < c; col++) {
@@ -466,7 +466,7 @@ int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, in
         F3M_REQUIRE(which == F3M_LIST_SMALL || which == F3M_LIST_KEEP, 13, "which must be F3M_LIST_SMALL or F3M_LIST_KEEP");
         hipStream_t s = (hipStream_t)stream;
         check_device_ptr(b, "b"); check_device_ptr(out, "out");
-        DBuf<float> bs((size_t)plan->M), outs((size_t)plan->N);
+        DBuf<float> bs((size_t)plan->M + 32), outs((size_t)plan->N);
         PlanLevel &L = plan->levels[level - 1];
         for (int col = 0; col < c; col++) {
             gather_column(b, plan->ty->perm.get(), plan->M, c, col, bs.get(), s);

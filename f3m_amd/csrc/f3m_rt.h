@@ -180,26 +180,6 @@ struct f32x16 {
     float &operator[](int i) { return v[i]; }
     const float &operator[](int i) const { return v[i]; }
 };
-// D = A(32x2) B(2x32) + C on one wavefront: lane l supplies A[l%32][l/32] and B[l/32][l%32] and
-// holds D[8(r/4) + 4(l/32) + r%4][l%32] in element r
-__device__ inline f32x16 mfma_32x32x2(float a, float b, f32x16 c)
-{
-    uint32_t A[64], B[64];
-    uint32_t ua, ub;
-    memcpy(&ua, &a, 4);
-    memcpy(&ub, &b, 4);
-    emu::gather_bits(ua, A);
-    emu::gather_bits(ub, B);
-    const unsigned l = lane_id(), j = l & 31, h = l >> 5;
-    for (int r = 0; r < 16; r++) {
-        unsigned i = 8 * (r / 4) + 4 * h + (r % 4);
-        float a0, a1, b0, b1;
-        memcpy(&a0, &A[i], 4); memcpy(&a1, &A[i + 32], 4);
-        memcpy(&b0, &B[j], 4); memcpy(&b1, &B[j + 32], 4);
-        c.v[r] = fmaf(a1, b1, fmaf(a0, b0, c.v[r]));
-    }
-    return c;
-}
 // IEEE binary16 stand-ins for the CPU build (round to nearest even, subnormals kept)
 struct half_t { uint16_t bits; };
 __device__ inline half_t to_half(float f)
@@ -250,8 +230,8 @@ struct h8 {
     const half_t &operator[](int i) const { return v[i]; }
 };
 // D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation: lane l supplies row l%32 of A and
-// column l%32 of B for the eight inner indices of its half-wave; the output layout is that of
-// mfma_32x32x2
+// column l%32 of B for the eight inner indices of its half-wave and holds D[8(r/4) + 4(l/32) + r%4][l%32]
+// in element r
 __device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
 {
     uint32_t A[4][64], B[4][64];
@@ -280,19 +260,13 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 __device__ __forceinline__ int wave_shfl_i(int v, int src) { return __shfl(v, src, 64); }
 __device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
-// D = A(32x2) B(2x32) + C on the matrix pipe (v_mfma_f32_32x32x2_f32): lane l supplies A[l%32][l/32]
-// and B[l/32][l%32] and holds D[8(r/4) + 4(l/32) + r%4][l%32] in element r
-__device__ __forceinline__ f32x16 mfma_32x32x2(float a, float b, f32x16 c)
-{
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
-}
 typedef _Float16 half_t;
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
 __device__ __forceinline__ half_t to_half(float f) { return (_Float16)f; }
 __device__ __forceinline__ float half_to_float(half_t h) { return (float)h; }
 // D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation (v_mfma_f32_32x32x16_f16): lane l
-// supplies row l%32 of A and column l%32 of B for the eight inner indices of its half-wave; the
-// output layout is that of mfma_32x32x2
+// supplies row l%32 of A and column l%32 of B for the eight inner indices of its half-wave and holds
+// D[8(r/4) + 4(l/32) + r%4][l%32] in element r
 __device__ __forceinline__ f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
 {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
