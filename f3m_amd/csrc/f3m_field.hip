@@ -645,18 +645,21 @@ void set_node_offsets(NodeSet &ns, float edge, hipStream_t s)
 __device__ inline void basis_1d(float t, const float *__restrict__ nt, const float *__restrict__ nw, int n,
                                 float *__restrict__ out, float scale)
 {
+    // out[a] holds w_a/(t-t_a) until the sum is known; reciprocals by v_rcp_f32 (1 ulp)
     float sum = 0.f;
     int hit = -1;
     for (int a = 0; a < n; a++) {
         float diff = t - nt[a];
-        if (diff == 0.f) { hit = a; break; }
-        sum += nw[a] / diff;
+        if (diff == 0.f) hit = a;
+        float q = nw[a] * fast_rcp(diff);
+        out[a] = q;
+        sum += q;
     }
     if (hit >= 0) {
         for (int a = 0; a < n; a++) out[a] = (a == hit) ? scale : 0.f;
     } else {
-        float inv = scale / sum;
-        for (int a = 0; a < n; a++) out[a] = (nw[a] / (t - nt[a])) * inv;
+        float inv = scale * fast_rcp(sum);
+        for (int a = 0; a < n; a++) out[a] *= inv;
     }
 }
 

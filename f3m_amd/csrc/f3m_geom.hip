@@ -201,12 +201,20 @@ __global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__rest
     __syncthreads();
     const long long tile = (long long)blockIdx.x * kSortTile;
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    // the whole tile goes to registers first, so that the loads of all rounds are in flight together
+    uint32_t key[kSortRounds];
+    int val[kSortRounds];
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        long long i = tile + r * kWave + lane;
+        key[r] = (i < n) ? keys_in[i] : 0u;
+        val[r] = (i < n) ? idx_in[i] : 0;
+    }
+#pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
         long long i = tile + r * kWave + lane;
         bool valid = i < n;
-        uint32_t key = valid ? keys_in[i] : 0u;
-        int val = valid ? idx_in[i] : 0;
-        uint32_t digit = (key >> shift) & 255u;
+        uint32_t digit = (key[r] >> shift) & 255u;
         unsigned long long same = wave_ballot(valid);
 #pragma unroll
         for (int bit = 0; bit < 8; bit++) {
@@ -220,8 +228,8 @@ __global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__rest
         if (valid && rank == 0) run[digit] = start + __popcll(same);
         __syncthreads();
         if (valid) {
-            keys_out[start + rank] = key;
-            idx_out[start + rank] = val;
+            keys_out[start + rank] = key[r];
+            idx_out[start + rank] = val[r];
         }
     }
 }

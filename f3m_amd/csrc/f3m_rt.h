@@ -166,6 +166,7 @@ inline void check_launch(const char *what)
 __device__ inline unsigned long long wave_ballot(bool p) { return emu::ballot(p); }
 __device__ inline unsigned lane_id() { return emu::S().cur->tid % 64; }
 __device__ inline float fast_exp2(float x) { return exp2f(x); }
+__device__ inline float fast_rcp(float x) { return 1.0f / x; }
 __device__ inline int wave_shfl_i(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }
 __device__ inline float wave_shfl_xor_f(float v, int mask)
 {
@@ -257,6 +258,7 @@ __device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
 __device__ __forceinline__ unsigned long long wave_ballot(bool p) { return __ballot(p); }
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }   // v_rcp_f32, 1 ulp
 __device__ __forceinline__ int wave_shfl_i(int v, int src) { return __shfl(v, src, 64); }
 __device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
