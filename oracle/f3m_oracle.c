@@ -22,8 +22,8 @@
  *   M2L ............................................ pinned (dense exp(-lcs*cdist^2) of shifted nodes)
  *   end to end ..................................... pinned (reduces to the dense product when no
  *                                                    pair is far; rel-L2 vs fp64 exact; linearity)
- *   var_compression classification ................. parity unpinned beyond the brute-force
- *                                                    restatement of the same predicates
+ *   var_compression classification ................. pinned (independent numpy restatement of the
+ *                                                    predicates, brute force over all box pairs)
  */
 #include <math.h>
 #include <stdint.h>

@@ -58,3 +58,40 @@ def box_of_point(level, which="x"):
     box = np.empty(perm.shape[0], np.int64)
     box[perm] = np.repeat(np.arange(off.shape[0] - 1), np.diff(off))
     return box
+
+
+def classify_var_comp_np(cx, cy, nx, ny, edge, nr_interp, small_limit, d, lcs, eff_var_limit):
+    """var_compression=True predicates (F3M_src/n_tree.cu:727-743, F3M_src/1_d_conv.cu:983-1026), fp32.
+    0 small, 1 far, 2 keep, 3 dropped."""
+    edge, lcs, eff = f32(edge), f32(lcs), f32(eff_var_limit)
+    sq = f32(f32(edge * edge) * lcs)
+    do_init = sq <= 5
+    quarter = f32(f32(f32(d) * sq) / f32(4))
+    en_pair = quarter <= eff
+    en_all = quarter <= f32(eff / f32(2))
+    crit = np.sqrt(f32(f32(eff * f32(2)) / f32(f32(d) * lcs))).astype(f32)
+    size = nx.astype(np.int64) + ny.astype(np.int64)
+    diff = (cy.astype(f32) - cx.astype(f32)).astype(f32)
+    acc = np.zeros(diff.shape[0], f32)
+    for j in range(diff.shape[1]):
+        acc = (acc + (diff[:, j] * diff[:, j]).astype(f32)).astype(f32)
+    dist = np.sqrt(acc).astype(f32)
+    out = np.full(diff.shape[0], -1, np.int64)
+    todo = np.ones(diff.shape[0], bool)
+
+    def settle(mask, code):
+        nonlocal todo
+        m = todo & mask
+        out[m] = code
+        todo = todo & ~m
+
+    if do_init:
+        settle(size < 2 * nr_interp, 0)
+    settle(dist >= f32(edge * f32(2)), 1 if do_init else 3)
+    if en_pair:
+        settle(((dist * dist).astype(f32) * lcs).astype(f32).astype(np.float64) <= 1e-2, 1)
+    if en_all:
+        settle(dist <= crit, 1)
+    settle(size < 2 * small_limit, 0)
+    settle(np.ones_like(todo), 2)
+    return out

@@ -47,10 +47,14 @@ def clouds(name, rng):
     if name == "lattice_faces_dups":
         g = (np.stack(np.meshgrid(*[np.arange(33)] * 3, indexing="ij"), -1).reshape(-1, 3) / 32.0).astype(f32)
         return np.concatenate([g, g[::-1], g[::2]]), None, dict(ls=0.3, min_points=200, small_field_points=100)
+    if name == "uniform3_varcomp":   # the reference's FALKON experiments run with var_compression=True
+        return rng.random((80000, 3), dtype=f32), None, dict(ls=3.0, var_compression=True, eff_var_limit=0.3,
+                                                              min_points=500, small_field_points=300)
     raise KeyError(name)
 
 
-NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "uniform2", "uniform1", "lattice_faces_dups"]
+NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "uniform2", "uniform1", "lattice_faces_dups",
+         "uniform3_varcomp"]
 
 
 @pytest.mark.parametrize("name", NAMES)
@@ -82,7 +86,7 @@ def test_exact_kernels(eng, oracle, d):
     assert rel_l2(eng.exact_grad_f32(dev(X), dev(Y), dev(b), ls).cpu().numpy(), oracle.exact_grad_f32(X, Y, b, ls)) < 1e-5
 
 
-@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5"])
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform3_varcomp"])
 def test_stages_against_oracle(eng, oracle, name):
     print("case stages", name, flush=True)
     rng = np.random.default_rng(7)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 from hypothesis import given, settings, strategies as st
 
-from helpers import box_ids_by_morton_rank, box_of_point, cell_coords, classify_np
+from helpers import box_ids_by_morton_rank, box_of_point, cell_coords, classify_np, classify_var_comp_np
 
 f32 = np.float32
 
@@ -148,3 +148,38 @@ def test_tree_hypothesis_random_clouds(oracle, seed, d, n):
         L = P.level(k)
         ref_box, _ = box_ids_by_morton_rank(X, xmin, edge0, k + 1)
         assert np.array_equal(box_of_point(L, "x"), ref_box)
+
+
+@pytest.mark.parametrize("ls,eff", [(2.0, 0.3), (0.7, 0.3), (0.25, 0.15), (8.0, 0.5)])
+def test_var_compression_lists_bruteforce(oracle, ls, eff):
+    """The var_compression=True classification against an independent numpy restatement of its
+    predicates, over all pairs of non-empty boxes whose parents were kept."""
+    rng = np.random.default_rng(17)
+    X = rng.random((3000, 3), dtype=f32)
+    prm = dict(ls=ls, min_points=60, nr_of_interpolation=27, small_field_points=40, var_compression=True,
+               eff_var_limit=eff)
+    P = oracle.Plan(X, None, **prm)
+    keep_prev = {(0, 0)}
+    parent = None
+    seen_shortcut = False
+    for k in range(P.nlevels):
+        L = P.level(k)
+        box = box_of_point(L, "x")
+        nb = len(L["cntx"])
+        par = np.zeros(nb, int)
+        if k > 0:
+            par[box] = parent
+        BX, BY = np.meshgrid(np.arange(nb), np.arange(nb), indexing="ij")
+        BX, BY = BX.ravel(), BY.ravel()
+        alive = np.fromiter(((int(a), int(b)) in keep_prev for a, b in zip(par[BX], par[BY])), bool, len(BX))
+        BX, BY = BX[alive], BY[alive]
+        cls = classify_var_comp_np(L["cx"][BX], L["cx"][BY], L["cntx"][BX], L["cntx"][BY], L["edge"], 27, 40, 3,
+                                   P.lcs, eff)
+        for name_, code in (("small", 0), ("far", 1), ("keep", 2)):
+            ref = np.stack([BX[cls == code], BY[cls == code]], 1)
+            assert np.array_equal(L[name_], ref), (k, name_)
+        plain = classify_np(L["cx"][BX], L["cx"][BY], L["cntx"][BX], L["cntx"][BY], L["edge"], 27, 40)
+        seen_shortcut |= bool((plain != cls).any())
+        keep_prev = set(map(tuple, L["keep"].tolist()))
+        parent = box
+    assert seen_shortcut or ls < 1.0        # smooth kernels must trigger the extra far-field shortcuts
