@@ -365,12 +365,23 @@ template <int D, int TPW>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     float *__restrict__ outs, const int *__restrict__ offx, const int *__restrict__ offy, const float *__restrict__ ctry,
-    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc)
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
+    int stripe)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
     const int lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
-    const int wid = blockIdx.x * kNearWavesPerBlock + (threadIdx.x >> 6);      // work item: TPW*32 targets of one box
+    // Workgroups are handed to the 8 XCDs round-robin.  Work items are in Morton order of their x box
+    // and neighbouring boxes share their source boxes, so the work items are cut into stripes of
+    // `stripe` consecutive workgroups and each stripe runs on one XCD: its L2 then serves the re-reads
+    // of the sources.  (gridDim.x is a multiple of 8*stripe.)
+    int vblock;
+    if (stripe <= 0) vblock = blockIdx.x;
+    else {
+        const int r = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+        vblock = (r / stripe) * (8 * stripe) + xcd * stripe + (r % stripe);
+    }
+    const int wid = vblock * kNearWavesPerBlock + (threadIdx.x >> 6);          // work item: TPW*32 targets of one box
     if (wid >= tileoff[nbx]) return;
     const int bx = find_box(tileoff, nbx, wid);
     const int x0 = offx[bx] + (wid - tileoff[bx]) * (TPW * 32), x1 = offx[bx + 1];
@@ -500,13 +511,17 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #undef F3M_CASE
             check_launch("near_operands");
         }
+        int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
+        if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
+        int nblk = (int)cdiv(ntiles, kNearWavesPerBlock);
+        int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_g_kernel<DD, tpw>), cdiv(ntiles, kNearWavesPerBlock), kNearWavesPerBlock * 64, 0, s,         \
+        F3M_LAUNCH((near_g_kernel<DD, tpw>), ngrid, kNearWavesPerBlock * 64, 0, s,                                    \
                    tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, outs,              \
                    lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
-                   lx.nb, sc);                                                                                        \
+                   lx.nb, sc, stripe);                                                                                \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
