@@ -865,6 +865,120 @@ __global__ void __launch_bounds__(1024) m2l_sep_kernel(const float *__restrict__
     if (live) loc[(long long)bx * P + tid] = acc;
 }
 
+// Separable M2L for the 4 x 4 x 4 node grid (64 nodes, the default), one wavefront per x box, lane =
+// node (a0 + 4 a1 + 16 a2).  The far boxes of an x box differ from it by cell offsets (o0, o1, o2).
+// Per far box only the first factor is applied (four multiply-adds on values broadcast inside groups of
+// four lanes) and the result is added to the LDS slot of its (o1, o2); the second factor is then applied
+// once per (o1, o2) slot and the third once per o2, instead of once per far box.  SPAN = number of
+// distinct offsets per dimension that can occur: 7 with one tree (-3..3), 10 with two trees.
+template <int SPAN>
+__global__ void __launch_bounds__(64) m2l_q64_kernel(const float *__restrict__ tables, SepMeta sm, int lo1, int lo2,
+                                                      const int *__restrict__ cellx, const int *__restrict__ celly,
+                                                      const int *__restrict__ pairs, const int *__restrict__ rowptr,
+                                                      const float *__restrict__ mom, float *__restrict__ loc)
+{
+    constexpr int NTAB = 3 * kM2LOffsets * 16;
+    __shared__ __align__(16) float tab[NTAB];
+    __shared__ float U[SPAN * SPAN * 64];
+    const int bx = blockIdx.x, lane = threadIdx.x;
+    const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    if (m0 == m1) return;
+    const int a0 = lane & 3, a1 = (lane >> 2) & 3, a2 = lane >> 4;
+    for (int e = lane; e < NTAB; e += 64) tab[e] = tables[e];
+    for (int e = lane; e < SPAN * SPAN * 64; e += 64) U[e] = 0.f;
+    int cx[3];
+#pragma unroll
+    for (int j = 0; j < 3; j++) cx[j] = cellx[(long long)bx * 3 + j] + sm.omin[j];
+    float extra = 0.f;
+    __syncthreads();
+    // the far list is consumed 64 boxes at a time: every lane fetches the id and the table indices of one
+    // far box, then the wavefront walks through them (four moment vectors in flight at a time)
+    for (int mb = m0; mb < m1; mb += 64) {
+        const int mi = mb + lane;
+        int byv = 0, pk = 0;
+        if (mi < m1) {
+            byv = pairs[2 * (long long)mi + 1];
+            int o0 = celly[(long long)byv * 3 + 0] - cx[0];
+            int o1 = celly[(long long)byv * 3 + 1] - cx[1];
+            int o2 = celly[(long long)byv * 3 + 2] - cx[2];
+            o0 = min(max(o0, 0), kM2LOffsets - 1);
+            o1 = min(max(o1, 0), kM2LOffsets - 1);
+            o2 = min(max(o2, 0), kM2LOffsets - 1);
+            pk = o0 | (o1 << 8) | (o2 << 16);
+        }
+        const int cnt = min(64, m1 - mb);
+        for (int j = 0; j < cnt; j += 4) {
+            float v[4];
+            int pkj[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int jj = min(j + u, cnt - 1);
+                const int by = wave_readlane(byv, jj);
+                pkj[u] = wave_readlane(pk, jj);
+                v[u] = mom[(long long)by * 64 + lane];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                if (j + u >= cnt) break;             // uniform over the wavefront
+                const int o0 = pkj[u] & 255, o1 = (pkj[u] >> 8) & 255, o2 = pkj[u] >> 16;
+                const int g1 = o1 - lo1, g2 = o2 - lo2;
+                const float4 r = *reinterpret_cast<const float4 *>(&tab[(0 * kM2LOffsets + o0) * 16 + a0 * 4]);
+                float sacc = r.x * quad_bcast<0>(v[u]);
+                sacc = fmaf(r.y, quad_bcast<1>(v[u]), sacc);
+                sacc = fmaf(r.z, quad_bcast<2>(v[u]), sacc);
+                sacc = fmaf(r.w, quad_bcast<3>(v[u]), sacc);
+                if (g1 >= 0 && g1 < SPAN && g2 >= 0 && g2 < SPAN) {
+                    U[(g1 * SPAN + g2) * 64 + lane] += sacc;
+                } else {
+                    // An offset outside the expected span (a parent pair that sat exactly on the far
+                    // threshold and was decided by rounding): apply the other two factors directly.
+                    const float4 r1 = *reinterpret_cast<const float4 *>(&tab[(1 * kM2LOffsets + o1) * 16 + a1 * 4]);
+                    float t = r1.x * wave_shfl_f(sacc, (lane & ~12) | 0);
+                    t = fmaf(r1.y, wave_shfl_f(sacc, (lane & ~12) | 4), t);
+                    t = fmaf(r1.z, wave_shfl_f(sacc, (lane & ~12) | 8), t);
+                    t = fmaf(r1.w, wave_shfl_f(sacc, (lane & ~12) | 12), t);
+                    const float4 r2 = *reinterpret_cast<const float4 *>(&tab[(2 * kM2LOffsets + o2) * 16 + a2 * 4]);
+                    extra = fmaf(r2.x, wave_shfl_f(t, (lane & 15) | 0), extra);
+                    extra = fmaf(r2.y, wave_shfl_f(t, (lane & 15) | 16), extra);
+                    extra = fmaf(r2.z, wave_shfl_f(t, (lane & 15) | 32), extra);
+                    extra = fmaf(r2.w, wave_shfl_f(t, (lane & 15) | 48), extra);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // second factor: per (o1, o2) slot; lanes that differ in a1 exchange values
+    float V[SPAN];
+#pragma unroll
+    for (int g2 = 0; g2 < SPAN; g2++) V[g2] = 0.f;
+    for (int g1 = 0; g1 < SPAN; g1++) {
+        const int o1 = min(lo1 + g1, kM2LOffsets - 1);
+        const float4 r = *reinterpret_cast<const float4 *>(&tab[(1 * kM2LOffsets + o1) * 16 + a1 * 4]);
+#pragma unroll
+        for (int g2 = 0; g2 < SPAN; g2++) {
+            const float u = U[(g1 * SPAN + g2) * 64 + lane];
+            float t = V[g2];
+            t = fmaf(r.x, wave_shfl_f(u, (lane & ~12) | 0), t);
+            t = fmaf(r.y, wave_shfl_f(u, (lane & ~12) | 4), t);
+            t = fmaf(r.z, wave_shfl_f(u, (lane & ~12) | 8), t);
+            t = fmaf(r.w, wave_shfl_f(u, (lane & ~12) | 12), t);
+            V[g2] = t;
+        }
+    }
+    // third factor: per o2; lanes that differ in a2 exchange values
+    float out = 0.f;
+#pragma unroll
+    for (int g2 = 0; g2 < SPAN; g2++) {
+        const int o2 = min(lo2 + g2, kM2LOffsets - 1);
+        const float4 r = *reinterpret_cast<const float4 *>(&tab[(2 * kM2LOffsets + o2) * 16 + a2 * 4]);
+        out = fmaf(r.x, wave_shfl_f(V[g2], (lane & 15) | 0), out);
+        out = fmaf(r.y, wave_shfl_f(V[g2], (lane & 15) | 16), out);
+        out = fmaf(r.z, wave_shfl_f(V[g2], (lane & 15) | 32), out);
+        out = fmaf(r.w, wave_shfl_f(V[g2], (lane & 15) | 48), out);
+    }
+    loc[(long long)bx * 64 + lane] = out + extra;
+}
+
 // ------------------------------------------------------------------------------------------------
 // L2P (F3M_src/1_d_conv.cu:554-659): out_i += sum_m L_m(x_i) Loc[box][m].  One lane per point; the
 // product over dimensions >= 1 is reused along dimension 0.
@@ -988,6 +1102,22 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         check_launch("sep_tables");
         size_t shs = sizeof(float) * ((size_t)ntab + 2 * (size_t)P);
         timer_begin(kM2L, s);
+        const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
+        if (q64) {
+            // one tree: cell offsets of far pairs are -3..3; two trees: at most 10 distinct values per dimension
+            // table index of the lowest expected offset: one tree: cell offsets of far pairs are -3..3; two
+            // trees: centre distances stay below 5 edges, i.e. offsets from ceil(-5 - delta/edge) on, at most
+            // 11 distinct values.  (Anything outside is still handled, pair by pair.)
+            int lo[3];
+            for (int j = 0; j < 3; j++)
+                lo[j] = (&tx == &ty ? -3 : (int)std::ceil(-5.0 - sg.delta[j] / edge)) - sm.omin[j];
+            if (&tx == &ty)
+                F3M_LAUNCH((m2l_q64_kernel<7>), lx.nb, 64, 0, s, dtab.get(), sm, lo[1], lo[2], lx.cell.get(), ly.cell.get(),
+                           far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());
+            else
+                F3M_LAUNCH((m2l_q64_kernel<11>), lx.nb, 64, 0, s, dtab.get(), sm, lo[1], lo[2], lx.cell.get(), ly.cell.get(),
+                           far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());
+        } else {
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((m2l_sep_kernel<DD>), lx.nb, bdp, shs, s, dtab.get(), ntab, nm, sm, lx.cell.get(), ly.cell.get(),   \
@@ -999,6 +1129,7 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         default: throw Error(2, "dimension must be 1..10");
         }
 #undef F3M_CASE
+        }
         timer_end(s);
         check_launch("m2l_sep");
     } else {

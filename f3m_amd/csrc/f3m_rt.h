@@ -167,7 +167,18 @@ __device__ inline unsigned long long wave_ballot(bool p) { return emu::ballot(p)
 __device__ inline unsigned lane_id() { return emu::S().cur->tid % 64; }
 __device__ inline float fast_exp2(float x) { return exp2f(x); }
 __device__ inline float fast_rcp(float x) { return 1.0f / x; }
+__device__ inline float wave_shfl_f(float v, int src)
+{
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    u = emu::shfl_bits(u, src);
+    memcpy(&v, &u, 4);
+    return v;
+}
+// value of lane (l & ~3) | K of the same group of four lanes
+template <int K> __device__ inline float quad_bcast(float v) { return wave_shfl_f(v, (int)((lane_id() & ~3u) | K)); }
 __device__ inline int wave_shfl_i(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }
+__device__ inline int wave_readlane(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }   // src uniform
 __device__ inline float wave_shfl_xor_f(float v, int mask)
 {
     uint32_t u;
@@ -259,7 +270,15 @@ __device__ __forceinline__ unsigned long long wave_ballot(bool p) { return __bal
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }   // v_rcp_f32, 1 ulp
+__device__ __forceinline__ float wave_shfl_f(float v, int src) { return __shfl(v, src, 64); }
+// value of lane (l & ~3) | K of the same group of four lanes (DPP quad_perm:[K,K,K,K], no LDS traffic)
+template <int K> __device__ __forceinline__ float quad_bcast(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), K * 0x55, 0xf, 0xf, false));
+}
 __device__ __forceinline__ int wave_shfl_i(int v, int src) { return __shfl(v, src, 64); }
+// value of one lane, the same lane for the whole wavefront (v_readlane_b32: the result is scalar)
+__device__ __forceinline__ int wave_readlane(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
 __device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half_t;
