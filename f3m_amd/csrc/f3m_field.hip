@@ -398,12 +398,27 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
 #pragma unroll
     for (int q = 0; q < TPW; q++) acc[q] = 0.f;
     const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
-    for (int m = m0; m < m1; m++) {
-        const int by = pairs[2 * (long long)m + 1];
-        const int s0 = offy[by], s1 = offy[by + 1];
+    // the list is consumed 64 y boxes at a time: every lane fetches the range and centre of one y box,
+    // then the wavefront walks through them (one round of memory latency per 64 boxes)
+    for (int mb = m0; mb < m1; mb += 64) {
+      const int mi = mb + lane;
+      int s0v = 0, s1v = 0;
+      float cyv[D];
+#pragma unroll
+      for (int k = 0; k < D; k++) cyv[k] = 0.f;
+      if (mi < m1) {
+          const int byv = pairs[2 * (long long)mi + 1];
+          s0v = offy[byv];
+          s1v = offy[byv + 1];
+#pragma unroll
+          for (int k = 0; k < D; k++) cyv[k] = ctry[(long long)byv * D + k];
+      }
+      const int mcnt = min(64, m1 - mb);
+      for (int mj = 0; mj < mcnt; mj++) {
+        const int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mj);
         float cy[D];
 #pragma unroll
-        for (int k = 0; k < D; k++) cy[k] = ctry[(long long)by * D + k];
+        for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
         // target operands relative to the centre of this y box
         h8 bop[TPW][NS];
 #pragma unroll
@@ -460,6 +475,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
                 }
             }
         }
+      }
     }
 #pragma unroll
     for (int q = 0; q < TPW; q++) {
