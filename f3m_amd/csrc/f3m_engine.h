@@ -96,6 +96,22 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);
 
+// the three stages of one level on their own; flag (one int per box, or nullptr = every box) selects
+// the boxes whose points are interpolated
+void mark_far_boxes(const PairList &far, int nbx, int nby, int *fx, int *fy, hipStream_t s);
+void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, NodeSet &ns, const float *bs, float *mom,
+               hipStream_t s);
+void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
+               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc /* overwritten */, hipStream_t s);
+void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
+               hipStream_t s);
+// expansions moved between a level and the next deeper one: moments up (down = false, dst = parent
+// moments, overwritten) or local expansions down (down = true, dst = child expansions, added to)
+bool nodes_nest(const NodeSet &coarse, const NodeSet &fine);
+void make_shift_tables(const NodeSet &nsp, const NodeSet &nsc, DBuf<float> &tab, hipStream_t s);
+void shift_level(bool down, const TreeLevel &parent, const TreeLevel &child, const NodeSet &nsp, const NodeSet &nsc,
+                 const float *tab, const float *src, float *dst, hipStream_t s);
+
 void exact_f32(int d, const float *X, long long N, const float *Y, long long M, const float *b, int c, float ls,
                bool grad, float *out, hipStream_t s);
 void exact_f64(int d, const double *X, long long N, const double *Y, long long M, const double *b, int c, double ls,

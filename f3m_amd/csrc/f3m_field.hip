@@ -1053,27 +1053,33 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict_
     outs[i] += acc;
 }
 
-void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
-               NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode, float *mom_out, float *loc_out,
+void mark_far_boxes(const PairList &far, int nbx, int nby, int *fx, int *fy, hipStream_t s)
+{
+    // participating boxes: x boxes with a non-empty far row, y boxes that occur in the far list
+    F3M_LAUNCH(mark_rows_kernel, cdiv(nbx, 256), 256, 0, s, far.rowptr.get(), nbx, fx);
+    check_launch("mark_rows");
+    F3M_HIP(hipMemsetAsync(fy, 0, sizeof(int) * (size_t)nby, s));
+    if (far.n > 0) {
+        F3M_LAUNCH(mark_cols_kernel, cdiv(far.n, 256), 256, 0, s, far.pairs.get(), far.n, fy);
+        check_launch("mark_cols");
+    }
+}
+
+static void check_nodes(const NodeSet &ns)
+{
+    F3M_REQUIRE(ns.P <= 1024, 30, "at most 1024 interpolation nodes per box are supported (got %d)", ns.P);
+}
+
+void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, NodeSet &ns, const float *bs, float *mom,
                hipStream_t s)
 {
-    if (far.n == 0) return;
+    check_nodes(ns);
     const int P = ns.P;
-    F3M_REQUIRE(P <= 1024, 30, "at most 1024 interpolation nodes per box are supported (got %d)", P);
     NodeMeta nm = meta_of(ns);
-    const float factor = 2 / lx.edge;                  // F3M_src/1_d_conv.cu:473
-    // participating boxes: x boxes with a non-empty far row, y boxes that occur in the far list
-    DBuf<int> fx((size_t)lx.nb), fy((size_t)ly.nb);
-    F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, far.rowptr.get(), lx.nb, fx.get());
-    check_launch("mark_rows");
-    F3M_HIP(hipMemsetAsync(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s));
-    F3M_LAUNCH(mark_cols_kernel, cdiv(far.n, 256), 256, 0, s, far.pairs.get(), far.n, fy.get());
-    check_launch("mark_cols");
-
-    // P2M
+    const float factor = 2 / ly.edge;                  // F3M_src/1_d_conv.cu:473
     DBuf<int> tiley;
-    int nty = build_tiles(ly.off.get(), fy.get(), ly.nb, ty.n, kP2MChunk, tiley, s);
-    DBuf<float> partial((size_t)std::max(1, nty) * P), mom((size_t)ly.nb * P), loc((size_t)lx.nb * P);
+    int nty = build_tiles(ly.off.get(), flag, ly.nb, ty.n, kP2MChunk, tiley, s);
+    DBuf<float> partial((size_t)std::max(1, nty) * P);
     int bdp = ((P + kWave - 1) / kWave) * kWave;
     size_t shp = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)kP2MSub * ns.S1);
 #define F3M_CASE(DD)                                                                                                   \
@@ -1081,8 +1087,8 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         F3M_LAUNCH((p2m_kernel<DD>), nty, bdp, shp, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(), \
                    ly.nb, nm, ns.dt.get(), ns.dw.get(), factor, partial.get());                                        \
         break;
+    timer_begin(kP2M, s);
     if (nty > 0) {
-        timer_begin(kP2M, s);
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
             F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
@@ -1091,12 +1097,20 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         check_launch("p2m");
     }
 #undef F3M_CASE
-    F3M_LAUNCH(p2m_reduce_kernel, cdiv((long long)ly.nb * P, 256), 256, 0, s, partial.get(), tiley.get(), ly.nb, P, mom.get());
-    if (nty > 0) timer_end(s);
+    F3M_LAUNCH(p2m_reduce_kernel, cdiv((long long)ly.nb * P, 256), 256, 0, s, partial.get(), tiley.get(), ly.nb, P, mom);
+    timer_end(s);
     check_launch("p2m_reduce");
+}
 
-    // M2L
-    F3M_HIP(hipMemsetAsync(loc.get(), 0, sizeof(float) * (size_t)lx.nb * P, s));
+void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
+               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc, hipStream_t s)
+{
+    check_nodes(ns);
+    const int P = ns.P;
+    NodeMeta nm = meta_of(ns);
+    int bdp = ((P + kWave - 1) / kWave) * kWave;
+    F3M_HIP(hipMemsetAsync(loc, 0, sizeof(float) * (size_t)lx.nb * P, s));
+    if (far.n == 0) return;
     int NT = 1;
     for (int j = 0; j < d; j++) NT = std::max(NT, ns.n[j]);
     const int ntab = d * kM2LOffsets * NT * NT;
@@ -1120,7 +1134,6 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         timer_begin(kM2L, s);
         const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
         if (q64) {
-            // one tree: cell offsets of far pairs are -3..3; two trees: at most 10 distinct values per dimension
             // table index of the lowest expected offset: one tree: cell offsets of far pairs are -3..3; two
             // trees: centre distances stay below 5 edges, i.e. offsets from ceil(-5 - delta/edge) on, at most
             // 11 distinct values.  (Anything outside is still handled, pair by pair.)
@@ -1129,15 +1142,15 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                 lo[j] = (&tx == &ty ? -3 : (int)std::ceil(-5.0 - sg.delta[j] / edge)) - sm.omin[j];
             if (&tx == &ty)
                 F3M_LAUNCH((m2l_q64_kernel<7>), lx.nb, 64, 0, s, dtab.get(), sm, lo[1], lo[2], lx.cell.get(), ly.cell.get(),
-                           far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());
+                           far.pairs.get(), far.rowptr.get(), mom, loc);
             else
                 F3M_LAUNCH((m2l_q64_kernel<11>), lx.nb, 64, 0, s, dtab.get(), sm, lo[1], lo[2], lx.cell.get(), ly.cell.get(),
-                           far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());
+                           far.pairs.get(), far.rowptr.get(), mom, loc);
         } else {
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((m2l_sep_kernel<DD>), lx.nb, bdp, shs, s, dtab.get(), ntab, nm, sm, lx.cell.get(), ly.cell.get(),   \
-                   far.pairs.get(), far.rowptr.get(), mom.get(), loc.get());                                           \
+                   far.pairs.get(), far.rowptr.get(), mom, loc);                                                       \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -1155,7 +1168,7 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((m2l_direct_kernel<DD>), lx.nb, bdp, shm, s, ns.noff.get(), P, lx.ctr.get(), ly.ctr.get(),          \
-                   far.pairs.get(), far.rowptr.get(), mom.get(), lcs * kLog2e, loc.get());                             \
+                   far.pairs.get(), far.rowptr.get(), mom, lcs * kLog2e, loc);                                         \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -1166,15 +1179,22 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         timer_end(s);
         check_launch("m2l");
     }
+}
 
-    // L2P
+void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
+               hipStream_t s)
+{
+    check_nodes(ns);
+    const int P = ns.P;
+    NodeMeta nm = meta_of(ns);
+    const float factor = 2 / lx.edge;
     DBuf<int> tilex;
-    int ntx = build_tiles(lx.off.get(), fx.get(), lx.nb, tx.n, kL2PBlock, tilex, s);
+    int ntx = build_tiles(lx.off.get(), flag, lx.nb, tx.n, kL2PBlock, tilex, s);
     size_t shl = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)P + (size_t)kL2PBlock * (ns.S1 | 1));
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((l2p_kernel<DD>), ntx, kL2PBlock, shl, s, tx.pts.get(), tx.n, outs, lx.off.get(), lx.ctr.get(),     \
-                   tilex.get(), lx.nb, nm, ns.dt.get(), ns.dw.get(), factor, loc.get());                               \
+                   tilex.get(), lx.nb, nm, ns.dt.get(), ns.dw.get(), factor, loc);                                     \
         break;
     if (ntx > 0) {
         timer_begin(kL2P, s);
@@ -1187,8 +1207,170 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         check_launch("l2p");
     }
 #undef F3M_CASE
+}
+
+// the far field of one level on its own, as the reference computes it (F3M_src/n_tree.cu:489-593)
+void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
+               NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode, float *mom_out, float *loc_out,
+               hipStream_t s)
+{
+    if (far.n == 0) return;
+    const int P = ns.P;
+    DBuf<int> fx((size_t)lx.nb), fy((size_t)ly.nb);
+    mark_far_boxes(far, lx.nb, ly.nb, fx.get(), fy.get(), s);
+    DBuf<float> mom((size_t)ly.nb * P), loc((size_t)lx.nb * P);
+    p2m_level(d, ty, ly, fy.get(), ns, bs, mom.get(), s);
+    m2l_level(d, tx, lx, ty, ly, far, ns, lcs, m2l_mode, mom.get(), loc.get(), s);
+    l2p_level(d, tx, lx, fx.get(), ns, loc.get(), outs, s);
     if (mom_out) F3M_HIP(hipMemcpyAsync(mom_out, mom.get(), sizeof(float) * (size_t)ly.nb * P, hipMemcpyDeviceToDevice, s));
     if (loc_out) F3M_HIP(hipMemcpyAsync(loc_out, loc.get(), sizeof(float) * (size_t)lx.nb * P, hipMemcpyDeviceToDevice, s));
+}
+
+// ------------------------------------------------------------------------------------------------
+// Moving expansions between a box and its children (no counterpart in the reference, which
+// interpolates every level from the points: F3M_src/n_tree.cu:489-593).  The Lagrange polynomials of
+// a box, restricted to a child, are polynomials of the same degree, so interpolation at the child's
+// nodes reproduces them exactly when the child has at least as many nodes per dimension:
+//     L^parent_m(y) = sum_a L^parent_m(node^child_a) L^child_a(y)   for y in the child.
+// Hence  Mom_parent[m] = sum_children sum_a T[m][a] Mom_child[a]   (upward) and the local expansion
+// of a parent acts on a child's points as  Loc_child[a] += sum_m T[m][a] Loc_parent[m]  (downward),
+// with T = tensor product of 1-D tables T_j[s][m][a] = l_m(s/2 + t_a/2), s = -1/+1 for the lower/upper
+// half.  The sums are the same as the reference's up to rounding; the points are read once per product
+// instead of once per level.
+
+struct ShiftMeta {
+    int np[kMaxD], nc[kMaxD];   // nodes per dimension of the parent's and of the child's node set
+    int Pp, Pc, NTp, NTc;
+};
+
+__global__ void shift_tables_kernel(ShiftMeta sm, int d, NodeMeta nmp, NodeMeta nmc, const float *__restrict__ tp,
+                                    const float *__restrict__ wp, const float *__restrict__ tc, float *__restrict__ tab)
+{
+    int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= d * 2 * sm.NTp * sm.NTc) return;
+    const int a = e % sm.NTc, m = (e / sm.NTc) % sm.NTp, sg = (e / (sm.NTc * sm.NTp)) % 2, j = e / (sm.NTc * sm.NTp * 2);
+    float v = 0.f;
+    if (m < sm.np[j] && a < sm.nc[j]) {
+        const double tau = (sg ? 0.5 : -0.5) + 0.5 * (double)tc[nmc.start[j] + a];
+        double sum = 0, mine = 0;
+        int hit = -1;
+        for (int l = 0; l < sm.np[j]; l++) {
+            double diff = tau - (double)tp[nmp.start[j] + l];
+            if (diff == 0) { hit = l; continue; }
+            double q = (double)wp[nmp.start[j] + l] / diff;
+            if (l == m) mine = q;
+            sum += q;
+        }
+        v = hit >= 0 ? (hit == m ? 1.f : 0.f) : (float)(mine / sum);
+    }
+    tab[e] = v;
+}
+
+// One workgroup per parent box.  DOWN = false: dst[parent] = sum over children of T src[child];
+// DOWN = true: dst[child] += T^t src[parent].  The d one-dimensional factors are applied one after
+// the other through two LDS buffers.
+template <bool DOWN>
+__global__ void __launch_bounds__(1024) shift_kernel(const float *__restrict__ tables, int ntab, ShiftMeta sm, int d,
+                                                      const int *__restrict__ childstart, const int *__restrict__ cellc,
+                                                      const float *__restrict__ src, float *__restrict__ dst)
+{
+    F3M_DYN_SHARED(float, smem);
+    float *tab = smem;                     // ntab
+    float *bufA = smem + ntab;             // Pc (the larger of the two node counts)
+    float *bufB = bufA + sm.Pc;
+    float *par = bufB + sm.Pc;             // Pp: the parent's expansion (DOWN only)
+    const int b = blockIdx.x, tid = threadIdx.x, BD = blockDim.x;
+    for (int e = tid; e < ntab; e += BD) tab[e] = tables[e];
+    if (DOWN)
+        for (int e = tid; e < sm.Pp; e += BD) par[e] = src[(long long)b * sm.Pp + e];
+    const int *nin = DOWN ? sm.np : sm.nc, *nout = DOWN ? sm.nc : sm.np;
+    const int Pin = DOWN ? sm.Pp : sm.Pc, Pout = DOWN ? sm.Pc : sm.Pp;
+    float acc = 0.f;                       // UP: this lane's element of the parent (BD >= Pp)
+    for (int c = childstart[b]; c < childstart[b + 1]; c++) {
+        __syncthreads();
+        for (int e = tid; e < Pin; e += BD) bufA[e] = DOWN ? par[e] : src[(long long)c * sm.Pc + e];
+        __syncthreads();
+        float *in = bufA, *out = bufB;
+        int lo = 1;                        // product of nout over the dimensions already done
+        int hi = Pin;                      // product of nin over the dimensions still to do (incl. j)
+        for (int j = 0; j < d; j++) {
+            hi /= nin[j];
+            const int sg = cellc[(long long)c * d + j] & 1;
+            const float *T = tab + (size_t)(j * 2 + sg) * sm.NTp * sm.NTc;
+            const int size = lo * nout[j] * hi;
+            for (int e = tid; e < size; e += BD) {
+                const int l = e % lo, q = (e / lo) % nout[j], h = e / (lo * nout[j]);
+                const float *sp = in + l + lo * nin[j] * h;
+                float sum = 0.f;
+                for (int r = 0; r < nin[j]; r++) {
+                    // T[m][a] with m = parent node, a = child node
+                    const float t = DOWN ? T[r * sm.NTc + q] : T[q * sm.NTc + r];
+                    sum = fmaf(t, sp[lo * r], sum);
+                }
+                if (j == d - 1) {
+                    if (DOWN) dst[(long long)c * sm.Pc + e] += sum;
+                    else acc += sum;
+                } else {
+                    out[e] = sum;
+                }
+            }
+            lo *= nout[j];
+            __syncthreads();
+            float *t = in; in = out; out = t;
+        }
+    }
+    if (!DOWN && tid < Pout) dst[(long long)b * sm.Pp + tid] = acc;
+}
+
+bool nodes_nest(const NodeSet &coarse, const NodeSet &fine)
+{
+    if (coarse.d != fine.d) return false;
+    for (int j = 0; j < coarse.d; j++)
+        if (coarse.n[j] > fine.n[j]) return false;
+    return true;
+}
+
+static ShiftMeta shift_meta(const NodeSet &nsp, const NodeSet &nsc)
+{
+    ShiftMeta sm;
+    sm.Pp = nsp.P; sm.Pc = nsc.P; sm.NTp = 1; sm.NTc = 1;
+    for (int j = 0; j < kMaxD; j++) {
+        sm.np[j] = j < nsp.d ? nsp.n[j] : 1;
+        sm.nc[j] = j < nsc.d ? nsc.n[j] : 1;
+        sm.NTp = std::max(sm.NTp, sm.np[j]);
+        sm.NTc = std::max(sm.NTc, sm.nc[j]);
+    }
+    return sm;
+}
+
+void make_shift_tables(const NodeSet &nsp, const NodeSet &nsc, DBuf<float> &tab, hipStream_t s)
+{
+    F3M_REQUIRE(nodes_nest(nsp, nsc), 33, "child node set is coarser than the parent's");
+    ShiftMeta sm = shift_meta(nsp, nsc);
+    const int ntab = nsp.d * 2 * sm.NTp * sm.NTc;
+    tab.reset((size_t)ntab);
+    F3M_LAUNCH(shift_tables_kernel, cdiv(ntab, 256), 256, 0, s, sm, nsp.d, meta_of(nsp), meta_of(nsc), nsp.dt.get(),
+               nsp.dw.get(), nsc.dt.get(), tab.get());
+    check_launch("shift_tables");
+}
+
+void shift_level(bool down, const TreeLevel &parent, const TreeLevel &child, const NodeSet &nsp, const NodeSet &nsc,
+                 const float *tab, const float *src, float *dst, hipStream_t s)
+{
+    check_nodes(nsc);
+    ShiftMeta sm = shift_meta(nsp, nsc);
+    const int d = nsp.d, ntab = d * 2 * sm.NTp * sm.NTc;
+    const int bd = ((sm.Pc + kWave - 1) / kWave) * kWave;
+    size_t sh = sizeof(float) * ((size_t)ntab + 2 * (size_t)sm.Pc + (size_t)sm.Pp);
+    timer_begin(down ? kL2P : kP2M, s);
+    if (down)
+        F3M_LAUNCH((shift_kernel<true>), parent.nb, bd, sh, s, tab, ntab, sm, d, parent.childstart.get(), child.cell.get(),
+                   src, dst);
+    else
+        F3M_LAUNCH((shift_kernel<false>), parent.nb, bd, sh, s, tab, ntab, sm, d, parent.childstart.get(), child.cell.get(),
+                   src, dst);
+    timer_end(s);
+    check_launch("shift");
 }
 
 }  // namespace f3m

@@ -86,6 +86,18 @@ struct f3m_plan {
     std::vector<PlanLevel> levels;         // levels[k-1] = depth k
     std::map<int, std::unique_ptr<NodeSet>> nodes;
     DBuf<float> Xraw, Yraw;                // row-major copies, only when no division happened
+    std::map<std::pair<int, int>, std::unique_ptr<DBuf<float>>> shift_tabs;   // (parent nodes, child nodes)
+    const float *shift_table(int nodes_parent, int nodes_child, hipStream_t s)
+    {
+        auto key = std::make_pair(nodes_parent, nodes_child);
+        auto it = shift_tabs.find(key);
+        if (it == shift_tabs.end()) {
+            std::unique_ptr<DBuf<float>> t(new DBuf<float>());
+            make_shift_tables(nodeset(nodes_parent, s), nodeset(nodes_child, s), *t, s);
+            it = shift_tabs.emplace(key, std::move(t)).first;
+        }
+        return it->second->get();
+    }
     NodeSet &nodeset(int num_nodes, hipStream_t s)
     {
         auto it = nodes.find(num_nodes);
@@ -237,15 +249,74 @@ static void check_level(const f3m_plan *P, int level)
     F3M_REQUIRE(level >= 1 && level <= (int)P->levels.size(), 11, "level %d out of range 1..%d", level, (int)P->levels.size());
 }
 
+static int m2l_mode_env()
+{
+    // F3M_M2L=direct|separable forces one form of the M2L kernel (default: separable when its tables fit)
+    int mode = 0;
+    if (const char *e = getenv("F3M_M2L")) mode = !strcmp(e, "direct") ? 1 : (!strcmp(e, "separable") ? 2 : 0);
+    return mode;
+}
+
 static void far_level(f3m_plan *P, int level, const float *bs, float *outs, float *mom, float *loc, hipStream_t s)
 {
     PlanLevel &L = P->levels[level - 1];
     if (L.far.n == 0) return;
     NodeSet &ns = P->nodeset(L.num_nodes, s);
-    // F3M_M2L=direct|separable forces one form of the M2L kernel (default: separable when its tables fit)
-    int mode = 0;
-    if (const char *e = getenv("F3M_M2L")) mode = !strcmp(e, "direct") ? 1 : (!strcmp(e, "separable") ? 2 : 0);
+    const int mode = m2l_mode_env();
     far_field(P->d, P->tx, P->tx.lev[level], *P->ty, P->ty->lev[level], L.far, ns, bs, outs, P->lcs, mode, mom, loc, s);
+}
+
+// Far field of all levels in one upward and one downward sweep: the points are interpolated once, at
+// the deepest level with far pairs; moments of shallower levels come from their children and local
+// expansions are handed down to the children, level by level, before one evaluation at the points.
+// Where a level has more nodes per dimension than the next deeper one (var_compression lowers the node
+// count of small boxes, F3M_src/n_tree.cu:971-978) the hand-over would not be exact, and that level
+// is interpolated from / evaluated at the points directly, as the reference does for every level.
+static void far_tree(f3m_plan *P, const float *bs, float *outs, hipStream_t s)
+{
+    const int depth = (int)P->levels.size();
+    int ku = 0, kd = 0;
+    for (int k = 1; k <= depth; k++)
+        if (P->levels[k - 1].far.n > 0) { if (!ku) ku = k; kd = k; }
+    if (!ku) return;
+    const int mode = m2l_mode_env();
+    const int d = P->d;
+    auto ns_of = [&](int k) -> NodeSet & { return P->nodeset(P->levels[k - 1].num_nodes, s); };
+    std::vector<DBuf<float>> mom((size_t)depth + 1);
+    // upward
+    for (int k = kd; k >= ku; k--) {
+        NodeSet &ns = ns_of(k);
+        const TreeLevel &ly = P->ty->lev[k];
+        mom[k].reset((size_t)ly.nb * ns.P);
+        if (k < kd && nodes_nest(ns, ns_of(k + 1))) {
+            const float *tab = P->shift_table(P->levels[k - 1].num_nodes, P->levels[k].num_nodes, s);
+            shift_level(false, ly, P->ty->lev[k + 1], ns, ns_of(k + 1), tab, mom[k + 1].get(), mom[k].get(), s);
+        } else {
+            p2m_level(d, *P->ty, ly, nullptr, ns, bs, mom[k].get(), s);
+        }
+    }
+    // downward
+    DBuf<float> loc, prev;
+    int pending = 0;        // level whose local expansions (in prev) still wait to be evaluated
+    for (int k = ku; k <= kd; k++) {
+        NodeSet &ns = ns_of(k);
+        const TreeLevel &lx = P->tx.lev[k];
+        loc.reset((size_t)lx.nb * ns.P);
+        m2l_level(d, P->tx, lx, *P->ty, P->ty->lev[k], P->levels[k - 1].far, ns, P->lcs, mode, mom[k].get(), loc.get(), s);
+        mom[k].free();
+        if (pending) {
+            NodeSet &nsp = ns_of(pending);
+            if (nodes_nest(nsp, ns)) {
+                const float *tab = P->shift_table(P->levels[pending - 1].num_nodes, P->levels[k - 1].num_nodes, s);
+                shift_level(true, P->tx.lev[pending], lx, nsp, ns, tab, prev.get(), loc.get(), s);
+            } else {
+                l2p_level(d, P->tx, P->tx.lev[pending], nullptr, nsp, prev.get(), outs, s);
+            }
+        }
+        std::swap(loc, prev);
+        pending = k;
+    }
+    l2p_level(d, P->tx, P->tx.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s);
 }
 
 static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s)
@@ -263,6 +334,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     }
     DBuf<float> bs((size_t)P->M + 32), outs((size_t)P->N);   // bs padded: near_g_kernel reads whole tiles
     const int depth = (int)P->levels.size();
+    // F3M_FAR=levels: interpolate every level from the points like the reference (cross-check)
+    const char *fe = getenv("F3M_FAR");
+    const bool per_level = fe && !strcmp(fe, "levels");
     for (int col = 0; col < c; col++) {
         {
             Scope sc(kPerm, s);
@@ -273,8 +347,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             PlanLevel &L = P->levels[k - 1];
             // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
             near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s);
-            far_level(P, k, bs.get(), outs.get(), nullptr, nullptr, s);
+            if (per_level) far_level(P, k, bs.get(), outs.get(), nullptr, nullptr, s);
         }
+        if (!per_level) far_tree(P, bs.get(), outs.get(), s);
         // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
         near_field(P->d, P->tx, P->tx.lev[depth], *P->ty, P->ty->lev[depth], P->levels[depth - 1].keep, bs.get(),
                    outs.get(), P->lcs, s);

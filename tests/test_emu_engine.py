@@ -100,6 +100,41 @@ def test_stages_and_product(oracle, name, P):
     assert rel_l2(ee.kmvm(X, Y, b, **prm), got) == 0.0
 
 
+def test_far_sweeps_match_per_level_interpolation(oracle, monkeypatch):
+    """The engine interpolates the points once and moves moments / local expansions between levels;
+    F3M_FAR=levels interpolates every level from the points as the reference does
+    (F3M_src/n_tree.cu:489-593).  Both are the same sums up to rounding."""
+    rng = np.random.default_rng(21)
+    X = rng.random((8000, 2), dtype=f32)
+    b = rng.standard_normal((8000, 2)).astype(f32)
+    prm = dict(ls=0.7, min_points=60, nr_of_interpolation=9, small_field_points=4)
+    eng = ee.Plan(X, None, **prm)
+    far_levels = [k for k in range(1, eng.depth + 1) if eng.level_sizes(k)["nfar"]]
+    assert len(far_levels) >= 3                      # moments travel through at least two levels
+    sweeps = eng.apply(b)
+    monkeypatch.setenv("F3M_FAR", "levels")
+    per_level = eng.apply(b)
+    assert 0 < rel_l2(sweeps, per_level) < 2e-6       # two code paths, same sums up to rounding
+    assert rel_l2(sweeps, oracle.Plan(X, None, **prm).apply(b)) < 1e-5
+
+
+def test_far_sweeps_with_level_dependent_node_counts(oracle, monkeypatch):
+    """var_compression lowers the node count of deep levels (F3M_src/n_tree.cu:971-978): expansions
+    cannot be handed from a 4x4 grid to a 3x3 grid exactly, so those levels are interpolated directly."""
+    rng = np.random.default_rng(22)
+    X = rng.random((4000, 2), dtype=f32)
+    b = rng.standard_normal((4000, 1)).astype(f32)
+    prm = dict(ls=1.0, min_points=100, nr_of_interpolation=16, small_field_points=10, var_compression=True,
+               eff_var_limit=0.1)
+    eng = ee.Plan(X, None, **prm)
+    used = {eng.level_sizes(k)["num_nodes"] for k in range(1, eng.depth + 1) if eng.level_sizes(k)["nfar"]}
+    assert used == {16, 9}
+    sweeps = eng.apply(b)
+    assert rel_l2(sweeps, oracle.Plan(X, None, **prm).apply(b)) < 1e-5
+    monkeypatch.setenv("F3M_FAR", "levels")
+    assert rel_l2(sweeps, eng.apply(b)) < 2e-6
+
+
 def test_mfma_near_field(oracle, monkeypatch):
     monkeypatch.setenv("F3M_NEAR", "mfma")
     rng = np.random.default_rng(5)

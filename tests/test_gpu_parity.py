@@ -138,6 +138,23 @@ def test_product_error_vs_fp64_exact(eng, oracle, name):
     assert err <= 1e-3 or err_oracle > 1e-3 / 1.5, (err, err_oracle)
 
 
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform5", "uniform3_varcomp"])
+def test_far_sweeps_match_per_level_interpolation(eng, monkeypatch, name):
+    """Default: points interpolated once, moments and local expansions moved between levels.
+    F3M_FAR=levels: every level interpolated from the points like the reference
+    (F3M_src/n_tree.cu:489-593).  The same sums up to fp32 rounding."""
+    print("case far sweeps", name, flush=True)
+    rng = np.random.default_rng(13)
+    X, Y, prm = clouds(name, rng)
+    M = X.shape[0] if Y is None else Y.shape[0]
+    b = rng.standard_normal((M, 1)).astype(f32)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    sweeps = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_FAR", "levels")
+    per_level = plan.apply(dev(b)).cpu().numpy()
+    assert rel_l2(sweeps, per_level) < 5e-6
+
+
 def test_columns_linearity_and_plan_reuse(eng, oracle):
     rng = np.random.default_rng(11)
     X = rng.random((40000, 3), dtype=f32)
