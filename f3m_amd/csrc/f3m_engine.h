@@ -44,6 +44,10 @@ struct PairList {
     long long n = 0;
     DBuf<int> pairs;     // (n,2) int32: (bx, by), sorted by (bx, by)
     DBuf<int> rowptr;    // nbx+1: range of each x box
+    // far lists of one tree only: pairs whose y box is neither a child of one of the 3^d parents around
+    // the parent of the x box nor a child of a parent two cells away along one axis (a parent pair
+    // exactly on the far threshold, kept by rounding); -1 = not counted.  Expected to be 0.
+    long long outliers = -1;
 };
 
 struct ClassifyParams {

@@ -3,6 +3,7 @@
 #include "f3m_engine.h"
 
 #include <cmath>
+#include <type_traits>
 #include <cstdlib>
 #include <cstring>
 
@@ -996,6 +997,300 @@ __global__ void __launch_bounds__(64) m2l_q64_kernel(const float *__restrict__ t
 }
 
 // ------------------------------------------------------------------------------------------------
+// Separable M2L for d >= 3, one tree, one workgroup per PARENT box (or per group of GS of its 2^d
+// children when they do not all fit): the children ("siblings") of a box have almost the same far
+// boxes -- the children of the 3^d parents around their parent, 6^d cells, minus each sibling's own
+// neighbours -- so a moment vector is fetched once per workgroup and used by every sibling.
+//
+// Phase A writes the far rows of the siblings into a direct-address table in LDS, indexed by the cell
+// offset u = cell_y - 2 cell_parent in -2..3 per dimension (dimension 0 fastest), with a bit mask of
+// the siblings that list the box.  A parent pair two cells apart along one axis sits exactly on the
+// far threshold (distance = 2 edges) and fp32 rounding decides it; where it was kept, its children
+// appear in the far rows with u = -4, -3, 4 or 5 along that axis and 0 or 1 elsewhere.  Those cells
+// have a small table of their own.  Phase B walks each table in lexicographic order of the offsets,
+// last dimension outermost.  Lane (sibling, r2) owns the n0 x n1 nodes (a0, a1, r2) of one sibling:
+//   * per far box: factor 0 in registers (n0^2 n1 multiply-adds on the freshly loaded moments);
+//   * when the offsets of dimensions >= 1 change: factor 1 in registers;
+//   * when the offsets of dimensions >= j change (j >= 2): factor j, exchanging values between lanes
+//     through LDS.
+// So every factor beyond the first is applied once per group of far boxes that share the remaining
+// offsets instead of once per far box.  The per-sibling offset is u - (child bit), which shifts
+// every sibling's offsets by a constant and therefore leaves the walking order valid for all of them.
+// Preconditions (checked by the host): n0 = n1 = N, every far pair in one of the two tables.
+
+constexpr int kSibSpan = 6;
+__host__ __device__ constexpr int sib_codes(int d) { return d == 0 ? 1 : kSibSpan * sib_codes(d - 1); }
+__host__ __device__ constexpr int sib_ext_codes(int d) { return d * 4 * (1 << (d - 1)); }
+
+// table position of a far box from its cell offsets relative to twice the parent's cell, shifted by
+// 2 (so the regular range is 0..5): >= 0 regular table, -2 - e extension table entry e, -1 neither
+template <int D>
+__host__ __device__ inline int sib_code(const int *dg)
+{
+    int code = 0, mul = 1, nout = 0, jj = 0;
+    for (int j = 0; j < D; j++) {
+        if (dg[j] < 0 || dg[j] >= kSibSpan) { nout++; jj = j; }
+        code += dg[j] * mul;
+        mul *= kSibSpan;
+    }
+    if (nout == 0) return code;
+    if (nout > 1) return -1;
+    const int w = dg[jj];
+    const int v = w == -2 ? 0 : w == -1 ? 1 : w == 6 ? 2 : w == 7 ? 3 : -1;
+    if (v < 0) return -1;
+    int bits = 0, pos = 0;
+    for (int j = 0; j < D; j++) {
+        if (j == jj) continue;
+        if (dg[j] != 2 && dg[j] != 3) return -1;
+        bits |= (dg[j] - 2) << pos;
+        pos++;
+    }
+    return -2 - ((jj * 4 + v) * (1 << (D - 1)) + bits);
+}
+
+template <int D>
+__device__ inline void sib_ext_digits(int e, int *dg)
+{
+    constexpr int H = 1 << (D - 1);
+    const int jj = e / (4 * H), v = (e / H) % 4, bits = e % H;
+    int pos = 0;
+#pragma unroll
+    for (int j = 0; j < D; j++) {
+        if (j == jj) { dg[j] = v == 0 ? -2 : v == 1 ? -1 : v == 2 ? 6 : 7; }
+        else { dg[j] = 2 + ((bits >> pos) & 1); pos++; }
+    }
+}
+
+template <int K> struct __attribute__((aligned(4))) fvec { float v[K]; };
+
+template <int D, int N>
+__global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
+                                                        int R2, int GS, int nsub, const int *__restrict__ childstart,
+                                                        const int *__restrict__ cell, const int *__restrict__ pairs,
+                                                        const int *__restrict__ rowptr, const float *__restrict__ mom,
+                                                        float *__restrict__ loc)
+{
+    constexpr int NCODE = sib_codes(D), NEXT = sib_ext_codes(D), NN = N * N, NB = N <= 3 ? 4 : (D >= 4 ? 1 : 2);
+    F3M_DYN_SHARED(float, smem);
+    const int tid = threadIdx.x, BD = blockDim.x, lane = tid & 63;
+    int *tby = reinterpret_cast<int *>(smem);                       // NCODE: y box of a table cell
+    unsigned *tmask = reinterpret_cast<unsigned *>(smem) + NCODE;   // NCODE: siblings that list it
+    int *xby = reinterpret_cast<int *>(smem) + 2 * NCODE;           // NEXT: the same for the extension cells
+    unsigned *xmask = reinterpret_cast<unsigned *>(smem) + 2 * NCODE + NEXT;
+    int *xord = reinterpret_cast<int *>(smem) + 2 * NCODE + 2 * NEXT;   // NEXT: extension cells in walking order
+    int *xkey = xord + NEXT;                                        // NEXT
+    float *xbuf = smem + 2 * NCODE + 4 * NEXT;                      // NN * BD: exchange buffer
+    float *tabg = xbuf + NN * BD;                                   // ntab: E_j[o][a][q], row length sm.NT
+    float *tab01 = tabg + ((ntab + 3) & ~3);                        // 2 * 13 * N rows of 4: E_0, E_1 padded
+    float *zrow = tab01 + 2 * kM2LOffsets * N * 4;                  // N rows of zeros
+    int *sib = reinterpret_cast<int *>(zrow + N * 4);               // GS: compact id of each sibling or -1
+    const int px = blockIdx.x / nsub, sg = blockIdx.x % nsub;
+    const int P = nm.P;
+
+    for (int e = tid; e < NCODE; e += BD) { tby[e] = 0; tmask[e] = 0u; }
+    for (int e = tid; e < NEXT; e += BD) {
+        xby[e] = 0; xmask[e] = 0u;
+        int dg[D], key = 0, mul = 1;
+        sib_ext_digits<D>(e, dg);
+#pragma unroll
+        for (int j = 0; j < D; j++) { key += (dg[j] + 2) * mul; mul *= 10; }
+        xkey[e] = key;
+    }
+    for (int e = tid; e < ntab; e += BD) tabg[e] = tables[e];
+    for (int e = tid; e < 2 * kM2LOffsets * N * 4; e += BD) {
+        const int q = e & 3, a = (e >> 2) % N, o = (e / (4 * N)) % kM2LOffsets, j = e / (4 * N * kM2LOffsets);
+        tab01[e] = q < N ? tables[((j * kM2LOffsets + o) * sm.NT + a) * sm.NT + q] : 0.f;
+    }
+    for (int e = tid; e < N * 4; e += BD) zrow[e] = 0.f;
+    if (tid < GS) sib[tid] = -1;
+    __syncthreads();
+    for (int e = tid; e < NEXT; e += BD) {                 // walking order of the extension cells
+        const int key = xkey[e];
+        int rank = 0;
+        for (int f = 0; f < NEXT; f++) rank += xkey[f] < key;
+        xord[rank] = e;
+    }
+    const int c0 = childstart[px], c1 = childstart[px + 1];
+    for (int c = c0 + tid; c < c1; c += BD) {
+        int code = 0;
+#pragma unroll
+        for (int j = 0; j < D; j++) code |= (cell[(long long)c * D + j] & 1) << j;
+        const int sl = code - sg * GS;
+        if (sl >= 0 && sl < GS) sib[sl] = c;
+    }
+    int pc[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) pc[j] = 2 * (cell[(long long)c0 * D + j] >> 1) - 2;
+    __syncthreads();
+    for (int sl = 0; sl < GS; sl++) {
+        const int bx = sib[sl];
+        if (bx < 0) continue;                              // uniform over the workgroup
+        const int m1 = rowptr[bx + 1];
+        for (int m = rowptr[bx] + tid; m < m1; m += BD) {
+            const int by = pairs[2 * (long long)m + 1];
+            int dg[D];
+#pragma unroll
+            for (int j = 0; j < D; j++) dg[j] = cell[(long long)by * D + j] - pc[j];
+            const int code = sib_code<D>(dg);
+            if (code >= 0) { tby[code] = by; atomicOr(&tmask[code], 1u << sl); }
+            else if (code <= -2) { xby[-2 - code] = by; atomicOr(&xmask[-2 - code], 1u << sl); }
+        }
+    }
+    __syncthreads();
+
+    // this lane: sibling sl, position r2 among the nodes of dimensions >= 2
+    const int sl = tid / R2, r2 = tid % R2;
+    const bool valid = sl < GS;                            // lanes past the last sibling only keep step
+    const int mybox = valid ? sib[sl] : -1;
+    const bool live = mybox >= 0;
+    int cbit[D], dig[D], lstride[D];
+    {
+        const int code = sg * GS + (valid ? sl : 0);
+        int rem = r2, st = 1;
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            cbit[j] = 2 + ((code >> j) & 1) + sm.omin[j];  // table index of dimension j = digit_j - cbit[j]
+            dig[j] = 0; lstride[j] = 0;
+            if (j >= 2) { dig[j] = rem % nm.n[j]; rem /= nm.n[j]; lstride[j] = st; st *= nm.n[j]; }
+        }
+    }
+    const float *mine = mom + (long long)NN * (live ? r2 : 0);
+
+    float acc[D][NN];
+#pragma unroll
+    for (int j = 0; j < D; j++)
+#pragma unroll
+        for (int i = 0; i < NN; i++) acc[j][i] = 0.f;
+    int cur[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) cur[j] = 0;
+    bool have = false;
+
+    // applies factor l+1 to acc[l], adds the result to acc[l+1] and clears acc[l]
+    auto flush = [&](auto level) {
+        constexpr int l = decltype(level)::value, j = l + 1;
+        if constexpr (j == 1) {
+            int oi = cur[1] - cbit[1];
+            oi = min(max(oi, 0), kM2LOffsets - 1);
+            const float *T1 = tab01 + ((kM2LOffsets + oi) * N) * 4;
+#pragma unroll
+            for (int a1 = 0; a1 < N; a1++) {
+                const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
+                const float ev[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+                for (int a0 = 0; a0 < N; a0++) {
+                    float t = acc[1][a0 + N * a1];
+#pragma unroll
+                    for (int q = 0; q < N; q++) t = fmaf(ev[q], acc[0][a0 + N * q], t);
+                    acc[1][a0 + N * a1] = t;
+                }
+            }
+        } else {
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NN; i++) xbuf[i * BD + tid] = acc[l][i];
+            __syncthreads();
+            if (valid) {
+                int oi = cur[j] - cbit[j];
+                oi = min(max(oi, 0), kM2LOffsets - 1);
+                const float *row = tabg + ((j * kM2LOffsets + oi) * sm.NT + dig[j]) * sm.NT;
+                for (int q = 0; q < nm.n[j]; q++) {
+                    const float w = row[q];
+                    const float *src = xbuf + tid + (q - dig[j]) * lstride[j];
+#pragma unroll
+                    for (int i = 0; i < NN; i++) acc[j][i] = fmaf(w, src[i * BD], acc[j][i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NN; i++) acc[l][i] = 0.f;
+    };
+    auto flush_upto = [&](int jt) {       // levels 0 .. jt-1, jt uniform over the workgroup
+        if (jt > 0) flush(std::integral_constant<int, 0>());
+        if constexpr (D > 2) { if (jt > 1) flush(std::integral_constant<int, 1>()); }
+        if constexpr (D > 3) { if (jt > 2) flush(std::integral_constant<int, 2>()); }
+        if constexpr (D > 4) { if (jt > 3) flush(std::integral_constant<int, 3>()); }
+    };
+    // one far box: dg = its digits (uniform), v = its moments at this lane's nodes
+    auto far_box = [&](const int *dg, unsigned smask, const fvec<NN> &v) {
+        if (have) {
+            int jt = 0;
+#pragma unroll
+            for (int j = 1; j < D; j++) if (dg[j] != cur[j]) jt = j;
+            flush_upto(jt);
+        }
+#pragma unroll
+        for (int j = 0; j < D; j++) cur[j] = dg[j];
+        have = true;
+        const bool part = live && ((smask >> sl) & 1u);
+        int oi = dg[0] - cbit[0];
+        oi = min(max(oi, 0), kM2LOffsets - 1);
+        const float *T0 = part ? tab01 + (oi * N) * 4 : zrow;
+#pragma unroll
+        for (int a0 = 0; a0 < N; a0++) {
+            const float4 e = *reinterpret_cast<const float4 *>(T0 + a0 * 4);
+            const float ev[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+            for (int q1 = 0; q1 < N; q1++) {
+                float t = acc[0][a0 + N * q1];
+#pragma unroll
+                for (int q = 0; q < N; q++) t = fmaf(ev[q], v.v[q + N * q1], t);
+                acc[0][a0 + N * q1] = t;
+            }
+        }
+    };
+    // walks 64 table cells: ml, byl = this lane's cell; cellid = its id (regular code or extension entry)
+    auto walk64 = [&](unsigned ml, int byl, int cellid, auto ext) {
+        unsigned long long bal = wave_ballot(ml != 0u);
+        while (bal) {                                      // identical in every wavefront of the workgroup
+            int ls[NB], cnt = 0;
+            fvec<NN> v[NB];
+#pragma unroll
+            for (int u = 0; u < NB; u++) {
+                ls[u] = 0;
+                if (bal) { ls[u] = __ffsll(bal) - 1; bal &= bal - 1; cnt++; }
+                const int by = wave_readlane(byl, ls[u]);
+                v[u] = *reinterpret_cast<const fvec<NN> *>(mine + (long long)by * P);
+            }
+#pragma unroll
+            for (int u = 0; u < NB; u++) {
+                if (u >= cnt) break;                       // uniform
+                const int id = wave_readlane(cellid, ls[u]);
+                const unsigned smask = (unsigned)wave_readlane((int)ml, ls[u]);
+                int dg[D];
+                if constexpr (decltype(ext)::value) {
+                    sib_ext_digits<D>(id, dg);
+                } else {
+                    int rem = id;
+#pragma unroll
+                    for (int j = 0; j < D; j++) { dg[j] = rem % kSibSpan; rem /= kSibSpan; }
+                }
+                far_box(dg, smask, v[u]);
+            }
+        }
+    };
+
+    for (int base = 0; base < NCODE; base += 64) {
+        const int idx = base + lane;
+        walk64(idx < NCODE ? tmask[idx] : 0u, idx < NCODE ? tby[idx] : 0, idx, std::false_type());
+    }
+    if (have) flush_upto(D - 1);
+    have = false;
+    for (int base = 0; base < NEXT; base += 64) {
+        const int r = base + lane;
+        const int e = r < NEXT ? xord[r] : 0;
+        walk64(r < NEXT ? xmask[e] : 0u, xby[e], e, std::true_type());
+    }
+    if (have) flush_upto(D - 1);
+    if (live) {
+        fvec<NN> r;
+#pragma unroll
+        for (int i = 0; i < NN; i++) r.v[i] = acc[D - 1][i];
+        *reinterpret_cast<fvec<NN> *>(loc + (long long)mybox * P + (long long)NN * r2) = r;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // L2P (F3M_src/1_d_conv.cu:554-659): out_i += sum_m L_m(x_i) Loc[box][m].  One lane per point; the
 // product over dimensions >= 1 is reused along dimension 0.
 
@@ -1133,7 +1428,45 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         size_t shs = sizeof(float) * ((size_t)ntab + 2 * (size_t)P);
         timer_begin(kM2L, s);
         const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
-        if (q64) {
+        // sibling-group kernel: one tree, 3 <= d <= 5, n0 = n1 in 2..4, every far pair inside the 6^d cells
+        int sibGS = 0, sibR2 = 0;
+        size_t shsib = 0;
+        if (!q64 && m2l_mode == 0 && &tx == &ty && d >= 3 && d <= 5 && ns.n[0] == ns.n[1] && ns.n[0] >= 2 && ns.n[0] <= 4 &&
+            far.outliers == 0 && lx.depth >= 1) {
+            const int N = ns.n[0];
+            sibR2 = P / (N * N);
+            if (sibR2 <= 1024) {
+                sibGS = 1 << d;
+                while (sibGS * sibR2 > 1024) sibGS >>= 1;
+                const int bd = ((sibGS * sibR2 + kWave - 1) / kWave) * kWave;
+                shsib = sizeof(float) * (2 * (size_t)sib_codes(d) + 4 * (size_t)sib_ext_codes(d) + (size_t)N * N * bd + (size_t)((ntab + 3) & ~3) +
+                                         2 * (size_t)kM2LOffsets * N * 4 + (size_t)N * 4) + sizeof(int) * (size_t)sibGS;
+                if (shsib > 150 * 1024) sibGS = 0;
+            }
+        }
+        if (sibGS > 0) {
+            const TreeLevel &par = tx.lev[lx.depth - 1];
+            const int nsub = (1 << d) / sibGS;
+            const int bd = ((sibGS * sibR2 + kWave - 1) / kWave) * kWave;
+#ifndef F3M_CPU_EMU
+#define F3M_SIB_ATTR(DD, NNODE)                                                                                        \
+    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE>),                            \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shsib));
+#else
+#define F3M_SIB_ATTR(DD, NNODE)
+#endif
+#define F3M_SIB(DD, NNODE)                                                                                             \
+    if (d == DD && ns.n[0] == NNODE) {                                                                                 \
+        F3M_SIB_ATTR(DD, NNODE)                                                                                        \
+        F3M_LAUNCH((m2l_sib_kernel<DD, NNODE>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2, sibGS,   \
+                   nsub, par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom, loc);            \
+    }
+            F3M_SIB(3, 2) F3M_SIB(3, 3) F3M_SIB(3, 4)
+            F3M_SIB(4, 2) F3M_SIB(4, 3) F3M_SIB(4, 4)
+            F3M_SIB(5, 2) F3M_SIB(5, 3) F3M_SIB(5, 4)
+#undef F3M_SIB
+#undef F3M_SIB_ATTR
+        } else if (q64) {
             // table index of the lowest expected offset: one tree: cell offsets of far pairs are -3..3; two
             // trees: centre distances stay below 5 edges, i.e. offsets from ceil(-5 - delta/edge) on, at most
             // 11 distinct values.  (Anything outside is still handled, pair by pair.)

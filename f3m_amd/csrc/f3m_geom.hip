@@ -460,7 +460,9 @@ __global__ void expand_classify_kernel(long long T, const long long *__restrict_
                                        const int *__restrict__ csy, const int *__restrict__ offx,
                                        const int *__restrict__ offy, const float *__restrict__ ctrx,
                                        const float *__restrict__ ctry, int d, ClassifyParams cp,
-                                       int *__restrict__ cand, unsigned char *__restrict__ cls)
+                                       const int *__restrict__ cellx, const int *__restrict__ celly,
+                                       unsigned long long *__restrict__ outliers, int *__restrict__ cand,
+                                       unsigned char *__restrict__ cls)
 {
     long long pos = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (pos >= T) return;
@@ -491,7 +493,23 @@ __global__ void expand_classify_kernel(long long T, const long long *__restrict_
     int size = (offx[bx + 1] - offx[bx]) + (offy[by + 1] - offy[by]);
     cand[2 * pos] = bx;
     cand[2 * pos + 1] = by;
-    cls[pos] = (unsigned char)classify_pair(ctrx + (long long)bx * d, ctry + (long long)by * d, d, size, cp);
+    const int c = classify_pair(ctrx + (long long)bx * d, ctry + (long long)by * d, d, size, cp);
+    cls[pos] = (unsigned char)c;
+    if (c == 1 && cellx != nullptr) {
+        // regular: every offset from twice the parent's cell in -2..3; or a child of a parent two
+        // cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere
+        int nout = 0, nmid = 0, nbad = 0;
+        for (int j = 0; j < d; j++) {
+            int u = celly[(long long)by * d + j] - 2 * (cellx[(long long)bx * d + j] >> 1);
+            if (u < -2 || u > 3) {
+                nout++;
+                if (u < -4 || u > 5) nbad++;
+            } else if (u == 0 || u == 1) {
+                nmid++;
+            }
+        }
+        if (nout > 0 && (nout > 1 || nbad > 0 || nmid != d - 1)) atomicAdd(outliers, 1ull);
+    }
 }
 
 // order-preserving three-way split
@@ -559,7 +577,7 @@ __global__ void split_scatter_kernel(const unsigned char *__restrict__ cls, cons
 
 __global__ void gather3_kernel(const long long *a, const long long *b, const long long *c, long long *out)
 {
-    if (threadIdx.x == 0) { out[0] = *a; out[1] = *b; out[2] = *c; }
+    if (threadIdx.x == 0) { out[0] = *a; out[1] = *b; out[2] = *c; }   // out[3]: outlier counter, already there
 }
 
 __global__ void rowptr_kernel(const int *__restrict__ pairs, long long n, int nbx, int *__restrict__ rowptr)
@@ -615,12 +633,16 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     F3M_REQUIRE(T < (1ll << 40), 22, "candidate list too long (%lld)", T);
     DBuf<int> cand((size_t)T * 2);
     DBuf<unsigned char> cls((size_t)T);
+    DBuf<long long> dtot(4);
+    const bool one_tree = &tx == &ty;
+    F3M_HIP(hipMemsetAsync(dtot.get() + 3, 0, sizeof(long long), s));
     F3M_LAUNCH(expand_classify_kernel, cdiv(T, 256), 256, 0, s, T, B.get(), rowexcl.get(), nk, rowstart.get(),
                keep_prev.pairs.get(), W.get(), px.childstart.get(), py.childstart.get(), lx.off.get(), ly.off.get(),
-               lx.ctr.get(), ly.ctr.get(), d, cp, cand.get(), cls.get());
+               lx.ctr.get(), ly.ctr.get(), d, cp, one_tree ? lx.cell.get() : (const int *)nullptr, ly.cell.get(),
+               reinterpret_cast<unsigned long long *>(dtot.get() + 3), cand.get(), cls.get());
     check_launch("expand_classify");
     long long nblk = (T + kSplitTile - 1) / kSplitTile;
-    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1), dtot(3);
+    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1);
     F3M_LAUNCH(split_count_kernel, nblk, kSplitBlock, 0, s, cls.get(), T, blockcnt.get(), nblk);
     check_launch("split_count");
     exclusive_scan_i64(blockcnt.get(), nblk, off0.get(), s);
@@ -628,8 +650,9 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     exclusive_scan_i64(blockcnt.get() + 2 * nblk, nblk, off2.get(), s);
     F3M_LAUNCH(gather3_kernel, 1, 64, 0, s, off0.get() + nblk, off1.get() + nblk, off2.get() + nblk, dtot.get());
     check_launch("gather3");
-    long long tot[3];
-    d2h(tot, dtot.get(), 3, s);
+    long long tot[4];
+    d2h(tot, dtot.get(), 4, s);
+    out.far.outliers = one_tree ? tot[3] : -1;
     out.small_.n = tot[0];
     out.far.n = tot[1];
     out.keep.n = tot[2];

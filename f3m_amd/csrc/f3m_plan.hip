@@ -230,6 +230,9 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
             L.num_nodes = std::min((int)pow(3, d), prm->nr_of_interpolation);
         keep = &L.keep;
+        if (getenv("F3M_DEBUG"))
+            fprintf(stderr, "level %d: boxes %d far %lld (outliers %lld) small %lld keep %lld\n", k, P->tx.lev[k].nb, L.far.n,
+                    L.far.outliers, L.small_.n, L.keep.n);
     }
     if (P->levels.empty()) {
         P->Xraw.reset((size_t)N * d);

@@ -135,6 +135,24 @@ def test_far_sweeps_with_level_dependent_node_counts(oracle, monkeypatch):
     assert rel_l2(sweeps, eng.apply(b)) < 2e-6
 
 
+@pytest.mark.parametrize("d,n,P,mp", [(3, 3000, 27, 60), (4, 3000, 16, 60), (3, 3000, 8, 30)])
+def test_m2l_forms_agree(monkeypatch, d, n, P, mp):
+    """Three forms of M2L: sibling-group separable (default here), per-box separable, direct
+    (the reference's, F3M_src/1_d_conv.cu:741-817).  Same sums up to rounding."""
+    rng = np.random.default_rng(3)
+    X = rng.random((n, d), dtype=f32)
+    b = rng.standard_normal((n, 1)).astype(f32)
+    eng = ee.Plan(X, None, ls=0.6, min_points=mp, nr_of_interpolation=P, small_field_points=P + 10)
+    assert any(eng.level_sizes(k)["nfar"] for k in range(1, eng.depth + 1))
+    grouped = eng.apply(b)
+    monkeypatch.setenv("F3M_M2L", "separable")
+    per_box = eng.apply(b)
+    monkeypatch.setenv("F3M_M2L", "direct")
+    direct = eng.apply(b)
+    assert 0 < rel_l2(grouped, per_box) < 2e-6
+    assert rel_l2(grouped, direct) < 3e-6
+
+
 def test_mfma_near_field(oracle, monkeypatch):
     monkeypatch.setenv("F3M_NEAR", "mfma")
     rng = np.random.default_rng(5)

@@ -40,6 +40,9 @@ def clouds(name, rng):
     if name == "uniform5":
         return rng.random((60000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=32, min_points=100,
                                                               small_field_points=40)
+    if name == "uniform5_243":       # config 4: 3^5 nodes per box
+        return rng.random((200000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=243, min_points=1000,
+                                                               small_field_points=300)
     if name == "uniform2":
         return rng.random((80000, 2), dtype=f32), None, dict(ls=0.2)
     if name == "uniform1":
@@ -136,6 +139,49 @@ def test_product_error_vs_fp64_exact(eng, oracle, name):
     assert err <= 1.5 * err_oracle + 1e-7                # no worse than 1.5x the reference algorithm
     # north-star tolerance, wherever the reference algorithm itself reaches it at these parameters
     assert err <= 1e-3 or err_oracle > 1e-3 / 1.5, (err, err_oracle)
+
+
+@pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform3_varcomp"])
+def test_m2l_forms_agree(eng, monkeypatch, name):
+    """Sibling-group separable M2L (default for one tree, d >= 3) against the per-box separable form
+    and the direct form of the reference (F3M_src/1_d_conv.cu:741-817): same sums up to rounding."""
+    print("case m2l forms", name, flush=True)
+    rng = np.random.default_rng(14)
+    X, Y, prm = clouds(name, rng)
+    b = rng.standard_normal((X.shape[0], 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, **prm)
+    assert sum(plan.level_sizes(k)["nfar"] for k in range(1, plan.depth + 1)) > 0
+    grouped = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_M2L", "separable")
+    per_box = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_M2L", "direct")
+    direct = plan.apply(dev(b)).cpu().numpy()
+    assert rel_l2(grouped, per_box) < 2e-6
+    assert rel_l2(grouped, direct) < 5e-6
+
+
+def test_m2l_children_of_parent_pairs_kept_on_the_far_threshold(eng, monkeypatch):
+    """A parent pair two cells apart along one axis is exactly 2 edges away; fp32 rounding of the centres
+    decides whether the reference's predicate (F3M_src/1_d_conv.cu:936-941) calls it far.  Where it is
+    kept, its children are far pairs with cell offsets beyond the usual 6^d block; the sibling-group M2L
+    handles them through a table of their own."""
+    rng = np.random.default_rng(0)
+    sc, sh = rng.random() * 5 + 0.1, rng.standard_normal() * 3
+    X = (rng.random((45000, 3)) * sc + sh).astype(f32)
+    b = rng.standard_normal((45000, 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, ls=0.6 * sc, min_points=12, nr_of_interpolation=8, small_field_points=4)
+    beyond = 0
+    for k in range(3, plan.depth + 1):
+        L = plan.level(k)
+        cells = np.rint((L["cx"] - X.min(0)) / float(L["edge"]) - 0.5).astype(int)
+        if len(L["far"]):
+            u = cells[L["far"][:, 1]] - 2 * (cells[L["far"][:, 0]] >> 1)
+            beyond += int(((u < -2) | (u > 3)).any(1).sum())
+    assert beyond > 0                                  # the case is present in this cloud
+    grouped = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_M2L", "separable")
+    per_box = plan.apply(dev(b)).cpu().numpy()
+    assert 0 < rel_l2(grouped, per_box) < 2e-6
 
 
 @pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform5", "uniform3_varcomp"])
