@@ -22,23 +22,24 @@ PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak
 NEAR_TRAFFIC_BYTES = 5.685e9
 
 
-def cpu_baseline(X, b, ls, budget_s=15.0):
+def cpu_baseline(X, Y, b, ls, budget_s=15.0):
     """Exact tiled PyTorch product on the host cores for a bounded number of target rows against all
     sources (the checker's code, timed only here)."""
     import torch
     from oracle import f3m_oracle as fo
     Xc, bc = X.cpu(), b.cpu()
+    Yc = Xc if Y is None else Y.cpu()
     rows = 64
     t0 = time.perf_counter()
-    fo.exact_tiled_torch(Xc[:rows], Xc, bc, ls, row_tile=rows, col_tile=1 << 18)
+    fo.exact_tiled_torch(Xc[:rows], Yc, bc, ls, row_tile=rows, col_tile=1 << 18)
     t1 = time.perf_counter() - t0
     rows2 = int(max(64, min(20000, rows * budget_s / max(t1, 1e-3)))) // 64 * 64
     t0 = time.perf_counter()
-    fo.exact_tiled_torch(Xc[:rows2], Xc, bc, ls, row_tile=min(rows2, 256), col_tile=1 << 18)
+    fo.exact_tiled_torch(Xc[:rows2], Yc, bc, ls, row_tile=min(rows2, 256), col_tile=1 << 18)
     t2 = time.perf_counter() - t0
     return {"value": rows2 / t2, "unit": "points/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": "%d target rows x all %d sources, exact tiled torch fp32, %.1f s; implied full product %.0f s"
-                      % (rows2, Xc.shape[0], t2, Xc.shape[0] / (rows2 / t2)),
+                      % (rows2, Yc.shape[0], t2, Xc.shape[0] / (rows2 / t2)),
             "host_cpu_count": os.cpu_count()}
 
 
@@ -49,7 +50,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--n", type=int, default=10_000_000)
     ap.add_argument("--d", type=int, default=3)
-    ap.add_argument("--dist", default="uniform", choices=["uniform", "normal"])
+    ap.add_argument("--dist", default="uniform", choices=["uniform", "normal", "clustered"],
+                    help="clustered = BASELINE config 3: X from 50 anisotropic Gaussians, Y (n/10 points) uniform over "
+                         "X's bounding box, two trees")
     ap.add_argument("--ls", type=float, default=1.0)
     ap.add_argument("--nodes", type=int, default=64)
     ap.add_argument("--subsample", type=int, default=100_000)
@@ -71,8 +74,19 @@ def main():
     torch.cuda.set_device(0)
     g = torch.Generator().manual_seed(1)
     N, d = args.n, args.d
-    X = (torch.rand(N, d, generator=g) if args.dist == "uniform" else torch.randn(N, d, generator=g)).cuda()
-    b = torch.randn(N, 1, generator=g).cuda()
+    Y = None
+    if args.dist == "clustered":
+        mu, sd = 10 * torch.rand(50, d, generator=g), 0.05 + 0.45 * torch.rand(50, d, generator=g)
+        comp = torch.arange(N) % 50
+        X = (mu[comp] + sd[comp] * torch.randn(N, d, generator=g)).cuda()
+        lo, hi = X.min(0).values.cpu(), X.max(0).values.cpu()
+        Y = (lo + (hi - lo) * torch.rand(N // 10, d, generator=g)).cuda()
+        dist_name = "X: 50 anisotropic Gaussians, Y: %d uniform over the bounding box" % (N // 10)
+    else:
+        X = (torch.rand(N, d, generator=g) if args.dist == "uniform" else torch.randn(N, d, generator=g)).cuda()
+        dist_name = "uniform [0,1]^%d" % d if args.dist == "uniform" else "N(0,I)"
+    M = N if Y is None else Y.shape[0]
+    b = torch.randn(M, 1, generator=g).cuda()
     prm = dict(ls=args.ls, min_points=1000, nr_of_interpolation=args.nodes, small_field_points=1000)
 
     if args.copy_probe:
@@ -85,12 +99,12 @@ def main():
 
     engine.set_timing(True)
     for _ in range(args.warmup):
-        out = engine.kmvm(X, None, b, **prm)
+        out = engine.kmvm(X, Y, b, **prm)
     torch.cuda.synchronize()
     near_t, near_n, stage = 0.0, 0, {}
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        out = engine.kmvm(X, None, b, **prm)
+        out = engine.kmvm(X, Y, b, **prm)
         tm = engine.get_timing()
         near_t += tm["near"][0]
         near_n += tm["near"][1]
@@ -100,7 +114,7 @@ def main():
     dt = time.perf_counter() - t0
     ms = dt / args.steps * 1e3
 
-    plan = engine.Plan(X, None, **prm)
+    plan = engine.Plan(X, Y, **prm)
     work = plan.work()
     depth = plan.depth
     plan.close()
@@ -121,8 +135,9 @@ def main():
         "value": N / (dt / args.steps), "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
-        "config": {"workload": "3D Gaussian KMVM X=Y, N=%d %s, b~N(0,1) (N,1), ls=%g, %d nodes/box, cutoff 1000 "
-                               "(BASELINE.json configs[1])" % (N, "uniform [0,1]^%d" % d if args.dist == "uniform" else "N(0,I)", args.ls, args.nodes),
+        "config": {"workload": "%dD Gaussian KMVM %s, N=%d %s, b~N(0,1) (%d,1), ls=%g, %d nodes/box, cutoff 1000 "
+                               "(BASELINE.json configs[%d])" % (d, "X=Y" if Y is None else "X!=Y", N, dist_name, M, args.ls,
+                                                               args.nodes, 2 if Y is not None else (1 if d == 3 else 3)),
                    "N": N, "d": d, "ls": args.ls, "nodes": args.nodes, "tree_depth": depth},
         "roofline": roofline,
         "stage_ms_per_step": {k: v / args.steps * 1e3 for k, v in stage.items()},
@@ -130,12 +145,12 @@ def main():
     }
     if not args.no_accuracy:
         rows = torch.from_numpy(np.random.default_rng(1).choice(N, min(args.subsample, N), replace=False)).cuda()
-        exact = engine.exact_f64(X[rows].double(), X.double(), b.double(), args.ls)
+        exact = engine.exact_f64(X[rows].double(), (X if Y is None else Y).double(), b.double(), args.ls)
         diff = (out[rows].double() - exact)
         res["rel_l2_error"] = float(diff.norm() / exact.norm())
         res["rel_l2_rows"] = int(rows.numel())
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(X, b, args.ls)
+        res["cpu_baseline"] = cpu_baseline(X, Y, b, args.ls)
     print(json.dumps(res))
 
 

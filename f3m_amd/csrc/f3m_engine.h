@@ -35,7 +35,8 @@ struct Tree {
     Geo geo;
     long long n = 0;
     DBuf<float> pts;     // d*n, dimension-major, Morton-sorted
-    DBuf<uint32_t> keys; // n sorted keys
+    DBuf<uint32_t> keys; // n keys, sorted by their bits [sorted_from, d*L)
+    int sorted_from = 0;
     DBuf<int> perm;      // sorted position -> original row
     std::vector<TreeLevel> lev;   // lev[0] is the root
 };
@@ -70,7 +71,10 @@ void timer_end(hipStream_t s);
 
 // --- f3m_geom.hip ---
 void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s);
+// keys, order (perm) and the root level; the coordinates are gathered by gather_tree_points once
+// every division is done (divisions may still refine the order inside the boxes)
 void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s);
+void gather_tree_points(Tree &t, const float *X, hipStream_t s);
 // adds lev[k] from lev[k-1]; returns false (and adds nothing) if the key depth is exhausted
 bool divide_tree(Tree &t, hipStream_t s);
 void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,

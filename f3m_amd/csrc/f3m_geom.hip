@@ -234,14 +234,15 @@ __global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__rest
     }
 }
 
-static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int bits, hipStream_t s)
+// stable sort by key bits [from, bits), 8 bits per pass
+static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int from, int bits, hipStream_t s)
 {
     int nblk = (int)cdiv(n, kSortTile);
     DBuf<uint32_t> keys2((size_t)n);
     DBuf<int> idx2((size_t)n);
     DBuf<int> hist((size_t)256 * nblk);
     DBuf<int> base((size_t)256 * nblk + 1);
-    for (int shift = 0; shift < bits; shift += 8) {
+    for (int shift = from; shift < bits; shift += 8) {
         F3M_LAUNCH(sort_hist_kernel, nblk, kWave, 0, s, keys.get(), n, shift, hist.get(), nblk);
         check_launch("sort_hist");
         exclusive_scan_i32(hist.get(), (long long)256 * nblk, base.get(), s);
@@ -274,9 +275,10 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     t.perm.reset((size_t)n);
     F3M_LAUNCH(morton_kernel, cdiv(n, 256), 256, 0, s, X, n, geo, t.keys.get(), t.perm.get());
     check_launch("morton");
-    radix_sort(t.keys, t.perm, n, geo.d * geo.L, s);
-    t.pts.reset((size_t)n * geo.d);
-    gather_points(X, t.perm.get(), n, geo.d, t.pts.get(), s);
+    // Only the leading 16 key bits are sorted at first: a division at depth k looks at the leading d*k
+    // bits, and most trees stop before d*k exceeds 16.  divide_tree sorts further bits when it gets there.
+    t.sorted_from = std::max(0, geo.d * geo.L - 16);
+    radix_sort(t.keys, t.perm, n, t.sorted_from, geo.d * geo.L, s);
     // root level (F3M_src/n_tree.cu:86-95)
     t.lev.clear();
     t.lev.reserve(40);
@@ -292,6 +294,12 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     r.cell.reset(geo.d);
     F3M_LAUNCH(root_level_kernel, 1, 64, 0, s, geo, (int)n, r.off.get(), r.prefix.get(), r.ctr.get(), r.cell.get());
     check_launch("root_level");
+}
+
+void gather_tree_points(Tree &t, const float *X, hipStream_t s)
+{
+    t.pts.reset((size_t)t.n * t.geo.d);
+    gather_points(X, t.perm.get(), t.n, t.geo.d, t.pts.get(), s);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -358,11 +366,17 @@ bool divide_tree(Tree &t, hipStream_t s)
     const int d = t.geo.d;
     const int k = (int)t.lev.size();   // depth being built
     if (k > t.geo.L) return false;
+    int shift = d * (t.geo.L - k);
+    if (shift < t.sorted_from) {
+        // the points are grouped by the boxes built so far whatever the order inside a box, so the
+        // offsets of those levels stay valid when the order is refined
+        t.sorted_from = std::max(0, std::min(shift, t.sorted_from - 8));
+        radix_sort(t.keys, t.perm, t.n, t.sorted_from, d * t.geo.L, s);
+    }
     TreeLevel &prev = t.lev[k - 1];
     long long ncand = (long long)prev.nb << d;
     F3M_REQUIRE(ncand < (1ll << 31) - 2, 20, "too many candidate boxes at depth %d (%lld)", k, ncand);
     DBuf<int> natpos((size_t)ncand + 1), flag((size_t)ncand), cid((size_t)ncand + 1), stats(2);
-    int shift = d * (t.geo.L - k);
     F3M_LAUNCH(child_bounds_kernel, cdiv(ncand + 1, 256), 256, 0, s, t.keys.get(), prev.prefix.get(), prev.off.get(), ncand,
                d, shift, t.n, natpos.get());
     check_launch("child_bounds");
@@ -398,38 +412,6 @@ bool divide_tree(Tree &t, hipStream_t s)
 // Children of a keep pair (x,y) are enumerated in the reference's order (x, child of x, y, child of
 // y); only non-empty children exist here, so the filter step is implicit.
 
-__global__ void keep_rows_kernel(const int *__restrict__ pairs, long long nk, const int *__restrict__ csy,
-                                 long long *__restrict__ wy, int *__restrict__ rowflag)
-{
-    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= nk) return;
-    int y = pairs[2 * t + 1];
-    wy[t] = csy[y + 1] - csy[y];
-    rowflag[t] = (t == 0 || pairs[2 * t] != pairs[2 * (t - 1)]) ? 1 : 0;
-}
-
-__global__ void row_starts_kernel(const int *__restrict__ rowflag, const int *__restrict__ rowexcl, long long nk,
-                                  int *__restrict__ rowstart)
-{
-    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t > nk) return;
-    if (t == nk) { rowstart[rowexcl[nk]] = (int)nk; return; }
-    if (rowflag[t]) rowstart[rowexcl[t]] = (int)t;
-}
-
-__global__ void row_cand_kernel(const int *__restrict__ rowstart, const int *__restrict__ rowexcl, long long nk,
-                                const int *__restrict__ pairs, const int *__restrict__ csx, const long long *__restrict__ W,
-                                long long *__restrict__ rowcand)
-{
-    long long r = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= nk) return;
-    int nrows = rowexcl[nk];
-    if (r >= nrows) { rowcand[r] = 0; return; }
-    int t0 = rowstart[r], t1 = rowstart[r + 1];
-    int x = pairs[2 * (long long)t0];
-    rowcand[r] = (long long)(csx[x + 1] - csx[x]) * (W[t1] - W[t0]);
-}
-
 // 0 small, 1 far, 2 keep, 3 dropped (F3M_src/1_d_conv.cu:927-952 and :983-1026)
 __device__ inline int classify_pair(const float *__restrict__ cx, const float *__restrict__ cy, int d, int size,
                                     const ClassifyParams &cp)
@@ -454,130 +436,99 @@ __device__ inline int classify_pair(const float *__restrict__ cx, const float *_
     return 2;
 }
 
-__global__ void expand_classify_kernel(long long T, const long long *__restrict__ B, const int *__restrict__ rowexcl,
-                                       long long nk, const int *__restrict__ rowstart, const int *__restrict__ pairs,
-                                       const long long *__restrict__ W, const int *__restrict__ csx,
-                                       const int *__restrict__ csy, const int *__restrict__ offx,
-                                       const int *__restrict__ offy, const float *__restrict__ ctrx,
-                                       const float *__restrict__ ctry, int d, ClassifyParams cp,
-                                       const int *__restrict__ cellx, const int *__restrict__ celly,
-                                       unsigned long long *__restrict__ outliers, int *__restrict__ cand,
-                                       unsigned char *__restrict__ cls)
+// One wavefront per box bx of depth k.  Its candidates are the children of the keep partners of its
+// parent; lane l takes partner t0 + l (then t0 + 64 + l, ...) and walks that partner's children, so
+// candidates are met in the order (partner, child) = increasing y box, the order of the reference.
+// WRITE = false counts the three classes per box; WRITE = true recomputes the classes and writes the
+// pairs at the offsets that the scan of those counts gave (which are also the row pointers).
+constexpr int kListWaves = 4;   // wavefronts per workgroup
+
+template <bool WRITE>
+__global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
+    int nbx, const int *__restrict__ csx, int nbx_prev, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
+    const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
+    const float *__restrict__ ctrx, const float *__restrict__ ctry, int d, ClassifyParams cp,
+    const int *__restrict__ cellx, const int *__restrict__ celly, unsigned long long *__restrict__ outliers,
+    long long *__restrict__ cnt /* 3 arrays of nbx+1 */, const long long *__restrict__ pos /* 3 arrays of nbx+1 */,
+    int *__restrict__ out_small, int *__restrict__ out_far, int *__restrict__ out_keep, int *__restrict__ rp_small,
+    int *__restrict__ rp_far, int *__restrict__ rp_keep)
 {
-    long long pos = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (pos >= T) return;
-    int nrows = rowexcl[nk];
-    if (pos >= B[nrows]) { cls[pos] = 3; return; }   // T may be an upper bound of the candidate count
-    // last row r with B[r] <= pos
-    int lo = 0, hi = nrows;
+    const int lane = threadIdx.x & 63;
+    const int bx = blockIdx.x * kListWaves + (threadIdx.x >> 6);
+    if (bx > nbx) return;
+    const long long stride = (long long)nbx + 1;
+    if (bx == nbx) {                               // the closing entry of the row pointers
+        if (WRITE && lane == 0) {
+            rp_small[bx] = (int)pos[bx]; rp_far[bx] = (int)pos[stride + bx]; rp_keep[bx] = (int)pos[2 * stride + bx];
+        }
+        return;
+    }
+    // parent of bx: last x with csx[x] <= bx
+    int lo = 0, hi = nbx_prev;
     while (hi - lo > 1) {
         int mid = lo + ((hi - lo) >> 1);
-        if (B[mid] <= pos) lo = mid; else hi = mid;
+        if (csx[mid] <= bx) lo = mid; else hi = mid;
     }
-    int r = lo;
-    long long rem = pos - B[r];
-    int t0 = rowstart[r], t1 = rowstart[r + 1];
-    long long w0 = W[t0];
-    long long R = W[t1] - w0;
-    int ci = (int)(rem / R);
-    long long rem2 = rem - (long long)ci * R;
-    int a = t0, b = t1;
-    while (b - a > 1) {
-        int mid = a + ((b - a) >> 1);
-        if (W[mid] - w0 <= rem2) a = mid; else b = mid;
+    const int x = lo;
+    const int t0 = keep_rowptr[x], t1 = keep_rowptr[x + 1];
+    const int nx = offx[bx + 1] - offx[bx];
+    float cx[kMaxD];
+    for (int j = 0; j < d; j++) cx[j] = ctrx[(long long)bx * d + j];
+    long long base0 = 0, base1 = 0, base2 = 0;
+    if (WRITE) {
+        base0 = pos[bx]; base1 = pos[stride + bx]; base2 = pos[2 * stride + bx];
+        if (lane == 0) { rp_small[bx] = (int)base0; rp_far[bx] = (int)base1; rp_keep[bx] = (int)base2; }
     }
-    int t = a;
-    int cj = (int)(rem2 - (W[t] - w0));
-    int x = pairs[2 * (long long)t], y = pairs[2 * (long long)t + 1];
-    int bx = csx[x] + ci, by = csy[y] + cj;
-    int size = (offx[bx + 1] - offx[bx]) + (offy[by + 1] - offy[by]);
-    cand[2 * pos] = bx;
-    cand[2 * pos + 1] = by;
-    const int c = classify_pair(ctrx + (long long)bx * d, ctry + (long long)by * d, d, size, cp);
-    cls[pos] = (unsigned char)c;
-    if (c == 1 && cellx != nullptr) {
-        // regular: every offset from twice the parent's cell in -2..3; or a child of a parent two
-        // cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere
-        int nout = 0, nmid = 0, nbad = 0;
-        for (int j = 0; j < d; j++) {
-            int u = celly[(long long)by * d + j] - 2 * (cellx[(long long)bx * d + j] >> 1);
-            if (u < -2 || u > 3) {
-                nout++;
-                if (u < -4 || u > 5) nbad++;
-            } else if (u == 0 || u == 1) {
-                nmid++;
+    long long c0 = 0, c1 = 0, c2 = 0;              // candidates of each class met so far (uniform)
+    const int nchild = 1 << d;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    for (int tb = t0; tb < t1; tb += 64) {
+        // lane l holds the child range of partner tb + l; then the 64 x 2^d (partner, child) slots are
+        // classified 64 at a time, lane = slot, which keeps the order (partner, child)
+        int y0 = 0, y1 = 0;
+        if (tb + lane < t1) { const int y = keep_pairs[2 * (long long)(tb + lane) + 1]; y0 = csy[y]; y1 = csy[y + 1]; }
+        const int nslots = min(64, t1 - tb) << d;
+#pragma unroll 2
+        for (int s0 = 0; s0 < nslots; s0 += 64) {
+            const int slot = s0 + lane;
+            const int p = slot >> d, cj = slot & (nchild - 1);
+            const int by = wave_shfl_i(y0, p) + cj;
+            const bool there = by < wave_shfl_i(y1, p);
+            int c = 3;
+            if (there) {
+                const int size = nx + (offy[by + 1] - offy[by]);
+                c = classify_pair(cx, ctry + (long long)by * d, d, size, cp);
+                if (!WRITE && c == 1 && cellx != nullptr) {
+                    // regular: every offset from twice the parent's cell in -2..3; or a child of a parent two
+                    // cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere
+                    int nout = 0, nmid = 0, nbad = 0;
+                    for (int j = 0; j < d; j++) {
+                        int u = celly[(long long)by * d + j] - 2 * (cellx[(long long)bx * d + j] >> 1);
+                        if (u < -2 || u > 3) {
+                            nout++;
+                            if (u < -4 || u > 5) nbad++;
+                        } else if (u == 0 || u == 1) {
+                            nmid++;
+                        }
+                    }
+                    if (nout > 0 && (nout > 1 || nbad > 0 || nmid != d - 1)) atomicAdd(outliers, 1ull);
+                }
             }
-        }
-        if (nout > 0 && (nout > 1 || nbad > 0 || nmid != d - 1)) atomicAdd(outliers, 1ull);
-    }
-}
-
-// order-preserving three-way split
-constexpr int kSplitBlock = 256;
-constexpr int kSplitItems = 4;
-constexpr int kSplitTile = kSplitBlock * kSplitItems;
-
-__global__ void split_count_kernel(const unsigned char *__restrict__ cls, long long T, long long *__restrict__ blockcnt,
-                                   long long nblk)
-{
-    __shared__ int cnt[3];
-    if (threadIdx.x < 3) cnt[threadIdx.x] = 0;
-    __syncthreads();
-    long long base = (long long)blockIdx.x * kSplitTile + (long long)threadIdx.x * kSplitItems;
-    int c0 = 0, c1 = 0, c2 = 0;
-    for (int e = 0; e < kSplitItems; e++) {
-        long long i = base + e;
-        if (i < T) {
-            int c = cls[i];
-            c0 += c == 0; c1 += c == 1; c2 += c == 2;
+            const unsigned long long m0 = wave_ballot(c == 0), m1 = wave_ballot(c == 1), m2 = wave_ballot(c == 2);
+            if (WRITE) {
+                if (c == 0) { const long long q = base0 + c0 + __popcll(m0 & below); out_small[2 * q] = bx; out_small[2 * q + 1] = by; }
+                else if (c == 1) { const long long q = base1 + c1 + __popcll(m1 & below); out_far[2 * q] = bx; out_far[2 * q + 1] = by; }
+                else if (c == 2) { const long long q = base2 + c2 + __popcll(m2 & below); out_keep[2 * q] = bx; out_keep[2 * q + 1] = by; }
+            }
+            c0 += __popcll(m0); c1 += __popcll(m1); c2 += __popcll(m2);
         }
     }
-    if (c0) atomicAdd(&cnt[0], c0);
-    if (c1) atomicAdd(&cnt[1], c1);
-    if (c2) atomicAdd(&cnt[2], c2);
-    __syncthreads();
-    if (threadIdx.x < 3) blockcnt[(long long)threadIdx.x * nblk + blockIdx.x] = cnt[threadIdx.x];
+    if (!WRITE && lane == 0) { cnt[bx] = c0; cnt[stride + bx] = c1; cnt[2 * stride + bx] = c2; }
 }
 
-__global__ void split_scatter_kernel(const unsigned char *__restrict__ cls, const int *__restrict__ cand, long long T,
-                                     const long long *__restrict__ off0, const long long *__restrict__ off1,
-                                     const long long *__restrict__ off2, int *__restrict__ out_small,
-                                     int *__restrict__ out_far, int *__restrict__ out_keep)
+__global__ void list_totals_kernel(const long long *__restrict__ pos, long long stride, long long *__restrict__ out)
 {
-    // per-thread class counts packed 3 x 21 bits, scanned across the block
-    __shared__ unsigned long long sh[kSplitBlock];
-    const int tid = threadIdx.x;
-    long long base = (long long)blockIdx.x * kSplitTile + (long long)tid * kSplitItems;
-    int c[kSplitItems];
-    unsigned long long mine = 0;
-    for (int e = 0; e < kSplitItems; e++) {
-        long long i = base + e;
-        c[e] = (i < T) ? (int)cls[i] : 3;
-        if (c[e] < 3) mine += 1ull << (21 * c[e]);
-    }
-    sh[tid] = mine;
-    __syncthreads();
-    for (int off = 1; off < kSplitBlock; off <<= 1) {
-        unsigned long long t = (tid >= off) ? sh[tid - off] : 0ull;
-        __syncthreads();
-        sh[tid] += t;
-        __syncthreads();
-    }
-    unsigned long long excl = sh[tid] - mine;
-    long long p0 = off0[blockIdx.x] + (long long)(excl & 0x1fffff);
-    long long p1 = off1[blockIdx.x] + (long long)((excl >> 21) & 0x1fffff);
-    long long p2 = off2[blockIdx.x] + (long long)((excl >> 42) & 0x1fffff);
-    for (int e = 0; e < kSplitItems; e++) {
-        long long i = base + e;
-        if (c[e] == 0) { out_small[2 * p0] = cand[2 * i]; out_small[2 * p0 + 1] = cand[2 * i + 1]; p0++; }
-        else if (c[e] == 1) { out_far[2 * p1] = cand[2 * i]; out_far[2 * p1 + 1] = cand[2 * i + 1]; p1++; }
-        else if (c[e] == 2) { out_keep[2 * p2] = cand[2 * i]; out_keep[2 * p2 + 1] = cand[2 * i + 1]; p2++; }
-    }
-}
-
-__global__ void gather3_kernel(const long long *a, const long long *b, const long long *c, long long *out)
-{
-    if (threadIdx.x == 0) { out[0] = *a; out[1] = *b; out[2] = *c; }   // out[3]: outlier counter, already there
+    if (threadIdx.x < 3) out[threadIdx.x] = pos[threadIdx.x * stride + stride - 1];   // out[3]: outlier counter
 }
 
 __global__ void rowptr_kernel(const int *__restrict__ pairs, long long n, int nbx, int *__restrict__ rowptr)
@@ -603,55 +554,31 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                   PlanLevel &out, hipStream_t s)
 {
     const int d = tx.geo.d;
-    const long long nk = keep_prev.n;
     const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
     out.far.n = out.small_.n = out.keep.n = 0;
-    if (nk == 0) return;
-    F3M_REQUIRE(nk < (1ll << 31) - 2, 21, "keep list too long (%lld)", nk);
-    DBuf<long long> wy((size_t)nk), W((size_t)nk + 1), rowcand((size_t)nk), B((size_t)nk + 1);
-    DBuf<int> rowflag((size_t)nk), rowexcl((size_t)nk + 1), rowstart((size_t)nk + 1);
-    F3M_LAUNCH(keep_rows_kernel, cdiv(nk, 256), 256, 0, s, keep_prev.pairs.get(), nk, py.childstart.get(), wy.get(),
-               rowflag.get());
-    check_launch("keep_rows");
-    exclusive_scan_i64(wy.get(), nk, W.get(), s);
-    exclusive_scan_i32(rowflag.get(), nk, rowexcl.get(), s);
-    F3M_LAUNCH(row_starts_kernel, cdiv(nk + 1, 256), 256, 0, s, rowflag.get(), rowexcl.get(), nk, rowstart.get());
-    check_launch("row_starts");
-    F3M_LAUNCH(row_cand_kernel, cdiv(nk, 256), 256, 0, s, rowstart.get(), rowexcl.get(), nk, keep_prev.pairs.get(),
-               px.childstart.get(), W.get(), rowcand.get());
-    check_launch("row_cand");
-    exclusive_scan_i64(rowcand.get(), nk, B.get(), s);
-    // Candidate storage: every keep pair has at most 4^d child pairs.  When that bound is affordable
-    // the exact count is not fetched first (one host round-trip less per level).
-    const long long p2 = 1ll << (2 * d);
-    long long T = nk * p2;
-    if (T > (1ll << 28)) {
-        d2h(&T, B.get() + nk, 1, s);
-        if (T == 0) return;
-    }
-    F3M_REQUIRE(T < (1ll << 40), 22, "candidate list too long (%lld)", T);
-    DBuf<int> cand((size_t)T * 2);
-    DBuf<unsigned char> cls((size_t)T);
-    DBuf<long long> dtot(4);
+    if (keep_prev.n == 0) return;
+    F3M_REQUIRE(keep_prev.n < (1ll << 31) - 2, 21, "keep list too long (%lld)", keep_prev.n);
+    F3M_REQUIRE((1 << d) < (1 << 21), 21, "too many children per box");
     const bool one_tree = &tx == &ty;
+    const int nbx = lx.nb;
+    const long long stride = (long long)nbx + 1;
+    DBuf<long long> cnt((size_t)(3 * stride)), pos((size_t)(3 * stride)), dtot(4);
     F3M_HIP(hipMemsetAsync(dtot.get() + 3, 0, sizeof(long long), s));
-    F3M_LAUNCH(expand_classify_kernel, cdiv(T, 256), 256, 0, s, T, B.get(), rowexcl.get(), nk, rowstart.get(),
-               keep_prev.pairs.get(), W.get(), px.childstart.get(), py.childstart.get(), lx.off.get(), ly.off.get(),
-               lx.ctr.get(), ly.ctr.get(), d, cp, one_tree ? lx.cell.get() : (const int *)nullptr, ly.cell.get(),
-               reinterpret_cast<unsigned long long *>(dtot.get() + 3), cand.get(), cls.get());
-    check_launch("expand_classify");
-    long long nblk = (T + kSplitTile - 1) / kSplitTile;
-    DBuf<long long> blockcnt((size_t)3 * nblk), off0((size_t)nblk + 1), off1((size_t)nblk + 1), off2((size_t)nblk + 1);
-    F3M_LAUNCH(split_count_kernel, nblk, kSplitBlock, 0, s, cls.get(), T, blockcnt.get(), nblk);
-    check_launch("split_count");
-    exclusive_scan_i64(blockcnt.get(), nblk, off0.get(), s);
-    exclusive_scan_i64(blockcnt.get() + nblk, nblk, off1.get(), s);
-    exclusive_scan_i64(blockcnt.get() + 2 * nblk, nblk, off2.get(), s);
-    F3M_LAUNCH(gather3_kernel, 1, 64, 0, s, off0.get() + nblk, off1.get() + nblk, off2.get() + nblk, dtot.get());
-    check_launch("gather3");
+    const int *cellx = one_tree ? lx.cell.get() : (const int *)nullptr;
+    unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot.get() + 3);
+    const unsigned grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
+    F3M_LAUNCH((lists_kernel<false>), grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+               keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
+               cellx, ly.cell.get(), outl, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
+               (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
+    check_launch("lists_count");
+    for (int c = 0; c < 3; c++) exclusive_scan_i64(cnt.get() + c * stride, nbx, pos.get() + c * stride, s);
+    F3M_LAUNCH(list_totals_kernel, 1, 64, 0, s, pos.get(), stride, dtot.get());
+    check_launch("list_totals");
     long long tot[4];
     d2h(tot, dtot.get(), 4, s);
+    for (int c = 0; c < 3; c++) F3M_REQUIRE(tot[c] < (1ll << 31) - 2, 22, "interaction list too long (%lld)", tot[c]);
     out.far.outliers = one_tree ? tot[3] : -1;
     out.small_.n = tot[0];
     out.far.n = tot[1];
@@ -659,12 +586,15 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     out.small_.pairs.reset((size_t)std::max<long long>(1, tot[0]) * 2);
     out.far.pairs.reset((size_t)std::max<long long>(1, tot[1]) * 2);
     out.keep.pairs.reset((size_t)std::max<long long>(1, tot[2]) * 2);
-    F3M_LAUNCH(split_scatter_kernel, nblk, kSplitBlock, 0, s, cls.get(), cand.get(), T, off0.get(), off1.get(), off2.get(),
-               out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get());
-    check_launch("split_scatter");
-    if (out.small_.n) build_rowptr(out.small_, lx.nb, s);
-    if (out.far.n) build_rowptr(out.far, lx.nb, s);
-    if (out.keep.n) build_rowptr(out.keep, lx.nb, s);
+    out.small_.rowptr.reset((size_t)stride);
+    out.far.rowptr.reset((size_t)stride);
+    out.keep.rowptr.reset((size_t)stride);
+    F3M_LAUNCH((lists_kernel<true>), grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+               keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
+               cellx, ly.cell.get(), outl, (long long *)nullptr, (const long long *)pos.get(), out.small_.pairs.get(),
+               out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(), out.far.rowptr.get(),
+               out.keep.rowptr.get());
+    check_launch("lists_write");
 }
 
 }  // namespace f3m

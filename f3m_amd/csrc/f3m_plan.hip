@@ -213,6 +213,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     root.n = 1;
     root.pairs.reset(2);
     F3M_HIP(hipMemsetAsync(root.pairs.get(), 0, 2 * sizeof(int), s));     // the root pair (0,0)
+    build_rowptr(root, 1, s);
     const PairList *keep = &root;
     P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
     // loop guard of F3M_src/n_tree.cu:1075 (symmetric) and :1099 (two trees)
@@ -233,6 +234,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         if (getenv("F3M_DEBUG"))
             fprintf(stderr, "level %d: boxes %d far %lld (outliers %lld) small %lld keep %lld\n", k, P->tx.lev[k].nb, L.far.n,
                     L.far.outliers, L.small_.n, L.keep.n);
+    }
+    if (need_tree) {
+        gather_tree_points(P->tx, X, s);
+        if (!sym) gather_tree_points(P->ty_, Y, s);
     }
     if (P->levels.empty()) {
         P->Xraw.reset((size_t)N * d);

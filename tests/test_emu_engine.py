@@ -50,6 +50,18 @@ def test_tree_and_lists_bit_exact(oracle, name):
     assert w[0] == ora.work_near_pairs and w[1] == ora.work_far_pairs and w[2] == ora.work_interp_pts
 
 
+def test_deep_tree_bit_exact(oracle):
+    """A tight cluster inside a sparse cloud forces divisions down to the depth cap; the engine sorts
+    further key bits only when a division needs them."""
+    rng = np.random.default_rng(12)
+    X = np.concatenate([rng.normal(0.3, 1e-3, (2000, 3)), rng.random((500, 3))]).astype(f32)
+    eng = ee.Plan(X, None, **PRM)
+    assert eng.depth >= 9
+    assert_plan_matches_oracle(eng, oracle.Plan(X, None, **PRM))
+    b = rng.standard_normal((2500, 1)).astype(f32)
+    assert rel_l2(eng.apply(b), oracle.Plan(X, None, **PRM).apply(b)) < 1e-5
+
+
 def test_var_compression_lists_bit_exact(oracle):
     X, _ = _cloud("uniform3", np.random.default_rng(3))
     prm = dict(PRM, var_compression=True, eff_var_limit=0.3, ls=2.0)
