@@ -19,7 +19,8 @@ class F3MError(RuntimeError):
 SYMBOLS = [
     "f3m_kmvm_f32", "f3m_exact_f32", "f3m_exact_grad_f32", "f3m_exact_f64", "f3m_plan_create", "f3m_plan_apply",
     "f3m_plan_destroy", "f3m_plan_depth", "f3m_plan_symmetric", "f3m_plan_level_sizes", "f3m_plan_level_copy",
-    "f3m_plan_far_level", "f3m_plan_near_level", "f3m_plan_work", "f3m_set_timing", "f3m_get_timing",
+    "f3m_plan_far_level", "f3m_plan_near_level", "f3m_plan_work", "f3m_plan_lookup_boxes", "f3m_hash_slot",
+    "f3m_set_timing", "f3m_get_timing",
     "f3m_last_error", "f3m_release_cache", "f3m_version",
 ]
 
@@ -46,9 +47,12 @@ def bind(lib):
     lib.f3m_get_timing.argtypes = [C.POINTER(dbl), C.POINTER(i)]
     lib.f3m_last_error.restype = C.c_char_p
     lib.f3m_version.restype = C.c_char_p
+    lib.f3m_plan_lookup_boxes.argtypes = [vp, i, i, vp, i64, vp, vp]
+    lib.f3m_hash_slot.argtypes = [C.c_uint32, C.c_uint32]
+    lib.f3m_hash_slot.restype = C.c_uint32
     for name in SYMBOLS:
         fn = getattr(lib, name)
-        if name not in ("f3m_last_error", "f3m_version"):
+        if name not in ("f3m_last_error", "f3m_version", "f3m_hash_slot"):
             fn.restype = C.c_int
     return lib
 

@@ -29,6 +29,9 @@ struct TreeLevel {
     // split-f16 matrix operand of its coordinates relative to its own box centre, scaled by nearops_sc
     mutable DBuf<unsigned char> nearops;
     mutable float nearops_sc = 0.f;
+    // grid key -> box id table of this level (built on first use by lookup_boxes)
+    mutable DBuf<uint32_t> hashtab;      // hashcap pairs (key, value), empty = 0xffffffff
+    mutable uint32_t hashcap = 0;
 };
 
 struct Tree {
@@ -82,6 +85,10 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
 void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
 void build_rowptr(PairList &l, int nbx, hipStream_t s);
+// slot of a key in a table of `capacity` slots (host and device use the same function)
+uint32_t hash_slot_host(uint32_t key, uint32_t capacity);
+// ids[i] = box of depth lev.depth whose integer cell is cells[i*d .. i*d+d), or -1 if that cell is empty
+void lookup_boxes(const Tree &t, const TreeLevel &lev, const int *cells, long long n, int *ids, hipStream_t s);
 
 // --- f3m_field.hip ---
 struct NodeSet {

@@ -407,6 +407,91 @@ bool divide_tree(Tree &t, hipStream_t s)
 }
 
 // ------------------------------------------------------------------------------------------------
+// Grid key -> box id through an open-addressing table in HBM (F3M_src/linearprobing.cu:18-87, used by
+// the reference in box_division_assign_hash, F3M_src/1_d_conv.cu:1127-1191): slot = Murmur3 finaliser
+// of the key modulo capacity-1, linear probing (slot+1) % (capacity-1), empty = 0xffffffff, which is
+// also the answer for an absent key (-1 as an int).  The engine itself never needs the table -- its
+// keys are sorted and its box ids dense -- but callers that hold cell coordinates (a point that is
+// not part of the plan, a neighbour cell) get the box id the reference's lookup would give.
+
+__host__ __device__ inline uint32_t hash_slot(uint32_t k, uint32_t capacity)
+{
+    k ^= k >> 16;
+    k *= 0x85ebca6bu;
+    k ^= k >> 13;
+    k *= 0xc2b2ae35u;
+    k ^= k >> 16;
+    return k % (capacity - 1u);
+}
+
+uint32_t hash_slot_host(uint32_t key, uint32_t capacity) { return hash_slot(key, capacity); }
+
+// the reference's key of a cell: sum_j g_j (2^k)^(d-1-j), int32 (F3M_src/1_d_conv.cu:1142-1144)
+__device__ inline uint32_t cell_key(const int *__restrict__ cell, int d, int depth)
+{
+    int key = 0;
+    for (int j = 0; j < d; j++) key = (key << depth) + cell[j];   // Horner form of the same sum
+    return (uint32_t)key;
+}
+
+__global__ void hash_insert_kernel(const int *__restrict__ cell, int nb, int d, int depth, uint32_t *__restrict__ table,
+                                   uint32_t capacity)
+{
+    int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nb) return;
+    const uint32_t key = cell_key(cell + (long long)b * d, d, depth);
+    uint32_t slot = hash_slot(key, capacity);
+    for (uint32_t tries = 0; tries < capacity; tries++) {           // bounded: the table is at most half full
+        const uint32_t prev = atomicCAS(&table[2 * (size_t)slot], 0xffffffffu, key);
+        if (prev == 0xffffffffu || prev == key) { table[2 * (size_t)slot + 1] = (uint32_t)b; return; }
+        slot = (slot + 1u) % (capacity - 1u);
+    }
+}
+
+__global__ void hash_lookup_kernel(const int *__restrict__ cells, long long n, int d, int depth,
+                                   const uint32_t *__restrict__ table, uint32_t capacity, int *__restrict__ ids)
+{
+    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int side = 1 << depth;
+    bool inside = true;
+    for (int j = 0; j < d; j++) inside = inside && cells[i * d + j] >= 0 && cells[i * d + j] < side;
+    int id = -1;
+    if (inside) {
+        const uint32_t key = cell_key(cells + i * d, d, depth);
+        uint32_t slot = hash_slot(key, capacity);
+        for (uint32_t tries = 0; tries < capacity; tries++) {
+            const uint32_t k = table[2 * (size_t)slot];
+            if (k == key) { id = (int)table[2 * (size_t)slot + 1]; break; }
+            if (k == 0xffffffffu) break;
+            slot = (slot + 1u) % (capacity - 1u);
+        }
+    }
+    ids[i] = id;
+}
+
+void lookup_boxes(const Tree &t, const TreeLevel &lev, const int *cells, long long n, int *ids, hipStream_t s)
+{
+    const int d = t.geo.d;
+    F3M_REQUIRE(d * lev.depth <= 31, 23, "grid keys of depth %d do not fit in 32 bits", lev.depth);
+    if (lev.hashcap == 0) {
+        // capacity: the power of two that leaves the table at most half full (the reference takes
+        // max(2^20, that), F3M_src/n_tree.cu:113-116)
+        uint32_t cap = 1024;
+        while (cap < 2u * (uint32_t)lev.nb) cap <<= 1;
+        lev.hashtab.reset(2 * (size_t)cap);
+        F3M_HIP(hipMemsetAsync(lev.hashtab.get(), 0xff, sizeof(uint32_t) * 2 * (size_t)cap, s));
+        F3M_LAUNCH(hash_insert_kernel, cdiv(lev.nb, 256), 256, 0, s, lev.cell.get(), lev.nb, d, lev.depth, lev.hashtab.get(),
+                   cap);
+        check_launch("hash_insert");
+        lev.hashcap = cap;
+    }
+    if (n == 0) return;
+    F3M_LAUNCH(hash_lookup_kernel, cdiv(n, 256), 256, 0, s, cells, n, d, lev.depth, lev.hashtab.get(), lev.hashcap, ids);
+    check_launch("hash_lookup");
+}
+
+// ------------------------------------------------------------------------------------------------
 // Interaction lists of depth k from the keep list of depth k-1
 // (F3M_src/n_tree.cu:594-641 expansion, 788-811 filter, 701-787 + F3M_src/1_d_conv.cu:903-1029 classes).
 // Children of a keep pair (x,y) are enumerated in the reference's order (x, child of x, y, child of

@@ -617,6 +617,22 @@ int f3m_plan_work(const f3m_plan *plan, double *w)
     });
 }
 
+int f3m_plan_lookup_boxes(f3m_plan *plan, int level, int tree, const int32_t *cells, int64_t n, int32_t *ids, void *stream)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        F3M_REQUIRE(tree == 0 || tree == 1, 13, "tree must be 0 (X) or 1 (Y)");
+        F3M_REQUIRE(n >= 0, 13, "negative count");
+        hipStream_t s = (hipStream_t)stream;
+        if (n > 0) { check_device_ptr(cells, "cells"); check_device_ptr(ids, "ids"); }
+        const Tree &t = tree == 0 ? plan->tx : *plan->ty;
+        lookup_boxes(t, t.lev[level], cells, n, ids, s);
+        F3M_HIP(hipStreamSynchronize(s));
+    });
+}
+
+uint32_t f3m_hash_slot(uint32_t key, uint32_t capacity) { return capacity > 1 ? hash_slot_host(key, capacity) : 0u; }
+
 int f3m_set_timing(int enabled)
 {
     g_timer.enabled = enabled != 0;

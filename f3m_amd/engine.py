@@ -190,6 +190,18 @@ class Plan:
         capi.check(self._lib, rc)
         return out
 
+    def lookup_boxes(self, level, cells, tree="x"):
+        """Box id at depth `level` of every integer cell in `cells` (n, d) int32 on the GPU; -1 where the
+        cell holds no point (reference: the key -> index hash table, F3M_src/linearprobing.cu:54-87)."""
+        assert cells.is_cuda and cells.dtype == torch.int32 and cells.dim() == 2 and cells.shape[1] == self.d
+        cells = cells.contiguous()
+        ids = torch.empty(cells.shape[0], dtype=torch.int32, device=self.device)
+        with torch.cuda.device(self.device):
+            rc = self._lib.f3m_plan_lookup_boxes(self._h, level, 0 if tree == "x" else 1, _ptr(cells), cells.shape[0],
+                                                 _ptr(ids), _stream())
+        capi.check(self._lib, rc)
+        return ids
+
     def work(self):
         """Work model: point pairs summed exactly, far box pairs, interpolated points, far pairs * P^2."""
         w = (C.c_double * 5)()

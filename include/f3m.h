@@ -92,6 +92,17 @@ int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, in
  * covered by far box pairs (w[0] + w[4] = N*M: every point pair is handled exactly once) */
 int f3m_plan_work(const f3m_plan *plan, double *w);
 
+/* Box lookup by grid cell: ids[i] = compact id, at depth `level`, of the box whose integer cell is
+ * cells[i*d .. i*d+d) (device int32, 0 <= cell < 2^level per dimension), or -1 if no point lies in that
+ * cell.  tree = 0 for the X tree, 1 for the Y tree.  Replaces the key -> index table of
+ * F3M_src/linearprobing.cu:41-87 as box_division_assign_hash uses it (F3M_src/1_d_conv.cu:1127-1191):
+ * same slot function (Murmur3 finaliser modulo capacity-1), same probing, same answer for an absent
+ * key.  The table of a level lives in device memory and is built on the first lookup. */
+int f3m_plan_lookup_boxes(f3m_plan *plan, int level, int tree, const int32_t *cells, int64_t n, int32_t *ids,
+                          void *stream);
+/* slot of `key` in a table of `capacity` slots (host function; hash_2 of F3M_src/linearprobing.cu:18-26) */
+uint32_t f3m_hash_slot(uint32_t key, uint32_t capacity);
+
 /* seconds spent by the last f3m_plan_apply / f3m_kmvm_f32 of this thread in each stage, measured
  * with HIP events on the call's stream when timing is enabled: t[0] plan, t[1] near, t[2] P2M,
  * t[3] M2L, t[4] L2P, t[5] permutations; n[] = kernel launches per stage */

@@ -839,3 +839,61 @@ int fo_m2l_block(int d, int nr_interp, const float *cx, const float *cy, float e
     free(nodes); free(w); free(grid);
     return Pn;
 }
+
+/* ------------------------------------------------------------------------------------------------
+ * Open-addressing key -> value table (F3M_src/linearprobing.cu:18-87).  Slot of a key: Murmur3's 32-bit
+ * finaliser, reduced modulo capacity-1 (hash_2, :18-26); collisions probe (slot+1) % (capacity-1)
+ * (:66,:84); an empty slot holds 0xffffffff in key and value (:47-49), which is also what a lookup of
+ * an absent key returns (:80-83).  table = capacity pairs (key, value).
+ * Pinned by: MurmurHash3_x86_32 of the empty string is fmix32(seed) -> 0x514E28B7 for seed 1 and
+ * 0x81F16F39 for seed 0xffffffff (published test vectors); table semantics against a Python dict. */
+uint32_t fo_hash32(uint32_t k)
+{
+    k ^= k >> 16;
+    k *= 0x85ebca6bu;
+    k ^= k >> 13;
+    k *= 0xc2b2ae35u;
+    k ^= k >> 16;
+    return k;
+}
+
+uint32_t fo_hash_slot(uint32_t key, uint32_t capacity) { return fo_hash32(key) % (capacity - 1u); }
+
+void fo_hash_clear(uint32_t *table, uint32_t capacity) { memset(table, 0xff, sizeof(uint32_t) * 2 * (size_t)capacity); }
+
+void fo_hash_insert(uint32_t *table, uint32_t capacity, uint32_t key, uint32_t value)
+{
+    uint32_t slot = fo_hash_slot(key, capacity);
+    for (;;) {
+        uint32_t prev = table[2 * (size_t)slot];
+        if (prev == 0xffffffffu || prev == key) {
+            table[2 * (size_t)slot] = key;
+            table[2 * (size_t)slot + 1] = value;
+            return;
+        }
+        slot = (slot + 1u) % (capacity - 1u);
+    }
+}
+
+uint32_t fo_hash_lookup(const uint32_t *table, uint32_t capacity, uint32_t key)
+{
+    uint32_t slot = fo_hash_slot(key, capacity);
+    for (;;) {
+        if (table[2 * (size_t)slot] == key) return table[2 * (size_t)slot + 1];
+        if (table[2 * (size_t)slot] == 0xffffffffu) return 0xffffffffu;
+        slot = (slot + 1u) % (capacity - 1u);
+    }
+}
+
+/* grid key of an integer cell at depth k: sum_j g_j (2^k)^(d-1-j), int32 arithmetic
+ * (F3M_src/1_d_conv.cu:1142-1144, stride update F3M_src/n_tree.cu:170) */
+int32_t fo_cell_key(int d, int k, const int32_t *cell)
+{
+    int32_t key = 0;
+    for (int j = 0; j < d; j++) {
+        int32_t mult = 1;
+        for (int l = 0; l < d - 1 - j; l++) mult *= (int32_t)1 << k;
+        key += mult * cell[j];
+    }
+    return key;
+}

@@ -62,6 +62,17 @@ def lib():
         L.fo_exact_f64.argtypes = [C.c_int, dp, C.c_long, dp, C.c_long, dp, C.c_int, C.c_double, dp]
         L.fo_m2l_block.argtypes = [C.c_int, C.c_int, fp, fp, C.c_float, C.c_float, fp]
         L.fo_m2l_block.restype = C.c_int
+        up = C.POINTER(C.c_uint32)
+        L.fo_hash32.argtypes = [C.c_uint32]
+        L.fo_hash32.restype = C.c_uint32
+        L.fo_hash_slot.argtypes = [C.c_uint32, C.c_uint32]
+        L.fo_hash_slot.restype = C.c_uint32
+        L.fo_hash_clear.argtypes = [up, C.c_uint32]
+        L.fo_hash_insert.argtypes = [up, C.c_uint32, C.c_uint32, C.c_uint32]
+        L.fo_hash_lookup.argtypes = [up, C.c_uint32, C.c_uint32]
+        L.fo_hash_lookup.restype = C.c_uint32
+        L.fo_cell_key.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_int32)]
+        L.fo_cell_key.restype = C.c_int32
         _lib = L
     return _lib
 
@@ -273,6 +284,39 @@ def m2l_block(d, nr_interp, cx, cy, edge, lcs):
 # path; this follows the tiling idea of its exact CUDA kernel (F3M_src/1_d_conv.cu:171-214, a
 # block of target rows against successive source tiles) behind benchmark_matmul
 # (experiments/FFM_classes.py:264-323).
+
+def hash32(k):
+    """Murmur3 32-bit finaliser (F3M_src/linearprobing.cu:18-26 before the reduction)."""
+    return int(lib().fo_hash32(int(k) & 0xffffffff))
+
+
+def hash_slot(key, capacity):
+    return int(lib().fo_hash_slot(int(key) & 0xffffffff, int(capacity)))
+
+
+def grid_key(d, k, cell):
+    c = np.ascontiguousarray(np.asarray(cell, np.int32))
+    return int(lib().fo_cell_key(int(d), int(k), c.ctypes.data_as(C.POINTER(C.c_int32))))
+
+
+class HashTable:
+    """Key -> value table of F3M_src/linearprobing.cu:41-87 (capacity pairs of uint32, empty = 0xffffffff)."""
+
+    def __init__(self, capacity):
+        self.capacity = int(capacity)
+        self.table = np.empty(2 * self.capacity, np.uint32)
+        lib().fo_hash_clear(self._p(), self.capacity)
+
+    def _p(self):
+        return self.table.ctypes.data_as(C.POINTER(C.c_uint32))
+
+    def insert(self, key, value):
+        lib().fo_hash_insert(self._p(), self.capacity, int(key) & 0xffffffff, int(value) & 0xffffffff)
+
+    def lookup(self, key):
+        v = int(lib().fo_hash_lookup(self._p(), self.capacity, int(key) & 0xffffffff))
+        return -1 if v == 0xffffffff else v
+
 
 def exact_tiled_torch(X, Y, b, ls, row_tile=2048, col_tile=16384, dtype=None):
     import torch

@@ -77,6 +77,13 @@ class Plan:
         out["edge"] = np.float32(e.value)
         return out
 
+    def lookup_boxes(self, level, cells, tree="x"):
+        cells = np.ascontiguousarray(np.asarray(cells, np.int32))
+        ids = np.empty(cells.shape[0], np.int32)
+        capi.check(lib(), lib().f3m_plan_lookup_boxes(self._h, level, 0 if tree == "x" else 1, _p(cells), cells.shape[0],
+                                                      _p(ids), None))
+        return ids
+
     def level(self, level):
         sz = self.level_sizes(level)
         shapes = {

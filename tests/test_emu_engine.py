@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 
 import emu_engine as ee
+from helpers import box_of_point, cell_coords
 from parity_checks import assert_plan_matches_oracle, rel_l2
 
 f32 = np.float32
@@ -60,6 +61,30 @@ def test_deep_tree_bit_exact(oracle):
     assert_plan_matches_oracle(eng, oracle.Plan(X, None, **PRM))
     b = rng.standard_normal((2500, 1)).astype(f32)
     assert rel_l2(eng.apply(b), oracle.Plan(X, None, **PRM).apply(b)) < 1e-5
+
+
+@pytest.mark.parametrize("name", ["uniform3", "asym3", "normal2"])
+def test_box_lookup_by_cell(oracle, name):
+    """Grid cell -> box id through the engine's open-addressing table: every point's cell (restated in
+    numpy) gives the box that holds the point; cells without points give -1; the slot function is the
+    reference's (F3M_src/linearprobing.cu:18-26)."""
+    X, Y = _cloud(name, np.random.default_rng(21))
+    eng = ee.Plan(X, Y, **PRM)
+    edge0, xmin, ymin = oracle.root(X, Y)
+    for tree, pts, org in (("x", X, xmin), ("y", X if Y is None else Y, xmin if Y is None else ymin)):
+        for k in range(1, eng.depth + 1):
+            L = eng.level(k)
+            cells = cell_coords(pts, org, edge0, k).astype(np.int32)
+            assert np.array_equal(eng.lookup_boxes(k, cells, tree), box_of_point(L, tree))
+            side = 1 << k
+            grid = np.stack(np.meshgrid(*[np.arange(-1, side + 1)] * X.shape[1], indexing="ij"), -1)
+            grid = grid.reshape(-1, X.shape[1])[:: max(1, (side + 2) ** X.shape[1] // 5000)].astype(np.int32)
+            occupied = {tuple(c) for c in cells.tolist()}
+            got = eng.lookup_boxes(k, grid, tree)
+            for c, g in zip(grid.tolist(), got.tolist()):
+                assert (g >= 0) == (tuple(c) in occupied)
+    for key, cap in ((1, 1 << 20), (0xFFFFFFFF, 1024), (123456789, 4096), (0, 2048)):
+        assert ee.lib().f3m_hash_slot(key, cap) == oracle.hash_slot(key, cap)
 
 
 def test_var_compression_lists_bit_exact(oracle):

@@ -75,6 +75,36 @@ def test_box_division_and_lists_bit_exact(eng, oracle, name):
     assert w["near_pairs"] + w["far_point_pairs"] == float(X.shape[0]) * M      # every pair exactly once
 
 
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform5"])
+def test_box_lookup_by_cell(eng, oracle, name):
+    """The HBM key -> index table (reference: F3M_src/linearprobing.cu:18-87): the cell of every point,
+    restated in numpy, must map to the box that holds the point; absent cells map to -1."""
+    import torch
+    from helpers import box_of_point, cell_coords
+    print("case box lookup", name, flush=True)
+    X, Y, prm = clouds(name, np.random.default_rng(7))
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    edge0, xmin, ymin = oracle.root(X, Y)
+    for tree, pts, org in (("x", X, xmin), ("y", X if Y is None else Y, xmin if Y is None else ymin)):
+        for k in range(1, plan.depth + 1):
+            L = plan.level(k)
+            cells = cell_coords(pts, org, edge0, k).astype(np.int32)
+            got = plan.lookup_boxes(k, dev(cells), tree).cpu().numpy()
+            assert np.array_equal(got, box_of_point(L, tree)), (tree, k)
+            shifted = cells + (1 << k)                 # outside the grid: never a box
+            assert (plan.lookup_boxes(k, dev(shifted), tree).cpu().numpy() == -1).all()
+    nb = plan.level_sizes(plan.depth)["nbx"]
+    side = 1 << plan.depth
+    rnd = np.random.default_rng(8).integers(0, side, (20000, X.shape[1])).astype(np.int32)
+    got = plan.lookup_boxes(plan.depth, dev(rnd), "x").cpu().numpy()
+    occupied = {tuple(c) for c in cell_coords(X, xmin, edge0, plan.depth).tolist()}
+    assert all((g >= 0) == (tuple(c) in occupied) for c, g in zip(rnd.tolist(), got.tolist()))
+    assert got.max() < nb
+    lib = eng._lib.get()
+    for key, cap in ((1, 1 << 20), (0xFFFFFFFF, 1024), (123456789, 4096)):
+        assert lib.f3m_hash_slot(key, cap) == oracle.hash_slot(key, cap)
+
+
 @pytest.mark.parametrize("d", [1, 2, 3, 5, 10])
 def test_exact_kernels(eng, oracle, d):
     print("case exact d=%d" % d, flush=True)

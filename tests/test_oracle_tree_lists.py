@@ -183,3 +183,42 @@ def test_var_compression_lists_bruteforce(oracle, ls, eff):
         keep_prev = set(map(tuple, L["keep"].tolist()))
         parent = box
     assert seen_shortcut or ls < 1.0        # smooth kernels must trigger the extra far-field shortcuts
+
+
+# ------------------------------------------------------------------------------------------------
+# key -> value table (F3M_src/linearprobing.cu:18-87)
+
+def test_hash_finaliser_known_answers(oracle):
+    """MurmurHash3_x86_32 of the empty string is its finaliser applied to the seed: the published
+    vectors 0 -> 0, seed 1 -> 0x514E28B7, seed 0xffffffff -> 0x81F16F39."""
+    assert oracle.hash32(0) == 0
+    assert oracle.hash32(1) == 0x514E28B7
+    assert oracle.hash32(0xFFFFFFFF) == 0x81F16F39
+    for key, cap in ((1, 1 << 20), (0xFFFFFFFF, 1024), (123456789, 4096)):
+        assert oracle.hash_slot(key, cap) == oracle.hash32(key) % (cap - 1)      # hash_2: modulo capacity-1
+
+
+def test_hash_table_against_dict(oracle):
+    rng = np.random.default_rng(5)
+    cap = 256
+    keys = rng.choice(1 << 16, 120, replace=False)
+    ref = {}
+    t = oracle.HashTable(cap)
+    for i, k in enumerate(keys.tolist()):
+        t.insert(k, i)
+        ref[k] = i
+    t.insert(int(keys[3]), 999)                       # same key again: value replaced, no second slot
+    ref[int(keys[3])] = 999
+    for k, v in ref.items():
+        assert t.lookup(k) == v
+    absent = [k for k in range(1 << 16, (1 << 16) + 50)]
+    assert all(t.lookup(k) == -1 for k in absent)     # kEmpty = 0xffffffff = -1 as an int
+    used = t.table[0::2] != 0xFFFFFFFF
+    assert used.sum() == len(ref) and not used[cap - 1]    # slots run 0 .. capacity-2 only
+
+
+def test_grid_key_is_the_reference_sum(oracle):
+    # sum_j g_j (2^k)^(d-1-j): dimension 0 most significant (F3M_src/1_d_conv.cu:1142-1144)
+    assert oracle.grid_key(3, 2, [1, 2, 3]) == 1 * 16 + 2 * 4 + 3
+    assert oracle.grid_key(2, 5, [7, 30]) == 7 * 32 + 30
+    assert oracle.grid_key(1, 9, [300]) == 300
