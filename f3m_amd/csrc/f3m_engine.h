@@ -105,8 +105,10 @@ void gather_points(const float *X, const int *perm, long long n, int d, float *p
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
 
+// nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
-                const float *bs, float *outs, float lcs, hipStream_t s);
+                const float *bs, float *outs, float lcs, hipStream_t s, int nc = 1, long long bstride = 0,
+                long long ostride = 0);
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);

@@ -362,12 +362,14 @@ __global__ void near_operands_kernel(const float *__restrict__ ys, long long M, 
 constexpr int kNearWavesPerBlock = 2;
 struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floats at any 4-byte boundary
 
-template <int D, int TPW>
+// NC right-hand sides at once: the exponential of a pair is computed once and multiplies NC weights
+// (columns of bs, bstride apart; results to NC columns of outs, ostride apart).
+template <int D, int TPW, int NC>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
-    float *__restrict__ outs, const int *__restrict__ offx, const int *__restrict__ offy, const float *__restrict__ ctry,
-    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
-    int stripe)
+    long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
+    const int *__restrict__ offy, const float *__restrict__ ctry, const int *__restrict__ pairs,
+    const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc, int stripe)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
@@ -395,9 +397,11 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
 #pragma unroll
         for (int k = 0; k < D; k++) xr[q][k] = (i < x1) ? xs[(long long)k * N + i] : 0.f;
     }
-    float acc[TPW];
+    float acc[TPW][NC];
 #pragma unroll
-    for (int q = 0; q < TPW; q++) acc[q] = 0.f;
+    for (int q = 0; q < TPW; q++)
+#pragma unroll
+        for (int c = 0; c < NC; c++) acc[q][c] = 0.f;
     const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
     // the list is consumed 64 y boxes at a time: every lane fetches the range and centre of one y box,
     // then the wavefront walks through them (one round of memory latency per 64 boxes)
@@ -451,15 +455,21 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
             for (int n = 0; n < NS; n++) a[n] = ops[(long long)(n * 2 + half) * stride + j0 + col];
             // weights of the 16 source rows this lane sees: rows 8g + 4 half + e of the tile (bs is
             // padded by one tile, so the loads stay in bounds; rows past the box get weight zero)
-            float bq[16];
+            float bq[NC][16];
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4u f = *reinterpret_cast<const float4u *>(bs + j0 + 8 * g + 4 * half);
-                bq[4 * g + 0] = f.x; bq[4 * g + 1] = f.y; bq[4 * g + 2] = f.z; bq[4 * g + 3] = f.w;
-            }
+            for (int c = 0; c < NC; c++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const float4u f = *reinterpret_cast<const float4u *>(bs + c * bstride + j0 + 8 * g + 4 * half);
+                    bq[c][4 * g + 0] = f.x; bq[c][4 * g + 1] = f.y; bq[c][4 * g + 2] = f.z; bq[c][4 * g + 3] = f.w;
+                }
             if (j0 + 32 > s1) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) bq[r] = (j0 + 8 * (r / 4) + 4 * half + (r % 4) < s1) ? bq[r] : 0.f;
+                for (int r = 0; r < 16; r++) {
+                    const bool in = j0 + 8 * (r / 4) + 4 * half + (r % 4) < s1;
+#pragma unroll
+                    for (int c = 0; c < NC; c++) bq[c][r] = in ? bq[c][r] : 0.f;
+                }
             }
 #pragma unroll
             for (int q = 0; q < TPW; q++) {
@@ -469,10 +479,12 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
                     for (int r = 0; r < 16; r++) t[r] = 0.f;
 #pragma unroll
                     for (int n = 0; n < NS; n++) t = mfma_32x32x16_f16(a[n], bop[q][n], t);
-                    float sum = acc[q];
 #pragma unroll
-                    for (int r = 0; r < 16; r++) sum = fmaf(fast_exp2(t[r]), bq[r], sum);
-                    acc[q] = sum;
+                    for (int r = 0; r < 16; r++) {
+                        const float e = fast_exp2(t[r]);
+#pragma unroll
+                        for (int c = 0; c < NC; c++) acc[q][c] = fmaf(e, bq[c][r], acc[q][c]);
+                    }
                 }
             }
         }
@@ -480,16 +492,20 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     }
 #pragma unroll
     for (int q = 0; q < TPW; q++) {
-        float total = acc[q] + wave_shfl_xor_f(acc[q], 32);
         const int i = x0 + q * 32 + col;
-        if (half == 0 && i < x1) outs[i] += total;
+#pragma unroll
+        for (int c = 0; c < NC; c++) {
+            float total = acc[q][c] + wave_shfl_xor_f(acc[q][c], 32);
+            if (half == 0 && i < x1) outs[c * ostride + i] += total;
+        }
     }
 }
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
-                const float *bs, float *outs, float lcs, hipStream_t s)
+                const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride)
 {
     if (list.n == 0) return;
+    F3M_REQUIRE(nc == 1 || nc == 4, 34, "near field takes 1 or 4 columns at a time");
     // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to about
     // 2^-22 times the largest term, |x''|^2 <= 30 d (sc edge)^2 (listed targets lie within 5.5 edges per
     // dimension of the source box centre); it is used while that bound stays below 1e-4 (box edge up to
@@ -535,10 +551,16 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_g_kernel<DD, tpw>), ngrid, kNearWavesPerBlock * 64, 0, s,                                    \
-                   tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, outs,              \
-                   lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
-                   lx.nb, sc, stripe);                                                                                \
+        if (nc == 4)                                                                                                  \
+            F3M_LAUNCH((near_g_kernel<DD, tpw, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
+                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       tileoff.get(), lx.nb, sc, stripe);                                                             \
+        else                                                                                                          \
+            F3M_LAUNCH((near_g_kernel<DD, tpw, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
+                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       tileoff.get(), lx.nb, sc, stripe);                                                             \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -550,9 +572,10 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_kernel<DD, T>), ntiles, bd, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n, bs, outs,          \
-                   lx.off.get(), ly.off.get(), lx.ctr.get(), list.pairs.get(), list.rowptr.get(), tileoff.get(),      \
-                   lx.nb, sc);                                                                                        \
+        for (int c = 0; c < nc; c++)                                                                                  \
+            F3M_LAUNCH((near_kernel<DD, T>), ntiles, bd, 0, s, tx.pts.get(), tx.n, ty.pts.get(), ty.n,                \
+                       bs + c * bstride, outs + c * ostride, lx.off.get(), ly.off.get(), lx.ctr.get(),                \
+                       list.pairs.get(), list.rowptr.get(), tileoff.get(), lx.nb, sc);                                \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)

@@ -340,31 +340,45 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         F3M_HIP(hipStreamSynchronize(s));
         return;
     }
-    DBuf<float> bs((size_t)P->M + 32), outs((size_t)P->N);   // bs padded: near_g_kernel reads whole tiles
+    // Columns are taken four at a time when at least two are left (the near field then computes every
+    // exponential once for the four), else one at a time.  bs columns are padded by one tile:
+    // near_g_kernel reads whole tiles.
+    const long long bstride = P->M + 32, ostride = P->N;
+    const int width = c >= 2 ? 4 : 1;
+    DBuf<float> bs((size_t)bstride * width), outs((size_t)ostride * width);
     const int depth = (int)P->levels.size();
     // F3M_FAR=levels: interpolate every level from the points like the reference (cross-check)
     const char *fe = getenv("F3M_FAR");
     const bool per_level = fe && !strcmp(fe, "levels");
-    for (int col = 0; col < c; col++) {
+    for (int col = 0; col < c;) {
+        const int left = c - col;
+        const int nc = left >= 2 ? 4 : 1;          // columns processed in this round (past `left`: zero weights)
+        const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
-            gather_column(b, P->ty->perm.get(), P->M, c, col, bs.get(), s);
-            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)P->N, s));
+            if (nc > ncol) F3M_HIP(hipMemsetAsync(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s));
+            for (int q = 0; q < ncol; q++) gather_column(b, P->ty->perm.get(), P->M, c, col + q, bs.get() + q * bstride, s);
+            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s));
         }
         for (int k = 1; k <= depth; k++) {
             PlanLevel &L = P->levels[k - 1];
             // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
-            near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s);
-            if (per_level) far_level(P, k, bs.get(), outs.get(), nullptr, nullptr, s);
+            near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s, nc,
+                       bstride, ostride);
+            if (per_level)
+                for (int q = 0; q < ncol; q++)
+                    far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
         }
-        if (!per_level) far_tree(P, bs.get(), outs.get(), s);
+        if (!per_level)
+            for (int q = 0; q < ncol; q++) far_tree(P, bs.get() + q * bstride, outs.get() + q * ostride, s);
         // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
         near_field(P->d, P->tx, P->tx.lev[depth], *P->ty, P->ty->lev[depth], P->levels[depth - 1].keep, bs.get(),
-                   outs.get(), P->lcs, s);
+                   outs.get(), P->lcs, s, nc, bstride, ostride);
         {
             Scope sc(kPerm, s);
-            scatter_column(outs.get(), P->tx.perm.get(), P->N, c, col, out, s);
+            for (int q = 0; q < ncol; q++) scatter_column(outs.get() + q * ostride, P->tx.perm.get(), P->N, c, col + q, out, s);
         }
+        col += ncol;
     }
     F3M_HIP(hipStreamSynchronize(s));
 }
