@@ -1537,6 +1537,58 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     }
 }
 
+// L2P for the 4 x 4 x 4 grid over every box of a level: one lane per point, 128 consecutive points per
+// workgroup whatever boxes they belong to (a level of small boxes keeps its lanes busy).  Each lane
+// finds its box among the box offsets that start inside the workgroup's range, reads the local expansion
+// of that box straight from global memory (lanes of one box read the same 16 bytes) and keeps its twelve
+// 1-D basis values in registers.
+__global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restrict__ xs, long long N, float *__restrict__ outs,
+                                                             const int *__restrict__ off, const float *__restrict__ ctr,
+                                                             int nb, const float *__restrict__ nt,
+                                                             const float *__restrict__ nw, float factor,
+                                                             const float *__restrict__ loc)
+{
+    __shared__ int bounds[kL2PBlock];
+    const int tid = threadIdx.x;
+    const long long i0 = (long long)blockIdx.x * kL2PBlock;
+    // box of the first point: last b with off[b] <= i0
+    int lo = 0, hi = nb;
+    while (hi - lo > 1) {
+        int mid = lo + ((hi - lo) >> 1);
+        if (off[mid] <= i0) lo = mid; else hi = mid;
+    }
+    const int b0 = lo;
+    bounds[tid] = off[min(b0 + 1 + tid, nb)];      // starts of the next boxes (off[nb] = N closes the list)
+    __syncthreads();
+    const long long i = i0 + tid;
+    if (i >= N) return;
+    // number of those starts that are <= i
+    int a = 0, b = kL2PBlock;
+    while (a < b) {
+        int mid = (a + b) >> 1;
+        if (bounds[mid] <= i) a = mid + 1; else b = mid;
+    }
+    const int box = b0 + a;
+    float l[3][4];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        const float t = factor * (xs[(long long)k * N + i] - ctr[(long long)box * 3 + k]);
+        basis_1d(t, nt + 4 * k, nw + 4 * k, 4, l[k], 1.f);
+    }
+    const float4 *lp = reinterpret_cast<const float4 *>(loc + (long long)box * 64);
+    float acc = 0.f;
+#pragma unroll
+    for (int h = 0; h < 16; h++) {
+        const float4 r = lp[h];
+        float inner = l[0][0] * r.x;
+        inner = fmaf(l[0][1], r.y, inner);
+        inner = fmaf(l[0][2], r.z, inner);
+        inner = fmaf(l[0][3], r.w, inner);
+        acc = fmaf(l[1][h & 3] * l[2][h >> 2], inner, acc);
+    }
+    outs[i] += acc;
+}
+
 void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
                hipStream_t s)
 {
@@ -1544,6 +1596,14 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     const int P = ns.P;
     NodeMeta nm = meta_of(ns);
     const float factor = 2 / lx.edge;
+    if (flag == nullptr && d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH(l2p_q64_kernel, cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_q64");
+        return;
+    }
     DBuf<int> tilex;
     int ntx = build_tiles(lx.off.get(), flag, lx.nb, tx.n, kL2PBlock, tilex, s);
     size_t shl = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)P + (size_t)kL2PBlock * (ns.S1 | 1));
@@ -1678,6 +1738,54 @@ __global__ void __launch_bounds__(1024) shift_kernel(const float *__restrict__ t
     if (!DOWN && tid < Pout) dst[(long long)b * sm.Pp + tid] = acc;
 }
 
+// The same transfer for the 4 x 4 x 4 grid on both levels: one wavefront per parent box, lane = node
+// (a0 + 4 a1 + 16 a2); the three 4 x 4 factors are applied with exchanges inside the wavefront (groups of
+// four lanes, lanes 4 apart, lanes 16 apart), no LDS traffic besides the 96-entry table, no barriers.
+constexpr int kShiftQWaves = 4;
+
+template <bool DOWN>
+__global__ void __launch_bounds__(kShiftQWaves * 64) shift_q64_kernel(const float *__restrict__ tables, int nbp,
+                                                                      const int *__restrict__ childstart,
+                                                                      const int *__restrict__ cellc,
+                                                                      const float *__restrict__ src, float *__restrict__ dst)
+{
+    // rows[(j*2+s)*4 + r] = the four table entries lane digit r needs: T[r][*] going up, T[*][r] going down
+    __shared__ __align__(16) float rows[3 * 2 * 4 * 4];
+    for (int e = threadIdx.x; e < 96; e += blockDim.x) {
+        const int q = e & 3, r = (e >> 2) & 3, js = e >> 4;
+        rows[e] = DOWN ? tables[(js * 4 + q) * 4 + r] : tables[(js * 4 + r) * 4 + q];
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int b = blockIdx.x * kShiftQWaves + (threadIdx.x >> 6);
+    if (b >= nbp) return;
+    const int a0 = lane & 3, a1 = (lane >> 2) & 3, a2 = lane >> 4;
+    const float v0 = DOWN ? src[(long long)b * 64 + lane] : 0.f;
+    float acc = 0.f;
+    for (int c = childstart[b]; c < childstart[b + 1]; c++) {
+        const int s0 = cellc[(long long)c * 3 + 0] & 1, s1 = cellc[(long long)c * 3 + 1] & 1, s2 = cellc[(long long)c * 3 + 2] & 1;
+        float v = DOWN ? v0 : src[(long long)c * 64 + lane];
+        const float4 r0 = *reinterpret_cast<const float4 *>(&rows[((0 * 2 + s0) * 4 + a0) * 4]);
+        float t = r0.x * quad_bcast<0>(v);
+        t = fmaf(r0.y, quad_bcast<1>(v), t);
+        t = fmaf(r0.z, quad_bcast<2>(v), t);
+        t = fmaf(r0.w, quad_bcast<3>(v), t);
+        const float4 r1 = *reinterpret_cast<const float4 *>(&rows[((1 * 2 + s1) * 4 + a1) * 4]);
+        float u = r1.x * wave_shfl_f(t, (lane & ~12) | 0);
+        u = fmaf(r1.y, wave_shfl_f(t, (lane & ~12) | 4), u);
+        u = fmaf(r1.z, wave_shfl_f(t, (lane & ~12) | 8), u);
+        u = fmaf(r1.w, wave_shfl_f(t, (lane & ~12) | 12), u);
+        const float4 r2 = *reinterpret_cast<const float4 *>(&rows[((2 * 2 + s2) * 4 + a2) * 4]);
+        float w = r2.x * wave_shfl_f(u, (lane & 15) | 0);
+        w = fmaf(r2.y, wave_shfl_f(u, (lane & 15) | 16), w);
+        w = fmaf(r2.z, wave_shfl_f(u, (lane & 15) | 32), w);
+        w = fmaf(r2.w, wave_shfl_f(u, (lane & 15) | 48), w);
+        if (DOWN) dst[(long long)c * 64 + lane] += w;
+        else acc += w;
+    }
+    if (!DOWN) dst[(long long)b * 64 + lane] = acc;
+}
+
 bool nodes_nest(const NodeSet &coarse, const NodeSet &fine)
 {
     if (coarse.d != fine.d) return false;
@@ -1719,7 +1827,15 @@ void shift_level(bool down, const TreeLevel &parent, const TreeLevel &child, con
     const int bd = ((sm.Pc + kWave - 1) / kWave) * kWave;
     size_t sh = sizeof(float) * ((size_t)ntab + 2 * (size_t)sm.Pc + (size_t)sm.Pp);
     timer_begin(down ? kL2P : kP2M, s);
-    if (down)
+    const bool q64 = d == 3 && sm.Pp == 64 && sm.Pc == 64 && sm.NTp == 4 && sm.NTc == 4 && nsp.n[0] == 4 && nsp.n[1] == 4 &&
+                     nsc.n[0] == 4 && nsc.n[1] == 4;
+    if (q64 && down)
+        F3M_LAUNCH((shift_q64_kernel<true>), cdiv(parent.nb, kShiftQWaves), kShiftQWaves * 64, 0, s, tab, parent.nb,
+                   parent.childstart.get(), child.cell.get(), src, dst);
+    else if (q64)
+        F3M_LAUNCH((shift_q64_kernel<false>), cdiv(parent.nb, kShiftQWaves), kShiftQWaves * 64, 0, s, tab, parent.nb,
+                   parent.childstart.get(), child.cell.get(), src, dst);
+    else if (down)
         F3M_LAUNCH((shift_kernel<true>), parent.nb, bd, sh, s, tab, ntab, sm, d, parent.childstart.get(), child.cell.get(),
                    src, dst);
     else
