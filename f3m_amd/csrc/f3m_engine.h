@@ -29,6 +29,7 @@ struct TreeLevel {
     // split-f16 matrix operand of its coordinates relative to its own box centre, scaled by nearops_sc
     mutable DBuf<unsigned char> nearops;
     mutable float nearops_sc = 0.f;
+    mutable bool nearops_partial = false;   // built for the source boxes of one list only
     // grid key -> box id table of this level (built on first use by lookup_boxes)
     mutable DBuf<uint32_t> hashtab;      // hashcap pairs (key, value), empty = 0xffffffff
     mutable uint32_t hashcap = 0;
@@ -105,10 +106,11 @@ void gather_points(const float *X, const int *perm, long long n, int d, float *p
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
 
-// nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride
+// nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride;
+// only_list: no other near list of this level will be applied with this plan
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc = 1, long long bstride = 0,
-                long long ostride = 0);
+                long long ostride = 0, bool only_list = false);
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);

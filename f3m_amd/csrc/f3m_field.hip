@@ -313,17 +313,43 @@ __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, in
 // as the rows (2y', -|y'|^2) of the matrix product in split-f16 form.  Layout: ops[(n*2 + h)*stride + i]
 // = the eight inner slots of half-wave h of instruction n; stride = npoints + 32 (the tail is zero so
 // that a wavefront may read one padded tile past the end).
+// need (nullable) = prefix count of the boxes that occur as sources (nb+1 entries): operands are then
+// written only for the points of those boxes and for the 31 points after them, which a wavefront may
+// read as the padding of a box's last tile.
+constexpr int kOpsBlock = 256;
+
 template <int D>
-__global__ void near_operands_kernel(const float *__restrict__ ys, long long M, const int *__restrict__ off, int nb,
-                                     const float *__restrict__ ctr, float sc, long long stride, h8 *__restrict__ ops)
+__global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *__restrict__ ys, long long M,
+                                                                  const int *__restrict__ off, int nb,
+                                                                  const float *__restrict__ ctr, float sc, long long stride,
+                                                                  const int *__restrict__ need, h8 *__restrict__ ops)
 {
     constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ int bounds[kOpsBlock];
+    const int tid = threadIdx.x;
+    const long long i0 = (long long)blockIdx.x * kOpsBlock, i = i0 + tid;
+    // boxes of the first point of this workgroup and of the point 31 before it (uniform)
+    const int b0 = find_box(off, nb, (int)min(i0, M - 1));
+    const int b0m = find_box(off, nb, (int)max(0ll, min(i0, M - 1) - 31));
+    bounds[tid] = off[min(b0 + 1 + tid, nb)];       // starts of the following boxes; off[nb] = M closes the list
+    __syncthreads();
     if (i >= stride) return;
     half_t hi[C], lo[C];
     if (i < M) {
-        const int box = find_box(off, nb, (int)i);
+        auto box_of = [&](long long p) {            // p >= i0: number of box starts <= p among the following boxes
+            int a = 0, b = kOpsBlock;
+            while (a < b) {
+                int mid = (a + b) >> 1;
+                if (bounds[mid] <= p) a = mid + 1; else b = mid;
+            }
+            return b0 + a;
+        };
+        const int box = box_of(i);
+        if (need != nullptr) {
+            const int first = (i - 31 >= i0) ? box_of(i - 31) : b0m;
+            if (need[box + 1] - need[first] == 0) return;
+        }
         float ny2 = 0.f;
 #pragma unroll
         for (int k = 0; k < C; k++) {
@@ -502,7 +528,8 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
 }
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
-                const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride)
+                const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride,
+                bool only_list)
 {
     if (list.n == 0) return;
     F3M_REQUIRE(nc == 1 || nc == 4, 34, "near field takes 1 or 4 columns at a time");
@@ -528,13 +555,26 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     if (use_mfma) {
         const int C = d + 2, NS = (3 * C + 15) / 16;
         const long long stride = ty.n + 32;
-        if (ly.nearops.size() == 0 || ly.nearops_sc != sc) {
+        // The operands of a level are kept in the plan.  only_list: this list is the only near list of
+        // its level, so operands are needed for its source boxes only (at most levels a small part).
+        if (ly.nearops.size() == 0 || ly.nearops_sc != sc || (ly.nearops_partial && !only_list)) {
             ly.nearops.reset((size_t)NS * 2 * stride * 16);
             ly.nearops_sc = sc;
+            ly.nearops_partial = only_list;
+            DBuf<int> need;
+            if (only_list) {
+                DBuf<int> fy((size_t)ly.nb);
+                F3M_HIP(hipMemsetAsync(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s));
+                F3M_LAUNCH(mark_cols_kernel, cdiv(list.n, 256), 256, 0, s, list.pairs.get(), list.n, fy.get());
+                check_launch("mark_cols");
+                need.reset((size_t)ly.nb + 1);
+                exclusive_scan_i32(fy.get(), ly.nb, need.get(), s);
+            }
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, 256), 256, 0, s, ty.pts.get(), ty.n, ly.off.get(), ly.nb, \
-                   ly.ctr.get(), sc, stride, reinterpret_cast<h8 *>(ly.nearops.get()));                               \
+        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
+                   ly.off.get(), ly.nb, ly.ctr.get(), sc, stride, only_list ? need.get() : (const int *)nullptr,      \
+                   reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
         break;
             switch (d) {
                 F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)

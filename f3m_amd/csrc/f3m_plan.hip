@@ -364,7 +364,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             PlanLevel &L = P->levels[k - 1];
             // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
             near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s, nc,
-                       bstride, ostride);
+                       bstride, ostride, /*only_list=*/k < depth || P->levels[depth - 1].keep.n == 0);
             if (per_level)
                 for (int q = 0; q < ncol; q++)
                     far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
