@@ -19,7 +19,7 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak
 # HBM bytes moved by one near-field launch of the default workload, from the rocprofv3 FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/ (None until measured)
-NEAR_TRAFFIC_BYTES = 5.685e9
+NEAR_TRAFFIC_BYTES = 5.722e9
 
 
 def cpu_baseline(X, Y, b, ls, budget_s=15.0):
@@ -124,7 +124,7 @@ def main():
     achieved = near_flops * args.steps / max(near_t, 1e-12) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_FP32_TFLOPS, "traffic": NEAR_TRAFFIC_BYTES if (N == 10_000_000 and d == 3) else None,
-                "kernel": "near_g_kernel<%d,4>" % d,
+                "kernel": "near_g_kernel<%d,4,1>" % d,
                 "note": "near field: exponents on the f16 matrix pipe (hi/lo-split operands, fp32 accumulate), exp2 + FMA on "
                         "the fp32 vector ALU; priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
                         "%.3e kernel evaluations/step x %d flops; traffic = HBM bytes per launch from rocprofv3 "
