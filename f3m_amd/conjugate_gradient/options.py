@@ -22,6 +22,9 @@ class FalkonOptions(ConjugateGradientOptions):
     pc_epsilon_32: float = 1e-5          # jitter (times M) added to K_MM before its Cholesky, fp32 data
     pc_epsilon_64: float = 1e-13
     pc_dtype: torch.dtype = torch.float64   # precision of the preconditioner factors
+    # keep T^-1 and A^-1 as dense matrices (two more M x M matrices) so that every triangular solve of
+    # the conjugate-gradient loop becomes one matrix-vector product; off: back-substitution each time
+    pc_explicit_inverse: bool = True
     use_cpu: bool = False                # kept for signature compatibility; the engine is GPU only
     debug: bool = False
 

@@ -21,6 +21,8 @@ class FalkonPreconditioner:
         self.params = opt
         self.T = None
         self.A = None
+        self.Tinv = None
+        self.Ainv = None
 
     def init(self, ny_points, weight_vec=None):
         if weight_vec is not None:
@@ -46,23 +48,46 @@ class FalkonPreconditioner:
         A.diagonal().add_(self.penalty)
         self.A = torch.linalg.cholesky(A, upper=True, out=A)
         self.T = T
+        self.Tinv = self.Ainv = None
+        if getattr(self.params, "pc_explicit_inverse", False) and 4 * nbytes <= self.MAX_MATRIX_BYTES * 2:
+            # the loop applies each factor's inverse (or its transpose) once or twice per iteration: as
+            # dense upper-triangular matrices these are matrix-vector products at memory speed
+            self.Tinv = self._inverse_upper(self.T)
+            self.Ainv = self._inverse_upper(self.A)
         return self
 
-    def _solve(self, tri, v, transpose):
-        out = torch.linalg.solve_triangular(tri.T if transpose else tri, v.to(tri.dtype), upper=not transpose)
+    @staticmethod
+    def _inverse_upper(U, block=1024):
+        """U^-1 by solves against blocks of identity columns (the library's triangular solve needs a
+        workspace that grows with the number of right-hand sides)."""
+        M = U.shape[0]
+        inv = torch.zeros_like(U)
+        for j0 in range(0, M, block):
+            j1 = min(M, j0 + block)
+            rhs = torch.zeros(j1, j1 - j0, dtype=U.dtype, device=U.device)      # rows past j1 of these columns are 0
+            rhs[j0:j1] = torch.eye(j1 - j0, dtype=U.dtype, device=U.device)
+            inv[:j1, j0:j1] = torch.linalg.solve_triangular(U[:j1, :j1], rhs, upper=True)
+        return inv
+
+    def _solve(self, tri, inv, v, transpose):
+        w = v.to(tri.dtype)
+        if inv is not None:
+            out = (inv.T if transpose else inv) @ w
+        else:
+            out = torch.linalg.solve_triangular(tri.T if transpose else tri, w, upper=not transpose)
         return out.to(v.dtype)
 
     def invA(self, v):
-        return self._solve(self.A, v, False)
+        return self._solve(self.A, self.Ainv, v, False)
 
     def invAt(self, v):
-        return self._solve(self.A, v, True)
+        return self._solve(self.A, self.Ainv, v, True)
 
     def invT(self, v):
-        return self._solve(self.T, v, False)
+        return self._solve(self.T, self.Tinv, v, False)
 
     def invTt(self, v):
-        return self._solve(self.T, v, True)
+        return self._solve(self.T, self.Tinv, v, True)
 
     def apply(self, v):
         return self.invT(self.invA(v))

@@ -63,3 +63,19 @@ def test_conjugate_gradient_solves_spd_system():
     X = cg.solve(None, B, lambda v: A @ v, max_iter=200)
     assert torch.allclose(A @ X, B, atol=1e-7)
     assert cg.iterations_ <= 70             # exact in about dim steps; stops at the tolerance
+
+
+def test_explicit_inverse_factors_equal_back_substitution():
+    """pc_explicit_inverse keeps T^-1 and A^-1 as matrices; every solve must agree with back-substitution."""
+    from f3m_amd.conjugate_gradient.options import FalkonOptions
+    from f3m_amd.conjugate_gradient.preconditioner import FalkonPreconditioner
+    torch.manual_seed(1)
+    C = 2 * torch.rand(120, 3) - 1
+    k = DenseGaussian(0.5)
+    fast = FalkonPreconditioner(1e-6, k, FalkonOptions(pc_explicit_inverse=True)).init(C)
+    slow = FalkonPreconditioner(1e-6, k, FalkonOptions(pc_explicit_inverse=False)).init(C)
+    assert fast.Tinv is not None and slow.Tinv is None
+    v = torch.randn(120, 3, dtype=torch.float64)
+    for name in ("invA", "invAt", "invT", "invTt", "apply", "apply_t"):
+        a, b = getattr(fast, name)(v), getattr(slow, name)(v)
+        assert torch.allclose(a, b, rtol=1e-8, atol=1e-8 * float(b.abs().max())), name
