@@ -168,51 +168,62 @@ __global__ void morton_kernel(const float *__restrict__ X, long long n, Geo g, u
 }
 
 // ------------------------------------------------------------------------------------------------
-// Counting sort by 8-bit digits, least significant first; stable.  One wavefront per workgroup:
-// inside a round of 64 keys the rank of a key among equal digits comes from eight ballots, and
-// the running digit offsets live in LDS.
+// Counting sort by 8-bit digits, least significant first; stable.  A workgroup of four wavefronts
+// takes a tile of 8192 keys (2048 per wavefront, in order).  Inside a round of 64 keys the rank of a key
+// among equal digits comes from eight ballots; running digit counts per wavefront live in LDS.  The
+// tile is first reordered by digit inside LDS and then written out, so that the ~32 keys of a tile that
+// share a digit leave as one contiguous run.
 
+constexpr int kSortWaves = 4;
 constexpr int kSortRounds = 32;
-constexpr int kSortTile = kWave * kSortRounds;
+constexpr int kSortTile = kSortWaves * kWave * kSortRounds;
 
-__global__ void __launch_bounds__(64) sort_hist_kernel(const uint32_t *__restrict__ keys, long long n, int shift,
-                                                         int *__restrict__ blockhist, int nblk)
+__global__ void __launch_bounds__(kSortWaves * 64) sort_hist_kernel(const uint32_t *__restrict__ keys, long long n, int shift,
+                                                                    int *__restrict__ blockhist, int nblk)
 {
     __shared__ int hist[256];
-    const int lane = threadIdx.x;
-    for (int b = lane; b < 256; b += kWave) hist[b] = 0;
+    const int tid = threadIdx.x;
+    hist[tid] = 0;
     __syncthreads();
     const long long base = (long long)blockIdx.x * kSortTile;
     for (int r = 0; r < kSortRounds; r++) {
-        long long i = base + r * kWave + lane;
+        long long i = base + (long long)r * (kSortWaves * kWave) + tid;
         if (i < n) atomicAdd(&hist[(keys[i] >> shift) & 255u], 1);
     }
     __syncthreads();
-    for (int b = lane; b < 256; b += kWave) blockhist[(long long)b * nblk + blockIdx.x] = hist[b];
+    blockhist[(long long)tid * nblk + blockIdx.x] = hist[tid];
 }
 
-__global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__restrict__ keys_in, const int *__restrict__ idx_in,
-                                                            uint32_t *__restrict__ keys_out, int *__restrict__ idx_out,
-                                                            long long n, int shift, const int *__restrict__ base, int nblk)
+__global__ void __launch_bounds__(kSortWaves * 64) sort_scatter_kernel(const uint32_t *__restrict__ keys_in,
+                                                                       const int *__restrict__ idx_in,
+                                                                       uint32_t *__restrict__ keys_out,
+                                                                       int *__restrict__ idx_out, long long n, int shift,
+                                                                       const int *__restrict__ base, int nblk)
 {
-    __shared__ int run[256];
-    const int lane = threadIdx.x;
-    for (int b = lane; b < 256; b += kWave) run[b] = base[(long long)b * nblk + blockIdx.x];
+    __shared__ int wrun[kSortWaves][256];     // per wavefront: keys of each digit met so far; then its offset
+    __shared__ int tstart[256];               // first position of each digit inside the reordered tile
+    __shared__ int gdelta[256];               // global position minus tile position, per digit
+    __shared__ uint32_t skey[kSortTile];
+    __shared__ int sval[kSortTile];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    for (int b = lane; b < 256; b += kWave) wrun[w][b] = 0;
     __syncthreads();
     const long long tile = (long long)blockIdx.x * kSortTile;
+    const long long mine = tile + (long long)w * (kWave * kSortRounds);      // this wavefront's 2048 keys
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    // the whole tile goes to registers first, so that the loads of all rounds are in flight together
+    // the whole share goes to registers first, so that the loads of all rounds are in flight together
     uint32_t key[kSortRounds];
     int val[kSortRounds];
+    int rk[kSortRounds];                      // rank among the keys of the same digit in this wavefront
 #pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
-        long long i = tile + r * kWave + lane;
+        long long i = mine + r * kWave + lane;
         key[r] = (i < n) ? keys_in[i] : 0u;
         val[r] = (i < n) ? idx_in[i] : 0;
     }
 #pragma unroll
     for (int r = 0; r < kSortRounds; r++) {
-        long long i = tile + r * kWave + lane;
+        long long i = mine + r * kWave + lane;
         bool valid = i < n;
         uint32_t digit = (key[r] >> shift) & 255u;
         unsigned long long same = wave_ballot(valid);
@@ -223,14 +234,55 @@ __global__ void __launch_bounds__(64) sort_scatter_kernel(const uint32_t *__rest
             same &= one ? m : ~m;
         }
         int rank = __popcll(same & below);
-        int start = valid ? run[digit] : 0;
-        __syncthreads();
-        if (valid && rank == 0) run[digit] = start + __popcll(same);
-        __syncthreads();
-        if (valid) {
-            keys_out[start + rank] = key[r];
-            idx_out[start + rank] = val[r];
+        int start = valid ? wrun[w][digit] : 0;           // only this wavefront touches wrun[w]
+        rk[r] = start + rank;
+        wave_sync();                                       // every lane has read before the first lane of a digit writes
+        if (valid && rank == 0) wrun[w][digit] = start + __popcll(same);
+        wave_sync();
+    }
+    __syncthreads();
+    // digit d: counts per wavefront -> offsets of the wavefronts, tile total -> start inside the tile
+    {
+        int c[kSortWaves], tot = 0;
+#pragma unroll
+        for (int v = 0; v < kSortWaves; v++) { c[v] = wrun[v][tid]; }
+#pragma unroll
+        for (int v = 0; v < kSortWaves; v++) { wrun[v][tid] = tot; tot += c[v]; }
+        tstart[tid] = tot;
+    }
+    __syncthreads();
+    if (w == 0) {                              // exclusive scan of the 256 totals by one wavefront
+        int v[4], sum = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { v[e] = tstart[lane * 4 + e]; sum += v[e]; }
+        int incl = sum;
+        for (int off = 1; off < 64; off <<= 1) {
+            int t = wave_shfl_i(incl, lane >= off ? lane - off : lane);
+            if (lane >= off) incl += t;
         }
+        int run = incl - sum;
+#pragma unroll
+        for (int e = 0; e < 4; e++) { tstart[lane * 4 + e] = run; run += v[e]; }
+    }
+    __syncthreads();
+    gdelta[tid] = base[(long long)tid * nblk + blockIdx.x] - tstart[tid];
+#pragma unroll
+    for (int r = 0; r < kSortRounds; r++) {
+        long long i = mine + r * kWave + lane;
+        if (i < n) {
+            uint32_t digit = (key[r] >> shift) & 255u;
+            int p = tstart[digit] + wrun[w][digit] + rk[r];
+            skey[p] = key[r];
+            sval[p] = val[r];
+        }
+    }
+    __syncthreads();
+    const int cnt = (int)min((long long)kSortTile, n - tile);
+    for (int j = tid; j < cnt; j += kSortWaves * kWave) {
+        const uint32_t k = skey[j];
+        const int g = gdelta[(k >> shift) & 255u] + j;
+        keys_out[g] = k;
+        idx_out[g] = sval[j];
     }
 }
 
@@ -243,10 +295,10 @@ static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int fr
     DBuf<int> hist((size_t)256 * nblk);
     DBuf<int> base((size_t)256 * nblk + 1);
     for (int shift = from; shift < bits; shift += 8) {
-        F3M_LAUNCH(sort_hist_kernel, nblk, kWave, 0, s, keys.get(), n, shift, hist.get(), nblk);
+        F3M_LAUNCH(sort_hist_kernel, nblk, kSortWaves * kWave, 0, s, keys.get(), n, shift, hist.get(), nblk);
         check_launch("sort_hist");
         exclusive_scan_i32(hist.get(), (long long)256 * nblk, base.get(), s);
-        F3M_LAUNCH(sort_scatter_kernel, nblk, kWave, 0, s, keys.get(), idx.get(), keys2.get(), idx2.get(), n, shift,
+        F3M_LAUNCH(sort_scatter_kernel, nblk, kSortWaves * kWave, 0, s, keys.get(), idx.get(), keys2.get(), idx2.get(), n, shift,
                    base.get(), nblk);
         check_launch("sort_scatter");
         std::swap(keys, keys2);

@@ -164,6 +164,8 @@ inline void check_launch(const char *what)
 // ---- wave helpers ---------------------------------------------------------------------------
 #ifdef F3M_CPU_EMU
 __device__ inline unsigned long long wave_ballot(bool p) { return emu::ballot(p); }
+// orders the LDS accesses of the lanes of one wavefront (the lanes run in lockstep on the GPU)
+__device__ inline void wave_sync() { (void)emu::ballot(false); }
 __device__ inline unsigned lane_id() { return emu::S().cur->tid % 64; }
 __device__ inline float fast_exp2(float x) { return exp2f(x); }
 __device__ inline float fast_rcp(float x) { return 1.0f / x; }
@@ -267,6 +269,9 @@ __device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
 }
 #else
 __device__ __forceinline__ unsigned long long wave_ballot(bool p) { return __ballot(p); }
+// orders the LDS accesses of the lanes of one wavefront (the lanes run in lockstep; this only keeps the
+// compiler from moving memory operations across the point)
+__device__ __forceinline__ void wave_sync() { __builtin_amdgcn_wave_barrier(); }
 __device__ __forceinline__ unsigned lane_id() { return __lane_id(); }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }   // v_rcp_f32, 1 ulp
