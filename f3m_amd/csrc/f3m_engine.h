@@ -79,10 +79,26 @@ void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipS
 // every division is done (divisions may still refine the order inside the boxes)
 void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s);
 void gather_tree_points(Tree &t, const float *X, hipStream_t s);
-// adds lev[k] from lev[k-1]; returns false (and adds nothing) if the key depth is exhausted
-bool divide_tree(Tree &t, hipStream_t s);
-void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
-                  PlanLevel &out, hipStream_t s);
+// One division in two steps, so that the host can wait once for several results: divide_launch starts
+// the kernels that build lev[k] from lev[k-1] and appends the level; divide_finish completes it with
+// the two numbers the kernels left in dstats (boxes, largest count) once the host has fetched them;
+// divide_discard drops a level that turned out not to be needed.
+void divide_launch(Tree &t, int *dstats, hipStream_t s);
+void divide_finish(Tree &t, const int *hstats);
+void divide_discard(Tree &t);
+// The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts (the four totals
+// -- small, far, keep, far pairs outside the M2L tables -- go to dtot on the device), lists_finish
+// allocates from the fetched totals and writes.
+struct ListsPending {
+    DBuf<long long> pos;
+    long long stride = 0;
+    unsigned grid = 0;
+    bool active = false;
+};
+void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+                  ListsPending &pend, long long *dtot, hipStream_t s);
+void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                  const ClassifyParams &cp, PlanLevel &out, hipStream_t s);
 void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
 void build_rowptr(PairList &l, int nbx, hipStream_t s);

@@ -413,11 +413,11 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
     }
 }
 
-bool divide_tree(Tree &t, hipStream_t s)
+void divide_launch(Tree &t, int *dstats, hipStream_t s)
 {
     const int d = t.geo.d;
     const int k = (int)t.lev.size();   // depth being built
-    if (k > t.geo.L) return false;
+    F3M_REQUIRE(k <= t.geo.L, 20, "depth %d exceeds the key depth", k);
     int shift = d * (t.geo.L - k);
     if (shift < t.sorted_from) {
         // the points are grouped by the boxes built so far whatever the order inside a box, so the
@@ -428,7 +428,7 @@ bool divide_tree(Tree &t, hipStream_t s)
     TreeLevel &prev = t.lev[k - 1];
     long long ncand = (long long)prev.nb << d;
     F3M_REQUIRE(ncand < (1ll << 31) - 2, 20, "too many candidate boxes at depth %d (%lld)", k, ncand);
-    DBuf<int> natpos((size_t)ncand + 1), flag((size_t)ncand), cid((size_t)ncand + 1), stats(2);
+    DBuf<int> natpos((size_t)ncand + 1), flag((size_t)ncand), cid((size_t)ncand + 1);
     F3M_LAUNCH(child_bounds_kernel, cdiv(ncand + 1, 256), 256, 0, s, t.keys.get(), prev.prefix.get(), prev.off.get(), ncand,
                d, shift, t.n, natpos.get());
     check_launch("child_bounds");
@@ -443,20 +443,25 @@ bool divide_tree(Tree &t, hipStream_t s)
     cur.ctr.reset(bound * d);
     cur.cell.reset(bound * d);
     prev.childstart.reset((size_t)prev.nb + 1);
-    F3M_HIP(hipMemsetAsync(stats.get(), 0, 2 * sizeof(int), s));
+    F3M_HIP(hipMemsetAsync(dstats, 0, 2 * sizeof(int), s));
     float quarter = 0.25f * prev.edge;
     F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
                prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
-               prev.childstart.get(), stats.get());
+               prev.childstart.get(), dstats);
     check_launch("build_level");
-    int h[2];
-    d2h(h, stats.get(), 2, s);
-    cur.nb = h[0];
-    cur.maxcount = h[1];
+    cur.nb = -1;                       // until divide_finish
+    cur.maxcount = -1;
     cur.edge = prev.edge * 0.5f;
     t.lev.push_back(std::move(cur));
-    return true;
 }
+
+void divide_finish(Tree &t, const int *hstats)
+{
+    t.lev.back().nb = hstats[0];
+    t.lev.back().maxcount = hstats[1];
+}
+
+void divide_discard(Tree &t) { t.lev.pop_back(); }
 
 // ------------------------------------------------------------------------------------------------
 // Grid key -> box id through an open-addressing table in HBM (F3M_src/linearprobing.cu:18-87, used by
@@ -687,34 +692,46 @@ void build_rowptr(PairList &l, int nbx, hipStream_t s)
     check_launch("rowptr");
 }
 
-void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
-                  PlanLevel &out, hipStream_t s)
+void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+                  ListsPending &pend, long long *dtot, hipStream_t s)
 {
     const int d = tx.geo.d;
     const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
-    out.far.n = out.small_.n = out.keep.n = 0;
+    pend.active = false;
+    F3M_HIP(hipMemsetAsync(dtot, 0, 4 * sizeof(long long), s));
     if (keep_prev.n == 0) return;
     F3M_REQUIRE(keep_prev.n < (1ll << 31) - 2, 21, "keep list too long (%lld)", keep_prev.n);
     F3M_REQUIRE((1 << d) < (1 << 21), 21, "too many children per box");
+    pend.active = true;
     const bool one_tree = &tx == &ty;
     const int nbx = lx.nb;
-    const long long stride = (long long)nbx + 1;
-    DBuf<long long> cnt((size_t)(3 * stride)), pos((size_t)(3 * stride)), dtot(4);
-    F3M_HIP(hipMemsetAsync(dtot.get() + 3, 0, sizeof(long long), s));
+    pend.stride = (long long)nbx + 1;
+    DBuf<long long> cnt((size_t)(3 * pend.stride));
+    pend.pos.reset((size_t)(3 * pend.stride));
     const int *cellx = one_tree ? lx.cell.get() : (const int *)nullptr;
-    unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot.get() + 3);
-    const unsigned grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
-    F3M_LAUNCH((lists_kernel<false>), grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+    unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
+    pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
+    F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
                cellx, ly.cell.get(), outl, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
-    for (int c = 0; c < 3; c++) exclusive_scan_i64(cnt.get() + c * stride, nbx, pos.get() + c * stride, s);
-    F3M_LAUNCH(list_totals_kernel, 1, 64, 0, s, pos.get(), stride, dtot.get());
+    for (int c = 0; c < 3; c++) exclusive_scan_i64(cnt.get() + c * pend.stride, nbx, pend.pos.get() + c * pend.stride, s);
+    F3M_LAUNCH(list_totals_kernel, 1, 64, 0, s, pend.pos.get(), pend.stride, dtot);
     check_launch("list_totals");
-    long long tot[4];
-    d2h(tot, dtot.get(), 4, s);
+}
+
+void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                  const ClassifyParams &cp, PlanLevel &out, hipStream_t s)
+{
+    out.far.n = out.small_.n = out.keep.n = 0;
+    if (!pend.active) return;
+    const int d = tx.geo.d;
+    const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
+    const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
+    const bool one_tree = &tx == &ty;
+    const int nbx = lx.nb;
     for (int c = 0; c < 3; c++) F3M_REQUIRE(tot[c] < (1ll << 31) - 2, 22, "interaction list too long (%lld)", tot[c]);
     out.far.outliers = one_tree ? tot[3] : -1;
     out.small_.n = tot[0];
@@ -723,15 +740,18 @@ void expand_lists(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     out.small_.pairs.reset((size_t)std::max<long long>(1, tot[0]) * 2);
     out.far.pairs.reset((size_t)std::max<long long>(1, tot[1]) * 2);
     out.keep.pairs.reset((size_t)std::max<long long>(1, tot[2]) * 2);
-    out.small_.rowptr.reset((size_t)stride);
-    out.far.rowptr.reset((size_t)stride);
-    out.keep.rowptr.reset((size_t)stride);
-    F3M_LAUNCH((lists_kernel<true>), grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+    out.small_.rowptr.reset((size_t)pend.stride);
+    out.far.rowptr.reset((size_t)pend.stride);
+    out.keep.rowptr.reset((size_t)pend.stride);
+    const int *cellx = one_tree ? lx.cell.get() : (const int *)nullptr;
+    F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cell.get(), outl, (long long *)nullptr, (const long long *)pos.get(), out.small_.pairs.get(),
-               out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(), out.far.rowptr.get(),
-               out.keep.rowptr.get());
+               cellx, ly.cell.get(), (unsigned long long *)nullptr, (long long *)nullptr, (const long long *)pend.pos.get(),
+               out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
+               out.far.rowptr.get(), out.keep.rowptr.get());
     check_launch("lists_write");
+    pend.pos.free();
+    pend.active = false;
 }
 
 }  // namespace f3m

@@ -216,24 +216,56 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     build_rowptr(root, 1, s);
     const PairList *keep = &root;
     P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
-    // loop guard of F3M_src/n_tree.cu:1075 (symmetric) and :1099 (two trees)
-    while (need_tree && keep->n > 0 && (float)P->tx.lev.back().maxcount > prm->min_points &&
-           (sym || (float)P->ty_.lev.back().maxcount > prm->min_points)) {
-        if ((int)P->tx.lev.size() > gx.L) break;
-        divide_tree(P->tx, s);
-        if (!sym) divide_tree(P->ty_, s);
-        int k = (int)P->tx.lev.size() - 1;
-        float e = P->tx.lev[k].edge;
-        P->levels.emplace_back();
-        PlanLevel &L = P->levels.back();
-        expand_lists(*keep, P->tx, *P->ty, k, classify_params(*P, e), L, s);
-        L.num_nodes = prm->nr_of_interpolation;
-        if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
-            L.num_nodes = std::min((int)pow(3, d), prm->nr_of_interpolation);
-        keep = &L.keep;
-        if (getenv("F3M_DEBUG"))
-            fprintf(stderr, "level %d: boxes %d far %lld (outliers %lld) small %lld keep %lld\n", k, P->tx.lev[k].nb, L.far.n,
-                    L.far.outliers, L.small_.n, L.keep.n);
+    // Loop of F3M_src/n_tree.cu:1075 (one tree) and :1099 (two trees): divide while the keep list is not
+    // empty and the fullest box of each tree holds more than min_points points.  The host has to fetch
+    // two things per level, the box counts of the division and the list sizes; to wait only once per
+    // level, the division of depth k+1 is started together with the list count of depth k whenever the
+    // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
+    DBuf<int> dres(16);          // [0..7]: four 64-bit list totals, [8,9]: X tree stats, [10,11]: Y tree stats
+    int hres[16];
+    auto wants_division = [&]() {
+        return (float)P->tx.lev.back().maxcount > prm->min_points &&
+               (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
+    };
+    auto start_division = [&]() {
+        divide_launch(P->tx, dres.get() + 8, s);
+        if (!sym) divide_launch(P->ty_, dres.get() + 10, s);
+    };
+    auto finish_division = [&]() {
+        divide_finish(P->tx, hres + 8);
+        if (!sym) divide_finish(P->ty_, hres + 10);
+    };
+    if (need_tree && wants_division()) {
+        start_division();
+        d2h(hres, dres.get(), 16, s);
+        finish_division();
+        for (;;) {
+            const int k = (int)P->tx.lev.size() - 1;
+            const float e = P->tx.lev[k].edge;
+            P->levels.emplace_back();
+            PlanLevel &L = P->levels.back();
+            const ClassifyParams cp = classify_params(*P, e);
+            ListsPending pend;
+            lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
+            const bool ahead = wants_division();
+            if (ahead) start_division();
+            d2h(hres, dres.get(), 16, s);
+            lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L, s);
+            if (ahead) finish_division();
+            L.num_nodes = prm->nr_of_interpolation;
+            if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
+                L.num_nodes = std::min((int)pow(3, d), prm->nr_of_interpolation);
+            keep = &L.keep;
+            if (getenv("F3M_DEBUG"))
+                fprintf(stderr, "level %d: boxes %d far %lld (outliers %lld) small %lld keep %lld\n", k, P->tx.lev[k].nb, L.far.n,
+                        L.far.outliers, L.small_.n, L.keep.n);
+            if (ahead && keep->n > 0) continue;
+            if (ahead) {
+                divide_discard(P->tx);
+                if (!sym) divide_discard(P->ty_);
+            }
+            break;
+        }
     }
     if (need_tree) {
         gather_tree_points(P->tx, X, s);
