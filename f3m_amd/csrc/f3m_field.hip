@@ -454,6 +454,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         h8 bop[TPW][NS];
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
+            if (q >= nlive) continue;                 // uniform per wavefront: tiles without targets need no operands
             const bool ok = x0 + q * 32 + col < x1;
             half_t hi[C], lo[C];
             float nx2 = 0.f;
