@@ -395,7 +395,8 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const float *__restrict__ ctry, const int *__restrict__ pairs,
-    const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc, int stripe)
+    const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc, int stripe, int nsplit,
+    float *__restrict__ part)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
@@ -410,7 +411,11 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         const int r = blockIdx.x >> 3, xcd = blockIdx.x & 7;
         vblock = (r / stripe) * (8 * stripe) + xcd * stripe + (r % stripe);
     }
-    const int wid = vblock * kNearWavesPerBlock + (threadIdx.x >> 6);          // work item: TPW*32 targets of one box
+    // work item: TPW*32 targets of one box; with few targets and long lists (nsplit > 1) the list of a
+    // work item is cut into nsplit slices, one wavefront each, whose sums go to `part` and are added up
+    // in a fixed order afterwards
+    const int wfull = vblock * kNearWavesPerBlock + (threadIdx.x >> 6);
+    const int wid = wfull / nsplit, slice = wfull % nsplit;
     if (wid >= tileoff[nbx]) return;
     const int bx = find_box(tileoff, nbx, wid);
     const int x0 = offx[bx] + (wid - tileoff[bx]) * (TPW * 32), x1 = offx[bx + 1];
@@ -429,6 +434,23 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
 #pragma unroll
         for (int c = 0; c < NC; c++) acc[q][c] = 0.f;
     const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
+    // slice of this wavefront, in 32-source tiles counted along the whole row: [tlo, thi)
+    int tlo = 0, thi = 0x7fffffff;
+    if (nsplit > 1) {
+        int ttot = 0;
+        for (int mb = m0; mb < m1; mb += 64) {
+            int nt = 0;
+            if (mb + lane < m1) {
+                const int byv = pairs[2 * (long long)(mb + lane) + 1];
+                nt = (offy[byv + 1] - offy[byv] + 31) >> 5;
+            }
+            for (int off = 32; off > 0; off >>= 1) nt += wave_shfl_i(nt, lane ^ off);
+            ttot += nt;
+        }
+        tlo = (int)((long long)ttot * slice / nsplit);
+        thi = (int)((long long)ttot * (slice + 1) / nsplit);
+    }
+    int tcur = 0;                                    // tiles of the row before the current y box
     // the list is consumed 64 y boxes at a time: every lane fetches the range and centre of one y box,
     // then the wavefront walks through them (one round of memory latency per 64 boxes)
     for (int mb = m0; mb < m1; mb += 64) {
@@ -446,7 +468,16 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
       }
       const int mcnt = min(64, m1 - mb);
       for (int mj = 0; mj < mcnt; mj++) {
-        const int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mj);
+        int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mj);
+        if (nsplit > 1) {                            // keep the part of this box that lies in the slice
+            const int nt = (s1 - s0 + 31) >> 5;
+            const int a = max(tlo, tcur), b = min(thi, tcur + nt);
+            const int first = s0 + 32 * (a - tcur);
+            if (b < tcur + nt) s1 = s0 + 32 * (b - tcur);
+            s0 = first;
+            tcur += nt;
+            if (a >= b) continue;                    // uniform
+        }
         float cy[D];
 #pragma unroll
         for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
@@ -523,9 +554,25 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             float total = acc[q][c] + wave_shfl_xor_f(acc[q][c], 32);
-            if (half == 0 && i < x1) outs[c * ostride + i] += total;
+            if (half == 0 && i < x1) {
+                if (nsplit > 1) part[((long long)slice * NC + c) * N + i] = total;
+                else outs[c * ostride + i] += total;
+            }
         }
     }
+}
+
+// outs += the slices of a split near field, in slice order
+__global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, int nc, long long N,
+                                   float *__restrict__ outs, long long ostride)
+{
+    long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= N * nc) return;
+    const int c = (int)(e / N);
+    const long long i = e % N;
+    float sum = 0.f;
+    for (int sl = 0; sl < nsplit; sl++) sum += part[((long long)sl * nc + c) * N + i];
+    outs[c * ostride + i] += sum;
 }
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
@@ -587,7 +634,18 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         }
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
-        int nblk = (int)cdiv(ntiles, kNearWavesPerBlock);
+        // Few targets against long lists (the transposed product of a tall kernel matrix): too few work
+        // items to fill the GPU, so every list is cut into slices with a wavefront each.
+        int nsplit = 1;
+        if (ntiles < 2048) {
+            nsplit = std::min(64, (int)cdiv(8192, std::max(1, ntiles)));
+        }
+        DBuf<float> part;
+        if (nsplit > 1) {
+            part.reset((size_t)nsplit * nc * tx.n);
+            F3M_HIP(hipMemsetAsync(part.get(), 0, sizeof(float) * (size_t)nsplit * nc * tx.n, s));
+        }
+        int nblk = (int)cdiv((long long)ntiles * nsplit, kNearWavesPerBlock);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
@@ -596,12 +654,12 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
             F3M_LAUNCH((near_g_kernel<DD, tpw, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
-                       tileoff.get(), lx.nb, sc, stripe);                                                             \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         else                                                                                                          \
             F3M_LAUNCH((near_g_kernel<DD, tpw, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
-                       tileoff.get(), lx.nb, sc, stripe);                                                             \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -609,6 +667,10 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         default: throw Error(2, "dimension must be 1..10");
         }
 #undef F3M_CASE
+        if (nsplit > 1) {
+            check_launch("near_g");
+            F3M_LAUNCH(near_reduce_kernel, cdiv(tx.n * nc, 256), 256, 0, s, part.get(), nsplit, nc, tx.n, outs, ostride);
+        }
     } else {
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
