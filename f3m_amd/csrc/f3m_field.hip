@@ -637,8 +637,11 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         // Few targets against long lists (the transposed product of a tall kernel matrix): too few work
         // items to fill the GPU, so every list is cut into slices with a wavefront each.
         int nsplit = 1;
-        if (ntiles < 2048) {
-            nsplit = std::min(64, (int)cdiv(8192, std::max(1, ntiles)));
+        if (ntiles < 16384) {
+            int target = 32768;      // wavefronts aimed at (K_nm^T u with 1e7 sources, 2e4 / 1e5 targets: 8192 -> 9.7 / 8.1 ms,
+                                     // 16384 -> 7.6 / 6.8, 32768 -> 7.5 / 6.0)
+            if (const char *e = getenv("F3M_SPLIT_TARGET")) target = atoi(e);
+            nsplit = std::min(128, (int)cdiv(target, std::max(1, ntiles)));
         }
         DBuf<float> part;
         if (nsplit > 1) {
