@@ -87,41 +87,68 @@ void exclusive_scan_i64(const long long *in, long long n, long long *out, hipStr
 // ------------------------------------------------------------------------------------------------
 // bounding box (F3M_src/n_tree.cu:28-31,42-43: per-dimension min and max)
 
-constexpr int kBBGrid = 512;
-
-__global__ void minmax_kernel(const float *__restrict__ X, long long n, int d, float *__restrict__ part)
+// signed integers ordered like the floats they come from (-0 below +0), and back
+__device__ inline int float_order(float v)
 {
-    __shared__ float sh[256];
-    float lo[kMaxD], hi[kMaxD];
-    for (int j = 0; j < kMaxD; j++) { lo[j] = INFINITY; hi[j] = -INFINITY; }
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
-        for (int j = 0; j < d; j++) {
-            float v = X[i * d + j];
-            lo[j] = fminf(lo[j], v);
-            hi[j] = fmaxf(hi[j], v);
-        }
-    for (int j = 0; j < d; j++)
-        for (int pass = 0; pass < 2; pass++) {
-            sh[threadIdx.x] = pass ? hi[j] : lo[j];
-            __syncthreads();
-            for (int off = 128; off > 0; off >>= 1) {
-                if ((int)threadIdx.x < off) {
-                    float a = sh[threadIdx.x], b = sh[threadIdx.x + off];
-                    sh[threadIdx.x] = pass ? fmaxf(a, b) : fminf(a, b);
-                }
-                __syncthreads();
-            }
-            if (threadIdx.x == 0) part[((long long)blockIdx.x * 2 + pass) * kMaxD + j] = sh[0];
-            __syncthreads();
-        }
+    const int b = __builtin_bit_cast(int, v);
+    return b >= 0 ? b : b ^ 0x7fffffff;
+}
+__device__ inline float float_unorder(int k) { return __builtin_bit_cast(float, k >= 0 ? k : k ^ 0x7fffffff); }
+
+// X is read as one flat array, four floats per load.  The number of threads is a multiple of d, so the
+// elements a thread meets always belong to the same four dimensions and it keeps four running pairs.
+constexpr int kBBBlocksPerDim = 192;
+
+// `prefix` (0..3) leading elements come before the first 16-byte boundary and are read one by one.
+__global__ void __launch_bounds__(256) minmax_kernel(const float *__restrict__ X, long long total, int d, int prefix,
+                                                     float *__restrict__ part)
+{
+    __shared__ int smin[kMaxD], smax[kMaxD];
+    const long long T = (long long)gridDim.x * blockDim.x;            // multiple of d
+    const long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    float lo[4], hi[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) { lo[c] = INFINITY; hi[c] = -INFINITY; }
+    const long long nvec = (total - prefix) / 4;
+    const float4 *X4 = reinterpret_cast<const float4 *>(X + prefix);
+    for (long long e = g; e < nvec; e += T) {
+        const float4 v = X4[e];
+        lo[0] = fminf(lo[0], v.x); hi[0] = fmaxf(hi[0], v.x);
+        lo[1] = fminf(lo[1], v.y); hi[1] = fmaxf(hi[1], v.y);
+        lo[2] = fminf(lo[2], v.z); hi[2] = fmaxf(hi[2], v.z);
+        lo[3] = fminf(lo[3], v.w); hi[3] = fmaxf(hi[3], v.w);
+    }
+    // per-dimension minimum and maximum of the workgroup through integer atomics in LDS on an
+    // order-preserving image of the floats (NaNs stay out, as with fminf/fmaxf)
+    if ((int)threadIdx.x < kMaxD) { smin[threadIdx.x] = 0x7fffffff; smax[threadIdx.x] = (int)0x80000000; }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const int j = (int)((prefix + 4 * g + c) % d);
+        if (lo[c] == lo[c]) atomicMin(&smin[j], float_order(lo[c]));
+        if (hi[c] == hi[c]) atomicMax(&smax[j], float_order(hi[c]));
+    }
+    if (g == 0) {                                                      // the few elements before and after the full loads
+        for (long long e = 0; e < prefix && e < total; e++)
+            if (X[e] == X[e]) { atomicMin(&smin[e % d], float_order(X[e])); atomicMax(&smax[e % d], float_order(X[e])); }
+        for (long long e = prefix + 4 * nvec; e < total; e++)
+            if (X[e] == X[e]) { atomicMin(&smin[e % d], float_order(X[e])); atomicMax(&smax[e % d], float_order(X[e])); }
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < d) {
+        part[((long long)blockIdx.x * 2 + 0) * kMaxD + threadIdx.x] = float_unorder(smin[threadIdx.x]);
+        part[((long long)blockIdx.x * 2 + 1) * kMaxD + threadIdx.x] = float_unorder(smax[threadIdx.x]);
+    }
 }
 
 void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s)
 {
-    unsigned grid = cdiv(n, 256);
-    if (grid > kBBGrid) grid = kBBGrid;
+    const int prefix = (int)(((16 - reinterpret_cast<uintptr_t>(X) % 16) % 16) / 4);
+    unsigned grid = (unsigned)d * kBBBlocksPerDim;                      // threads = 256 * grid: a multiple of d
+    const unsigned need = cdiv(cdiv(n * d, 4), 256);
+    if (need < grid) grid = (unsigned)d * std::max(1u, cdiv(need, d));
     DBuf<float> part((size_t)grid * 2 * kMaxD);
-    F3M_LAUNCH(minmax_kernel, grid, 256, 0, s, X, n, d, part.get());
+    F3M_LAUNCH(minmax_kernel, grid, 256, 0, s, X, n * d, d, std::min<long long>(prefix, n * d), part.get());
     check_launch("minmax");
     std::vector<float> h((size_t)grid * 2 * kMaxD);
     d2h(h.data(), part.get(), h.size(), s);

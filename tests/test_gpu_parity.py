@@ -231,6 +231,19 @@ def test_far_sweeps_match_per_level_interpolation(eng, monkeypatch, name):
     assert rel_l2(sweeps, per_level) < 5e-6
 
 
+def test_inputs_at_any_four_byte_alignment(eng):
+    """Views that start in the middle of an allocation (12-byte rows) are not 16-byte aligned."""
+    rng = np.random.default_rng(17)
+    big = dev(rng.random((30001, 3), dtype=f32))
+    b = dev(rng.standard_normal((30000, 1)).astype(f32))
+    for start in (1, 0):
+        view = big[start:start + 30000]
+        assert view.is_contiguous()
+        got = eng.kmvm(view, None, b, ls=0.5)
+        ref = eng.kmvm(view.clone(), None, b, ls=0.5)
+        assert np.array_equal(got.cpu().numpy(), ref.cpu().numpy())
+
+
 def test_columns_linearity_and_plan_reuse(eng, oracle):
     rng = np.random.default_rng(11)
     X = rng.random((40000, 3), dtype=f32)
