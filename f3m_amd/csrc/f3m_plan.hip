@@ -222,7 +222,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // level, the division of depth k+1 is started together with the list count of depth k whenever the
     // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
     DBuf<int> dres(16);          // [0..7]: four 64-bit list totals, [8,9]: X tree stats, [10,11]: Y tree stats
-    int hres[16];
+    alignas(8) int hres[16];
     auto wants_division = [&]() {
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
