@@ -117,6 +117,8 @@ def main():
     plan = engine.Plan(X, Y, **prm)
     work = plan.work()
     depth = plan.depth
+    nbx = plan.level_sizes(depth)["nbx"] if depth else 1
+    tiles_per_wave = 5 if (N // max(nbx, 1) + 31) // 32 == 5 else 4     # the library's choice (near_field)
     plan.close()
     F = 3 * d + 3                                  # flops per kernel evaluation (d sub, d mul, d-1 add, scale, exp, fma)
     near_flops = F * work["near_pairs"]
@@ -124,7 +126,7 @@ def main():
     achieved = near_flops * args.steps / max(near_t, 1e-12) / 1e12
     roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / PEAK_FP32_TFLOPS, "traffic": NEAR_TRAFFIC_BYTES if (N == 10_000_000 and d == 3) else None,
-                "kernel": "near_g_kernel<%d,4,1>" % d,
+                "kernel": "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
                 "note": "near field: exponents on the f16 matrix pipe (hi/lo-split operands, fp32 accumulate), exp2 + FMA on "
                         "the fp32 vector ALU; priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
                         "%.3e kernel evaluations/step x %d flops; traffic = HBM bytes per launch from rocprofv3 "

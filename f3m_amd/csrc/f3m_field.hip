@@ -597,7 +597,11 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     DBuf<int> flag((size_t)lx.nb), tileoff;
     F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
     check_launch("mark_rows");
-    constexpr int tpw = 4;      // target tiles of 32 per wavefront (2: 10.2 ms, 4: 9.2 ms, 8: 9.4 ms at N=1e7, d=3)
+    // target tiles of 32 per wavefront: 4 (2: 10.2 ms, 4: 9.2 ms, 5: 10.2 ms, 8: 9.4 ms at N=1e7, d=3, ten tiles
+    // per box), but 5 where a typical box has five tiles and would otherwise be cut into 4 + 1
+    // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms)
+    const long long avg_tiles = (tx.n / std::max(1, lx.nb) + 31) / 32;
+    const int tpw = (avg_tiles == 5 && nc == 1) ? 5 : 4;
     int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? tpw * 32 : bd * T, tileoff, s);
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
@@ -653,13 +657,18 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        if (nc == 4)                                                                                                  \
-            F3M_LAUNCH((near_g_kernel<DD, tpw, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
+        if (tpw == 5)                                                                                                 \
+            F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
+                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
+        else if (nc == 4)                                                                                             \
+            F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         else                                                                                                          \
-            F3M_LAUNCH((near_g_kernel<DD, tpw, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                             \
+            F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
