@@ -43,6 +43,9 @@ def clouds(name, rng):
     if name == "uniform5_243":       # config 4: 3^5 nodes per box
         return rng.random((200000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=243, min_points=1000,
                                                                small_field_points=300)
+    if name == "uniform5_1024":      # 4^5 nodes: the siblings of a box do not fit one workgroup and are split in two
+        return rng.random((1500000, 5), dtype=f32), None, dict(ls=1.5, nr_of_interpolation=1024, min_points=1000,
+                                                                small_field_points=300)
     if name == "uniform2":
         return rng.random((80000, 2), dtype=f32), None, dict(ls=0.2)
     if name == "uniform1":
@@ -171,7 +174,7 @@ def test_product_error_vs_fp64_exact(eng, oracle, name):
     assert err <= 1e-3 or err_oracle > 1e-3 / 1.5, (err, err_oracle)
 
 
-@pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform5_1024", "uniform3_varcomp"])
 def test_m2l_forms_agree(eng, monkeypatch, name):
     """Sibling-group separable M2L (default for one tree, d >= 3) against the per-box separable form
     and the direct form of the reference (F3M_src/1_d_conv.cu:741-817): same sums up to rounding."""
