@@ -1569,8 +1569,11 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         // sibling-group kernel: one tree, 3 <= d <= 5, n0 = n1 in 2..4, every far pair inside the 6^d cells
         int sibGS = 0, sibR2 = 0;
         size_t shsib = 0;
-        // (preferred to the per-box kernel for 4 x 4 x 4 nodes as well: 0.58 against 0.70 ms at N=1e7)
-        if (m2l_mode == 0 && &tx == &ty && d >= 3 && d <= 5 && ns.n[0] == ns.n[1] && ns.n[0] >= 2 && ns.n[0] <= 4 &&
+        // (preferred to the per-box kernel for 4 x 4 x 4 nodes as well once a level has a few hundred
+        // parents: 0.30 against 0.55 ms at depth 5 of N=1e7; with fewer parents the per-box kernel has
+        // more workgroups to offer)
+        const bool enough_parents = !q64 || (lx.depth >= 1 && tx.lev[lx.depth - 1].nb >= 256);
+        if (m2l_mode == 0 && enough_parents && &tx == &ty && d >= 3 && d <= 5 && ns.n[0] == ns.n[1] && ns.n[0] >= 2 && ns.n[0] <= 4 &&
             far.outliers == 0 && lx.depth >= 1) {
             const int N = ns.n[0];
             sibR2 = P / (N * N);

@@ -14,14 +14,20 @@ struct StageTimer {
     bool enabled = false;
     struct Span { int stage; hipEvent_t a, b; };
     std::vector<Span> spans;
+    std::vector<hipEvent_t> spare;      // events are kept for the next call
     double t[kNumStages] = {0};
     int n[kNumStages] = {0};
+    hipEvent_t take()
+    {
+        hipEvent_t e = nullptr;
+        if (!spare.empty()) { e = spare.back(); spare.pop_back(); }
+        else F3M_HIP(hipEventCreate(&e));
+        return e;
+    }
     void begin(int stage, hipStream_t s)
     {
         if (!enabled) return;
-        Span sp{stage, nullptr, nullptr};
-        F3M_HIP(hipEventCreate(&sp.a));
-        F3M_HIP(hipEventCreate(&sp.b));
+        Span sp{stage, take(), take()};
         F3M_HIP(hipEventRecord(sp.a, s));
         spans.push_back(sp);
     }
@@ -32,7 +38,7 @@ struct StageTimer {
     }
     void reset()
     {
-        for (auto &sp : spans) { (void)hipEventDestroy(sp.a); (void)hipEventDestroy(sp.b); }
+        for (auto &sp : spans) { spare.push_back(sp.a); spare.push_back(sp.b); }
         spans.clear();
         for (int i = 0; i < kNumStages; i++) { t[i] = 0; n[i] = 0; }
     }
@@ -45,8 +51,8 @@ struct StageTimer {
                 t[sp.stage] += ms * 1e-3;
                 n[sp.stage] += 1;
             }
-            (void)hipEventDestroy(sp.a);
-            (void)hipEventDestroy(sp.b);
+            spare.push_back(sp.a);
+            spare.push_back(sp.b);
         }
         spans.clear();
     }
