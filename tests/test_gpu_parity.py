@@ -63,6 +63,21 @@ NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "unif
          "uniform3_varcomp"]
 
 
+@pytest.mark.parametrize("fixture_name", __import__("golden_fixtures").names())
+def test_committed_oracle_fixtures(eng, fixture_name):
+    """tests/golden/oracle_fixtures.npz: box division and lists bit for bit, product within tolerance,
+    without running the oracle."""
+    import golden_fixtures as gf
+    print("case fixture", fixture_name, flush=True)
+    fx = gf.load()
+    X, Y, b, prm = gf.case(fx, fixture_name)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    gf.assert_plan_matches_fixture(plan, plan.depth, fx, fixture_name)
+    gf.assert_product_matches_fixture(plan.apply(dev(b)).cpu().numpy(), fx, fixture_name)
+    gf.assert_product_matches_fixture(eng.kmvm(dev(X), None if Y is None else dev(Y), dev(b), **prm).cpu().numpy(), fx,
+                                      fixture_name)
+
+
 @pytest.mark.parametrize("name", NAMES)
 def test_box_division_and_lists_bit_exact(eng, oracle, name):
     print("case", name, flush=True)
