@@ -390,7 +390,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     const bool per_level = fe && !strcmp(fe, "levels");
     for (int col = 0; col < c;) {
         const int left = c - col;
-        const int nc = left >= 2 ? 4 : 1;          // columns processed in this round (past `left`: zero weights)
+        const int nc = left >= 2 ? 4 : 1;          // columns processed in this pass (past `left`: zero weights)
         const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
