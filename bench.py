@@ -51,7 +51,7 @@ def main():
     ap.add_argument("--n", type=int, default=10_000_000)
     ap.add_argument("--d", type=int, default=3)
     ap.add_argument("--dist", default="uniform", choices=["uniform", "normal", "clustered"],
-                    help="clustered = BASELINE config 3: X from 50 anisotropic Gaussians, Y (n/10 points) uniform over "
+                    help="clustered = the asymmetric benchmark configuration: X from 50 anisotropic Gaussians, Y (n/10 points) uniform over "
                          "X's bounding box, two trees")
     ap.add_argument("--ls", type=float, default=1.0)
     ap.add_argument("--nodes", type=int, default=64)

@@ -1,4 +1,4 @@
-"""FALKON kernel ridge regression on the synthetic problem of BASELINE config 5.
+"""FALKON kernel ridge regression on a synthetic problem (the fifth benchmark configuration of this project).
 
     python -m f3m_amd.conjugate_gradient.run_krr --n 10000000 --m 100000 --maxiter 20
 

@@ -1,4 +1,4 @@
-"""FALKON drivers on the engine (BASELINE config 5 in miniature): the Nystrom coefficients must solve
+"""FALKON drivers on the engine (the kernel-ridge-regression benchmark configuration in miniature): the Nystrom coefficients must solve
 (K_nm^T K_nm + lambda n (K_mm + eps M I)) alpha = K_nm^T y (eps M I is the preconditioner's jitter, which
 the algorithm carries into the system it solves); a dense fp64 solve gives that in closed form."""
 import numpy as np
