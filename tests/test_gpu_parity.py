@@ -277,6 +277,21 @@ def test_columns_linearity_and_plan_reuse(eng, oracle):
     assert np.array_equal(one_shot, o)                   # deterministic: no float atomics anywhere
 
 
+@pytest.mark.parametrize("c", [2, 5, 6, 9])
+def test_column_groups(eng, c):
+    """Columns are multiplied four at a time, a last single column on its own; every column must equal
+    the product of that column alone, bit for bit, for two trees as well."""
+    rng = np.random.default_rng(c)
+    X = rng.random((30000, 3), dtype=f32)
+    Y = rng.random((20000, 3), dtype=f32)
+    b = rng.standard_normal((20000, c)).astype(f32)
+    plan = eng.Plan(dev(X), dev(Y), ls=0.4)
+    all_cols = plan.apply(dev(b)).cpu().numpy()
+    for col in range(c):
+        one = plan.apply(dev(b[:, col:col + 1])).cpu().numpy()
+        assert np.array_equal(one[:, 0], all_cols[:, col]), col
+
+
 def test_edge_cases(eng, oracle):
     import torch
     from f3m_amd.capi import F3MError
