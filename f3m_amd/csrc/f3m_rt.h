@@ -68,12 +68,15 @@ public:
     {
         if (bytes == 0) bytes = 256;
         bytes = (bytes + 255) & ~size_t(255);
+        int dev = 0;
+        (void)hipGetDevice(&dev);                   // blocks are cached per device
         std::lock_guard<std::mutex> g(mu_);
-        auto it = free_.lower_bound(bytes);
-        if (it != free_.end() && it->first <= bytes * 2 + (1 << 20)) {
+        auto &fr = free_[dev];
+        auto it = fr.lower_bound(bytes);
+        if (it != fr.end() && it->first <= bytes * 2 + (1 << 20)) {
             void *p = it->second;
-            live_[p] = it->first;
-            free_.erase(it);
+            live_[p] = Block{it->first, dev};
+            fr.erase(it);
             return p;
         }
         void *p = nullptr;
@@ -83,7 +86,7 @@ public:
             e = hipMalloc(&p, bytes);
         }
         if (e != hipSuccess) throw Error(101, fmt("device allocation of %zu bytes failed: %s", bytes, hipGetErrorString(e)));
-        live_[p] = bytes;
+        live_[p] = Block{bytes, dev};
         reserved_ += bytes;
         return p;
     }
@@ -93,7 +96,7 @@ public:
         std::lock_guard<std::mutex> g(mu_);
         auto it = live_.find(p);
         if (it == live_.end()) return;
-        free_.insert({it->second, p});
+        free_[it->second.dev].insert({it->second.bytes, p});
         live_.erase(it);
     }
     void release_cached()
@@ -104,14 +107,16 @@ public:
     size_t reserved() const { return reserved_; }
 
 private:
+    struct Block { size_t bytes; int dev; };
     void release_cached_locked()
     {
-        for (auto &kv : free_) { (void)hipFree(kv.second); reserved_ -= kv.first; }
+        for (auto &d : free_)
+            for (auto &kv : d.second) { (void)hipFree(kv.second); reserved_ -= kv.first; }
         free_.clear();
     }
     std::mutex mu_;
-    std::multimap<size_t, void *> free_;
-    std::map<void *, size_t> live_;
+    std::map<int, std::multimap<size_t, void *>> free_;
+    std::map<void *, Block> live_;
     size_t reserved_ = 0;
 };
 

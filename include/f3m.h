@@ -6,7 +6,8 @@
  * void* (NULL = the default stream).  Every function returns 0 on success or a positive error
  * code; f3m_last_error() then returns a message for the calling thread.  Calls are synchronous:
  * the stream is idle when they return.  One call at a time per device (the engine keeps a cache of
- * device buffers that concurrent calls would share).
+ * device buffers, per device, that concurrent calls would share).  The device of the pointers must be
+ * the calling thread's current device (hipSetDevice), for plans during create, apply and destroy.
  *
  * The citations name the interface of the upstream reference (repository MrHuff/F3M) that each
  * entry point replaces.
