@@ -529,21 +529,28 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
                     for (int c = 0; c < NC; c++) bq[c][r] = in ? bq[c][r] : 0.f;
                 }
             }
+            auto tile = [&](int q) {
+                f32x16 t;
 #pragma unroll
-            for (int q = 0; q < TPW; q++) {
-                if (q < nlive) {                     // uniform per wavefront
-                    f32x16 t;
+                for (int r = 0; r < 16; r++) t[r] = 0.f;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) t[r] = 0.f;
+                for (int n = 0; n < NS; n++) t = mfma_32x32x16_f16(a[n], bop[q][n], t);
 #pragma unroll
-                    for (int n = 0; n < NS; n++) t = mfma_32x32x16_f16(a[n], bop[q][n], t);
+                for (int r = 0; r < 16; r++) {
+                    const float e = fast_exp2(t[r]);
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const float e = fast_exp2(t[r]);
-#pragma unroll
-                        for (int c = 0; c < NC; c++) acc[q][c] = fmaf(e, bq[c][r], acc[q][c]);
-                    }
+                    for (int c = 0; c < NC; c++) acc[q][c] = fmaf(e, bq[c][r], acc[q][c]);
                 }
+            };
+            if (nlive == TPW) {
+                // the usual case, free of branches: the compiler may start the matrix products of the
+                // next tiles while the vector ALU works on the exponentials of this one
+#pragma unroll
+                for (int q = 0; q < TPW; q++) tile(q);
+            } else {
+#pragma unroll
+                for (int q = 0; q < TPW; q++)
+                    if (q < nlive) tile(q);              // uniform per wavefront
             }
         }
       }
