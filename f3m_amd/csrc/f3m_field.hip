@@ -14,17 +14,32 @@ constexpr float kLog2e = 1.4426950408889634f;
 // ------------------------------------------------------------------------------------------------
 // permutations between caller order and sorted order
 
-__global__ void gather_points_kernel(const float *__restrict__ X, const int *__restrict__ perm, long long n, int d,
+template <int K> struct __attribute__((aligned(4))) fvec { float v[K]; };   // K floats at any 4-byte boundary
+
+// A row of X sits at a random place: it is fetched with one load of D floats, so that the row costs
+// one request to the memory system rather than D.
+template <int D>
+__global__ void gather_points_kernel(const float *__restrict__ X, const int *__restrict__ perm, long long n,
                                      float *__restrict__ pts)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    long long src = perm[i];
-    for (int j = 0; j < d; j++) pts[(long long)j * n + i] = X[src * d + j];
+    const fvec<D> row = *reinterpret_cast<const fvec<D> *>(X + (long long)perm[i] * D);
+#pragma unroll
+    for (int j = 0; j < D; j++) pts[(long long)j * n + i] = row.v[j];
 }
 void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s)
 {
-    F3M_LAUNCH(gather_points_kernel, cdiv(n, 256), 256, 0, s, X, perm, n, d, pts);
+#define F3M_CASE(DD)                                                                                  \
+    case DD:                                                                                          \
+        F3M_LAUNCH((gather_points_kernel<DD>), cdiv(n, 256), 256, 0, s, X, perm, n, pts);             \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
     check_launch("gather_points");
 }
 
@@ -1205,8 +1220,6 @@ __device__ inline void sib_ext_digits(int e, int *dg)
         else { dg[j] = 2 + ((bits >> pos) & 1); pos++; }
     }
 }
-
-template <int K> struct __attribute__((aligned(4))) fvec { float v[K]; };
 
 template <int D, int N>
 __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
