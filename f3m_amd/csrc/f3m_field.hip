@@ -324,8 +324,9 @@ __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, in
     return v;
 }
 
-// Source operands, once per tree level: point i of box b, shifted to the centre of b and scaled,
-// as the rows (2y', -|y'|^2) of the matrix product in split-f16 form.  Layout: ops[(n*2 + h)*stride + i]
+// Source operands, once per tree level: point i of box b, shifted to the centre of b's parent cell
+// (near_anchor; shared by the boxes of that parent, which lets near_g_kernel take neighbouring boxes
+// in one go) and scaled, as the rows (2y', -|y'|^2) of the matrix product in split-f16 form.  Layout: ops[(n*2 + h)*stride + i]
 // = the eight inner slots of half-wave h of instruction n; stride = npoints + 32 (the tail is zero so
 // that a wavefront may read one padded tile past the end).
 // need (nullable) = prefix count of the boxes that occur as sources (nb+1 entries): operands are then
@@ -333,10 +334,18 @@ __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, in
 // read as the padding of a box's last tile.
 constexpr int kOpsBlock = 256;
 
+// Reference point of the near-field operands of a box: the centre of its parent cell, computed from
+// the integer cell so that every box of the parent (and both kernels) get the same bits.
+__device__ __forceinline__ float near_anchor(const Geo &geo, float edge, int cell, int k)
+{
+    return geo.origin[k] + (float)(2 * (cell >> 1) + 1) * edge;
+}
+
 template <int D>
 __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *__restrict__ ys, long long M,
                                                                   const int *__restrict__ off, int nb,
-                                                                  const float *__restrict__ ctr, float sc, long long stride,
+                                                                  const int *__restrict__ cell, Geo geo, float edge,
+                                                                  float sc, long long stride,
                                                                   const int *__restrict__ need, h8 *__restrict__ ops)
 {
     constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
@@ -370,7 +379,7 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
         for (int k = 0; k < C; k++) {
             float v;
             if (k < D) {
-                float y = sc * (ys[(long long)k * M + i] - ctr[(long long)box * D + k]);
+                float y = sc * (ys[(long long)k * M + i] - near_anchor(geo, edge, cell[(long long)box * D + k], k));
                 ny2 -= y * y;
                 v = 2.f * y;
             } else if (k == D) {
@@ -409,9 +418,9 @@ template <int D, int TPW, int NC>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
-    const int *__restrict__ offy, const float *__restrict__ ctry, const int *__restrict__ pairs,
-    const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc, int stripe, int nsplit,
-    float *__restrict__ part)
+    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
+    int stripe, int nsplit, float *__restrict__ part)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
@@ -466,24 +475,41 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         thi = (int)((long long)ttot * (slice + 1) / nsplit);
     }
     int tcur = 0;                                    // tiles of the row before the current y box
-    // the list is consumed 64 y boxes at a time: every lane fetches the range and centre of one y box,
-    // then the wavefront walks through them (one round of memory latency per 64 boxes)
+    // The list is consumed 64 y boxes at a time: every lane fetches the range and the anchor of one y
+    // box, then the wavefront walks through them (one round of memory latency per 64 boxes).  Boxes
+    // that follow each other in the list, in memory and under one parent share their anchor and are
+    // taken as one run of sources: one set of target operands and one padded last tile per run.
     for (int mb = m0; mb < m1; mb += 64) {
       const int mi = mb + lane;
-      int s0v = 0, s1v = 0;
+      int s0v = 0, s1v = 0, byv = -2;
+      int pcv[D];
       float cyv[D];
 #pragma unroll
-      for (int k = 0; k < D; k++) cyv[k] = 0.f;
+      for (int k = 0; k < D; k++) { cyv[k] = 0.f; pcv[k] = 0; }
       if (mi < m1) {
-          const int byv = pairs[2 * (long long)mi + 1];
+          byv = pairs[2 * (long long)mi + 1];
           s0v = offy[byv];
           s1v = offy[byv + 1];
 #pragma unroll
-          for (int k = 0; k < D; k++) cyv[k] = ctry[(long long)byv * D + k];
+          for (int k = 0; k < D; k++) {
+              const int cl = celly[(long long)byv * D + k];
+              pcv[k] = cl >> 1;
+              cyv[k] = near_anchor(geoy, edgey, cl, k);
+          }
       }
       const int mcnt = min(64, m1 - mb);
-      for (int mj = 0; mj < mcnt; mj++) {
-        int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mj);
+      // continues the run of the lane before (sliced lists keep one box per run: slices count tiles per box)
+      const int before = (lane + 63) & 63;
+      bool cont = (wave_shfl_i(byv, before) + 1 == byv);
+#pragma unroll
+      for (int k = 0; k < D; k++) cont = (wave_shfl_i(pcv[k], before) == pcv[k]) && cont;
+      cont = cont && lane > 0 && mi < m1 && nsplit == 1;
+      unsigned long long heads = wave_ballot(mi < m1 && !cont);
+      while (heads) {
+        const int mj = __builtin_ctzll(heads);
+        heads &= heads - 1;
+        const int mlast = heads ? __builtin_ctzll(heads) - 1 : mcnt - 1;
+        int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mlast);
         if (nsplit > 1) {                            // keep the part of this box that lies in the slice
             const int nt = (s1 - s0 + 31) >> 5;
             const int a = max(tlo, tcur), b = min(thi, tcur + nt);
@@ -496,7 +522,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         float cy[D];
 #pragma unroll
         for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
-        // target operands relative to the centre of this y box
+        // target operands relative to the anchor of this run
         h8 bop[TPW][NS];
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
@@ -647,7 +673,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
         F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
-                   ly.off.get(), ly.nb, ly.ctr.get(), sc, stride, only_list ? need.get() : (const int *)nullptr,      \
+                   ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
+                   only_list ? need.get() : (const int *)nullptr,                                                     \
                    reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
         break;
             switch (d) {
@@ -682,17 +709,17 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         if (tpw == 5)                                                                                                 \
             F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         else if (nc == 4)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         else                                                                                                          \
             F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.ctr.get(), list.pairs.get(), list.rowptr.get(),        \
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
         break;
         switch (d) {

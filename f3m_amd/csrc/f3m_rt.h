@@ -293,7 +293,15 @@ __device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __s
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half_t;
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ half_t to_half(float f) { return (_Float16)f; }
+// Rounds the fp32 value it is given.  The empty asm statement hides where f comes from: fused with a
+// preceding multiply-add (v_fma_mixlo_f16) the conversion would round the unrounded sum instead, and
+// code that also uses the fp32 value (lo = f - hi) would then see two different roundings of f at
+// exact ties, an error of one f16 unit in the last place.
+__device__ __forceinline__ half_t to_half(float f)
+{
+    asm("" : "+v"(f));
+    return (_Float16)f;
+}
 __device__ __forceinline__ float half_to_float(half_t h) { return (float)h; }
 // D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation (v_mfma_f32_32x32x16_f16): lane l
 // supplies row l%32 of A and column l%32 of B for the eight inner indices of its half-wave and holds
