@@ -53,6 +53,9 @@ struct PairList {
     // the parent of the x box nor a child of a parent two cells away along one axis (a parent pair
     // exactly on the far threshold, kept by rounding); -1 = not counted.  Expected to be 0.
     long long outliers = -1;
+    // x boxes with a non-empty row, their points, and the work items they make when cut into pieces of
+    // 128 and of 160 targets (near-field launch shapes); rows = -1: not counted
+    long long rows = -1, row_points = 0, items128 = 0, items160 = 0;
 };
 
 struct ClassifyParams {
@@ -98,7 +101,7 @@ struct ListsPending {
 void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
                   ListsPending &pend, long long *dtot, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
-                  const ClassifyParams &cp, PlanLevel &out, hipStream_t s);
+                  const ClassifyParams &cp, PlanLevel &out, long long *drow /* 8 zeroed words or null */, hipStream_t s);
 void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
 void build_rowptr(PairList &l, int nbx, hipStream_t s);

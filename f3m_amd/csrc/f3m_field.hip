@@ -420,7 +420,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
     const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
-    int stripe, int nsplit, float *__restrict__ part)
+    int stripe, int nsplit, float *__restrict__ part, int nitems)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = (3 * C + 15) / 16;
@@ -436,8 +436,8 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         vblock = (r / stripe) * (8 * stripe) + xcd * stripe + (r % stripe);
     }
     // work item: TPW*32 targets of one box; with few targets and long lists (nsplit > 1) the list of a
-    // work item is cut into nsplit slices, one wavefront each, whose sums go to `part` and are added up
-    // in a fixed order afterwards
+    // work item is cut into nsplit slices, one wavefront each, whose sums go to `part` (nsplit x NC x
+    // nitems x TPW*32 floats, indexed by work item) and are added up in a fixed order afterwards
     const int wfull = vblock * kNearWavesPerBlock + (threadIdx.x >> 6);
     const int wid = wfull / nsplit, slice = wfull % nsplit;
     if (wid >= tileoff[nbx]) return;
@@ -603,24 +603,29 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
         for (int c = 0; c < NC; c++) {
             float total = acc[q][c] + wave_shfl_xor_f(acc[q][c], 32);
             if (half == 0 && i < x1) {
-                if (nsplit > 1) part[((long long)slice * NC + c) * N + i] = total;
+                if (nsplit > 1) part[(((long long)slice * NC + c) * nitems + wid) * (TPW * 32) + q * 32 + col] = total;
                 else outs[c * ostride + i] += total;
             }
         }
     }
 }
 
-// outs += the slices of a split near field, in slice order
-__global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, int nc, long long N,
+// outs += the slices of a split near field, in slice order; one thread per target slot of a work item
+__global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, int nc, int nitems, int tile,
+                                   const int *__restrict__ tileoff, int nbx, const int *__restrict__ offx,
                                    float *__restrict__ outs, long long ostride)
 {
-    long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= N * nc) return;
-    const int c = (int)(e / N);
-    const long long i = e % N;
-    float sum = 0.f;
-    for (int sl = 0; sl < nsplit; sl++) sum += part[((long long)sl * nc + c) * N + i];
-    outs[c * ostride + i] += sum;
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int wid = (int)(e / tile), r = (int)(e % tile);
+    if (wid >= nitems || wid >= tileoff[nbx]) return;
+    const int bx = find_box(tileoff, nbx, wid);
+    const int i = offx[bx] + (wid - tileoff[bx]) * tile + r;
+    if (i >= offx[bx + 1]) return;
+    for (int c = 0; c < nc; c++) {
+        float sum = 0.f;
+        for (int sl = 0; sl < nsplit; sl++) sum += part[(((long long)sl * nc + c) * nitems + wid) * tile + r];
+        outs[c * ostride + i] += sum;
+    }
 }
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
@@ -648,9 +653,12 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // target tiles of 32 per wavefront: 4 (2: 10.2 ms, 4: 9.2 ms, 5: 10.2 ms, 8: 9.4 ms at N=1e7, d=3, ten tiles
     // per box), but 5 where a typical box has five tiles and would otherwise be cut into 4 + 1
     // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms)
-    const long long avg_tiles = (tx.n / std::max(1, lx.nb) + 31) / 32;
-    const int tpw = (avg_tiles == 5 && nc == 1) ? 5 : 4;
+    // Where the plan has counted the rows of the list, "typical" is the mean over the listed boxes and the
+    // number of work items is exact; otherwise the mean over all boxes and an upper bound.
+    const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
+    const int tpw = ((avg_points + 31) / 32 == 5 && nc == 1) ? 5 : 4;
     int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? tpw * 32 : bd * T, tileoff, s);
+    if (use_mfma && list.rows >= 0) ntiles = (int)std::max<long long>(1, tpw == 5 ? list.items160 : list.items128);
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
         const int C = d + 2, NS = (3 * C + 15) / 16;
@@ -697,10 +705,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
             nsplit = std::min(128, (int)cdiv(target, std::max(1, ntiles)));
         }
         DBuf<float> part;
-        if (nsplit > 1) {
-            part.reset((size_t)nsplit * nc * tx.n);
-            F3M_HIP(hipMemsetAsync(part.get(), 0, sizeof(float) * (size_t)nsplit * nc * tx.n, s));
-        }
+        if (nsplit > 1) part.reset((size_t)nsplit * nc * ntiles * tpw * 32);   // every slot of a live work item is written
         int nblk = (int)cdiv((long long)ntiles * nsplit, kNearWavesPerBlock);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
@@ -710,17 +715,17 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
             F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles);                                         \
         else if (nc == 4)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles);                                         \
         else                                                                                                          \
             F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get());                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles);                                         \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -730,7 +735,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #undef F3M_CASE
         if (nsplit > 1) {
             check_launch("near_g");
-            F3M_LAUNCH(near_reduce_kernel, cdiv(tx.n * nc, 256), 256, 0, s, part.get(), nsplit, nc, tx.n, outs, ostride);
+            F3M_LAUNCH(near_reduce_kernel, cdiv((long long)ntiles * tpw * 32, 256), 256, 0, s, part.get(), nsplit, nc, ntiles,
+                       tpw * 32, tileoff.get(), lx.nb, lx.off.get(), outs, ostride);
         }
     } else {
         timer_begin(kNear, s);

@@ -151,7 +151,7 @@ void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipS
     F3M_LAUNCH(minmax_kernel, grid, 256, 0, s, X, n * d, d, std::min<long long>(prefix, n * d), part.get());
     check_launch("minmax");
     std::vector<float> h((size_t)grid * 2 * kMaxD);
-    d2h(h.data(), part.get(), h.size(), s);
+    fetch_small(h.data(), part.get(), h.size(), s);
     for (int j = 0; j < d; j++) {
         mn[j] = h[j];
         mx[j] = h[kMaxD + j];
@@ -700,6 +700,34 @@ __global__ void list_totals_kernel(const long long *__restrict__ pos, long long 
     if (threadIdx.x < 3) out[threadIdx.x] = pos[threadIdx.x * stride + stride - 1];   // out[3]: outlier counter
 }
 
+// Row statistics of the small and the keep list of a level: out[4c .. 4c+3] (c = 0 small, 1 keep) += x
+// boxes with pairs, their points, their pieces of 128 and of 160 points (out is zero before).
+constexpr int kRowStatBlock = 256;
+__global__ void __launch_bounds__(kRowStatBlock) list_rowstats_kernel(const int *__restrict__ rowptr_small,
+                                                                       const int *__restrict__ rowptr_keep,
+                                                                       const int *__restrict__ offx, int nbx,
+                                                                       unsigned long long *__restrict__ out)
+{
+    __shared__ unsigned long long acc[8];
+    if (threadIdx.x < 8) acc[threadIdx.x] = 0;
+    __syncthreads();
+    const int b = blockIdx.x * kRowStatBlock + threadIdx.x;
+    if (b < nbx) {
+        const unsigned long long n = (unsigned long long)(offx[b + 1] - offx[b]);
+        for (int c = 0; c < 2; c++) {
+            const int *rp = c ? rowptr_keep : rowptr_small;
+            if (rp[b + 1] > rp[b]) {
+                atomicAdd(&acc[4 * c + 0], 1ull);
+                atomicAdd(&acc[4 * c + 1], n);
+                atomicAdd(&acc[4 * c + 2], (n + 127) / 128);
+                atomicAdd(&acc[4 * c + 3], (n + 159) / 160);
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < 8 && acc[threadIdx.x]) atomicAdd(&out[threadIdx.x], acc[threadIdx.x]);
+}
+
 __global__ void rowptr_kernel(const int *__restrict__ pairs, long long n, int nbx, int *__restrict__ rowptr)
 {
     int b = blockIdx.x * blockDim.x + threadIdx.x;
@@ -750,7 +778,7 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
 }
 
 void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
-                  const ClassifyParams &cp, PlanLevel &out, hipStream_t s)
+                  const ClassifyParams &cp, PlanLevel &out, long long *drow, hipStream_t s)
 {
     out.far.n = out.small_.n = out.keep.n = 0;
     if (!pend.active) return;
@@ -777,6 +805,11 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
                out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
                out.far.rowptr.get(), out.keep.rowptr.get());
     check_launch("lists_write");
+    if (drow != nullptr) {
+        F3M_LAUNCH(list_rowstats_kernel, cdiv(nbx, kRowStatBlock), kRowStatBlock, 0, s, out.small_.rowptr.get(),
+                   out.keep.rowptr.get(), lx.off.get(), nbx, reinterpret_cast<unsigned long long *>(drow));
+        check_launch("list_rowstats");
+    }
     pend.pos.free();
     pend.active = false;
 }

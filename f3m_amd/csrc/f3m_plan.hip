@@ -221,7 +221,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     F3M_HIP(hipMemsetAsync(root.pairs.get(), 0, 2 * sizeof(int), s));     // the root pair (0,0)
     build_rowptr(root, 1, s);
     const PairList *keep = &root;
-    P->levels.reserve(40);   // `keep` points into this vector: it must not reallocate
+    P->levels.reserve(64);   // `keep` points into this vector: it must not reallocate
     // Loop of F3M_src/n_tree.cu:1075 (one tree) and :1099 (two trees): divide while the keep list is not
     // empty and the fullest box of each tree holds more than min_points points.  The host has to fetch
     // two things per level, the box counts of the division and the list sizes; to wait only once per
@@ -229,6 +229,11 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
     DBuf<int> dres(16);          // [0..7]: four 64-bit list totals, [8,9]: X tree stats, [10,11]: Y tree stats
     alignas(8) int hres[16];
+    // row statistics of the small and keep lists, 8 words per level; nothing at plan time depends on
+    // them, so they are fetched once at the end instead of with the per-level wait
+    constexpr int kMaxLevels = 40;
+    DBuf<long long> drow((size_t)8 * kMaxLevels);
+    F3M_HIP(hipMemsetAsync(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s));
     auto wants_division = [&]() {
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
@@ -243,7 +248,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     };
     if (need_tree && wants_division()) {
         start_division();
-        d2h(hres, dres.get(), 16, s);
+        fetch_small(hres, dres.get(), 16, s);
         finish_division();
         for (;;) {
             const int k = (int)P->tx.lev.size() - 1;
@@ -255,8 +260,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
             const bool ahead = wants_division();
             if (ahead) start_division();
-            d2h(hres, dres.get(), 16, s);
-            lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L, s);
+            fetch_small(hres, dres.get(), 16, s);
+            F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
+            lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
+                         drow.get() + 8 * (P->levels.size() - 1), s);
             if (ahead) finish_division();
             L.num_nodes = prm->nr_of_interpolation;
             if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
@@ -283,6 +290,16 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         if (!sym) {
             P->Yraw.reset((size_t)M * d);
             F3M_HIP(hipMemcpyAsync(P->Yraw.get(), Y, sizeof(float) * (size_t)M * d, hipMemcpyDeviceToDevice, s));
+        }
+    }
+    if (!P->levels.empty()) {
+        std::vector<long long> hrow(8 * P->levels.size());
+        fetch_small(hrow.data(), drow.get(), hrow.size(), s);
+        for (size_t l = 0; l < P->levels.size(); l++) {
+            const long long *r = hrow.data() + 8 * l;
+            PairList &sm = P->levels[l].small_, &kp = P->levels[l].keep;
+            sm.rows = r[0], sm.row_points = r[1], sm.items128 = r[2], sm.items160 = r[3];
+            kp.rows = r[4], kp.row_points = r[5], kp.items128 = r[6], kp.items160 = r[7];
         }
     }
     F3M_HIP(hipStreamSynchronize(s));

@@ -151,6 +151,55 @@ inline void d2h(T *dst, const T *src, size_t n, hipStream_t s)
     F3M_HIP(hipMemcpyAsync(dst, src, n * sizeof(T), hipMemcpyDeviceToHost, s));
     F3M_HIP(hipStreamSynchronize(s));
 }
+// Small results the host waits for (box counts, list sizes): a one-workgroup kernel stores them into
+// pinned host memory and the host waits for the stream; a copy into pageable memory costs a staged
+// copy command on top of that.  Pinned blocks are kept for the life of the process.
+#ifdef F3M_CPU_EMU
+template <typename T>
+inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s) { d2h(dst, src, n, s); }
+#else
+constexpr size_t kPinnedBytes = 64 << 10;
+class PinnedBlock {
+public:
+    PinnedBlock()
+    {
+        {
+            std::lock_guard<std::mutex> g(mu());
+            if (!spare().empty()) { p_ = spare().back(); spare().pop_back(); }
+        }
+        if (!p_) F3M_HIP(hipHostMalloc(&p_, kPinnedBytes, hipHostMallocPortable | hipHostMallocMapped));
+    }
+    ~PinnedBlock()
+    {
+        std::lock_guard<std::mutex> g(mu());
+        spare().push_back(p_);
+    }
+    PinnedBlock(const PinnedBlock &) = delete;
+    PinnedBlock &operator=(const PinnedBlock &) = delete;
+    void *get() const { return p_; }
+
+private:
+    static std::mutex &mu() { static std::mutex m; return m; }
+    static std::vector<void *> &spare() { static std::vector<void *> v; return v; }
+    void *p_ = nullptr;
+};
+template <typename T>
+__global__ void export_kernel(const T *__restrict__ src, T *__restrict__ dst, int n)
+{
+    for (int i = threadIdx.x; i < n; i += blockDim.x) dst[i] = src[i];
+}
+template <typename T>
+inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s)
+{
+    if (n * sizeof(T) > kPinnedBytes) { d2h(dst, src, n, s); return; }
+    PinnedBlock blk;
+    hipLaunchKernelGGL(export_kernel<T>, dim3(1), dim3(256), 0, s, src, static_cast<T *>(blk.get()), (int)n);
+    F3M_HIP(hipGetLastError());
+    F3M_HIP(hipStreamSynchronize(s));
+    memcpy(dst, blk.get(), n * sizeof(T));
+}
+#endif
+
 template <typename T>
 inline void h2d(T *dst, const T *src, size_t n, hipStream_t s)
 {
