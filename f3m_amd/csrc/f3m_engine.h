@@ -104,6 +104,7 @@ void lists_finish(ListsPending &pend, const long long *htot, const PairList &kee
                   const ClassifyParams &cp, PlanLevel &out, long long *drow /* 8 zeroed words or null */, hipStream_t s);
 void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
+void exclusive_scan_i64_batched(const long long *in, long long n, long long pitch, int nch, long long *out, hipStream_t s);
 void build_rowptr(PairList &l, int nbx, hipStream_t s);
 // slot of a key in a table of `capacity` slots (host and device use the same function)
 uint32_t hash_slot_host(uint32_t key, uint32_t capacity);

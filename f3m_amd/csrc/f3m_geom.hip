@@ -78,6 +78,108 @@ static void exclusive_scan(const Tin *in, long long n, Tout *out, hipStream_t s)
     }
 }
 
+// Batched form: `nch` arrays of n elements each, `pitch` apart in `in` and in `out` (n+1 outputs per
+// array), scanned independently with three launches in all (one, if an array fits one tile).
+template <typename T>
+__global__ void scan_tile_batched_kernel(const T *__restrict__ in, long long n, long long pitch, unsigned ntiles,
+                                         T *__restrict__ out, T *__restrict__ tilesum)
+{
+    __shared__ T sh[kScanBlock];
+    const int tid = threadIdx.x;
+    const unsigned ch = blockIdx.x / ntiles, tile = blockIdx.x % ntiles;
+    in += ch * pitch;
+    out += ch * pitch;
+    const long long base = (long long)tile * kScanTile + (long long)tid * kScanItems;
+    T v[kScanItems];
+    T sum = 0;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        long long i = base + e;
+        v[e] = (i < n) ? in[i] : (T)0;
+        sum += v[e];
+    }
+    sh[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanBlock; off <<= 1) {
+        T t = (tid >= off) ? sh[tid - off] : (T)0;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    T run = sh[tid] - sum;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        long long i = base + e;
+        if (i <= n) out[i] = run;
+        run += v[e];
+    }
+    if (tid == kScanBlock - 1) tilesum[blockIdx.x] = sh[tid];
+}
+
+// tile sums of one array (at most kScanTile of them) -> their exclusive prefixes, in place; one workgroup per array
+template <typename T>
+__global__ void scan_sums_batched_kernel(T *__restrict__ tilesum, unsigned ntiles)
+{
+    __shared__ T sh[kScanBlock];
+    const int tid = threadIdx.x;
+    T *ts = tilesum + (size_t)blockIdx.x * ntiles;
+    T v[kScanItems];
+    T sum = 0;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        unsigned i = (unsigned)tid * kScanItems + e;
+        v[e] = (i < ntiles) ? ts[i] : (T)0;
+        sum += v[e];
+    }
+    sh[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanBlock; off <<= 1) {
+        T t = (tid >= off) ? sh[tid - off] : (T)0;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    T run = sh[tid] - sum;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        unsigned i = (unsigned)tid * kScanItems + e;
+        if (i < ntiles) ts[i] = run;
+        run += v[e];
+    }
+}
+
+template <typename T>
+__global__ void scan_add_batched_kernel(T *__restrict__ out, long long n1, long long pitch, unsigned ntiles,
+                                        const T *__restrict__ tileoff)
+{
+    const unsigned ch = blockIdx.x / ntiles, tile = blockIdx.x % ntiles;
+    out += ch * pitch;
+    long long i = (long long)tile * kScanTile + threadIdx.x;
+    T add = tileoff[blockIdx.x];
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++, i += kScanBlock)
+        if (i < n1) out[i] += add;
+}
+
+void exclusive_scan_i64_batched(const long long *in, long long n, long long pitch, int nch, long long *out, hipStream_t s)
+{
+    const long long n1 = n + 1;
+    const unsigned ntiles = cdiv(n1, kScanTile);
+    if (ntiles > (unsigned)kScanTile) {              // tile sums of an array would not fit one workgroup
+        for (int c = 0; c < nch; c++) exclusive_scan_i64(in + c * pitch, n, out + c * pitch, s);
+        return;
+    }
+    DBuf<long long> tilesum((size_t)ntiles * nch);
+    F3M_LAUNCH((scan_tile_batched_kernel<long long>), ntiles * nch, kScanBlock, 0, s, in, n, pitch, ntiles, out, tilesum.get());
+    check_launch("scan_tile_batched");
+    if (ntiles > 1) {
+        F3M_LAUNCH((scan_sums_batched_kernel<long long>), nch, kScanBlock, 0, s, tilesum.get(), ntiles);
+        check_launch("scan_sums_batched");
+        F3M_LAUNCH((scan_add_batched_kernel<long long>), ntiles * nch, kScanBlock, 0, s, out, n1, pitch, ntiles, tilesum.get());
+        check_launch("scan_add_batched");
+    }
+}
+
 void exclusive_scan_i32(const int *in, long long n, int *out, hipStream_t s) { exclusive_scan<int, int>(in, n, out, s); }
 void exclusive_scan_i64(const long long *in, long long n, long long *out, hipStream_t s)
 {
@@ -772,7 +874,7 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                cellx, ly.cell.get(), outl, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
-    for (int c = 0; c < 3; c++) exclusive_scan_i64(cnt.get() + c * pend.stride, nbx, pend.pos.get() + c * pend.stride, s);
+    exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
     F3M_LAUNCH(list_totals_kernel, 1, 64, 0, s, pend.pos.get(), pend.stride, dtot);
     check_launch("list_totals");
 }

@@ -16,6 +16,7 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <chrono>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -152,13 +153,16 @@ inline void d2h(T *dst, const T *src, size_t n, hipStream_t s)
     F3M_HIP(hipStreamSynchronize(s));
 }
 // Small results the host waits for (box counts, list sizes): a one-workgroup kernel stores them into
-// pinned host memory and the host waits for the stream; a copy into pageable memory costs a staged
-// copy command on top of that.  Pinned blocks are kept for the life of the process.
+// pinned host memory followed by a sequence number, and the host watches that number instead of
+// waiting for the stream (a stream wait costs some 15 us more, a copy into pageable memory a staged
+// copy command on top).  After kSpinLimitMs of watching the host falls back to the stream wait, which
+// also reports a failed kernel.  Pinned blocks are kept for the life of the process.
 #ifdef F3M_CPU_EMU
 template <typename T>
 inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s) { d2h(dst, src, n, s); }
 #else
-constexpr size_t kPinnedBytes = 64 << 10;
+constexpr size_t kPinnedBytes = 64 << 10, kPinnedHeader = 64;
+constexpr int kSpinLimitMs = 50;
 class PinnedBlock {
 public:
     PinnedBlock()
@@ -167,7 +171,10 @@ public:
             std::lock_guard<std::mutex> g(mu());
             if (!spare().empty()) { p_ = spare().back(); spare().pop_back(); }
         }
-        if (!p_) F3M_HIP(hipHostMalloc(&p_, kPinnedBytes, hipHostMallocPortable | hipHostMallocMapped));
+        if (!p_) {
+            F3M_HIP(hipHostMalloc(&p_, kPinnedBytes + kPinnedHeader, hipHostMallocPortable | hipHostMallocMapped | hipHostMallocCoherent));
+            memset(p_, 0, kPinnedHeader);
+        }
     }
     ~PinnedBlock()
     {
@@ -176,7 +183,9 @@ public:
     }
     PinnedBlock(const PinnedBlock &) = delete;
     PinnedBlock &operator=(const PinnedBlock &) = delete;
-    void *get() const { return p_; }
+    unsigned *flag() const { return static_cast<unsigned *>(p_); }            // written by the GPU
+    unsigned next_seq() const { return ++static_cast<unsigned *>(p_)[1]; }    // host only
+    void *data() const { return static_cast<char *>(p_) + kPinnedHeader; }
 
 private:
     static std::mutex &mu() { static std::mutex m; return m; }
@@ -184,19 +193,38 @@ private:
     void *p_ = nullptr;
 };
 template <typename T>
-__global__ void export_kernel(const T *__restrict__ src, T *__restrict__ dst, int n)
+__global__ void export_kernel(const T *__restrict__ src, T *__restrict__ dst, int n, unsigned *flag, unsigned seq)
 {
     for (int i = threadIdx.x; i < n; i += blockDim.x) dst[i] = src[i];
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+// waits until the GPU has stored seq into *flag
+inline void await_flag(const unsigned *flag, unsigned seq, hipStream_t s)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    for (unsigned spins = 1;; spins++) {
+        if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return;
+        __builtin_ia32_pause();
+        if ((spins & 0xfff) == 0 &&
+            std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(kSpinLimitMs)) {
+            F3M_HIP(hipStreamSynchronize(s));
+            if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) throw Error(102, "result of a device kernel did not arrive");
+            return;
+        }
+    }
 }
 template <typename T>
 inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s)
 {
     if (n * sizeof(T) > kPinnedBytes) { d2h(dst, src, n, s); return; }
     PinnedBlock blk;
-    hipLaunchKernelGGL(export_kernel<T>, dim3(1), dim3(256), 0, s, src, static_cast<T *>(blk.get()), (int)n);
+    const unsigned seq = blk.next_seq();
+    hipLaunchKernelGGL(export_kernel<T>, dim3(1), dim3(256), 0, s, src, static_cast<T *>(blk.data()), (int)n, blk.flag(), seq);
     F3M_HIP(hipGetLastError());
-    F3M_HIP(hipStreamSynchronize(s));
-    memcpy(dst, blk.get(), n * sizeof(T));
+    await_flag(blk.flag(), seq, s);
+    memcpy(dst, blk.data(), n * sizeof(T));
 }
 #endif
 
