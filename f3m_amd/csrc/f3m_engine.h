@@ -89,9 +89,11 @@ void gather_tree_points(Tree &t, const float *X, hipStream_t s);
 void divide_launch(Tree &t, int *dstats, hipStream_t s);
 void divide_finish(Tree &t, const int *hstats);
 void divide_discard(Tree &t);
-// The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts (the four totals
-// -- small, far, keep, far pairs outside the M2L tables -- go to dtot on the device), lists_finish
-// allocates from the fetched totals and writes.
+// The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts and scans (the
+// sizes of the small, far and keep list are then the last entries pos[(c+1)*stride - 1] of the three
+// scans; the number of far pairs outside the M2L tables is added to dtot[3], which the caller keeps
+// zero between levels), lists_finish allocates from the fetched totals htot[0..3] and writes.
+// divide_launch likewise adds to dstats[0..1], zero on entry.
 struct ListsPending {
     DBuf<long long> pos;
     long long stride = 0;

@@ -20,7 +20,8 @@ constexpr int kScanBlock = 256;
 constexpr int kScanItems = 8;
 constexpr int kScanTile = kScanBlock * kScanItems;
 
-template <typename Tin, typename Tout>
+// RISE: the scanned element i is 1 where in[i+1] > in[i] (in has n+1 entries), else 0
+template <typename Tin, typename Tout, bool RISE = false>
 __global__ void scan_tile_kernel(const Tin *__restrict__ in, long long n, Tout *__restrict__ out, Tout *__restrict__ tilesum)
 {
     __shared__ Tout sh[kScanBlock];
@@ -31,7 +32,8 @@ __global__ void scan_tile_kernel(const Tin *__restrict__ in, long long n, Tout *
 #pragma unroll
     for (int e = 0; e < kScanItems; e++) {
         long long i = base + e;
-        v[e] = (i < n) ? (Tout)in[i] : (Tout)0;   // element n (the extra output slot) reads as 0
+        if (RISE) v[e] = (i < n && in[i + 1] > in[i]) ? (Tout)1 : (Tout)0;
+        else v[e] = (i < n) ? (Tout)in[i] : (Tout)0;   // element n (the extra output slot) reads as 0
         sum += v[e];
     }
     sh[tid] = sum;
@@ -62,13 +64,13 @@ __global__ void scan_add_kernel(Tout *__restrict__ out, long long n1, const Tout
         if (i < n1) out[i] += add;
 }
 
-template <typename Tin, typename Tout>
+template <typename Tin, typename Tout, bool RISE = false>
 static void exclusive_scan(const Tin *in, long long n, Tout *out, hipStream_t s)
 {
     long long n1 = n + 1;
     unsigned ntiles = cdiv(n1, kScanTile);
     DBuf<Tout> tilesum(ntiles);
-    F3M_LAUNCH((scan_tile_kernel<Tin, Tout>), ntiles, kScanBlock, 0, s, in, n, out, tilesum.get());
+    F3M_LAUNCH((scan_tile_kernel<Tin, Tout, RISE>), ntiles, kScanBlock, 0, s, in, n, out, tilesum.get());
     check_launch("scan_tile");
     if (ntiles > 1) {
         DBuf<Tout> tileoff((size_t)ntiles + 1);
@@ -181,6 +183,8 @@ void exclusive_scan_i64_batched(const long long *in, long long n, long long pitc
 }
 
 void exclusive_scan_i32(const int *in, long long n, int *out, hipStream_t s) { exclusive_scan<int, int>(in, n, out, s); }
+// out[i] = number of j < i with pos[j+1] > pos[j] (pos: n+1 non-decreasing offsets)
+static void exclusive_scan_nonempty(const int *pos, long long n, int *out, hipStream_t s) { exclusive_scan<int, int, true>(pos, n, out, s); }
 void exclusive_scan_i64(const long long *in, long long n, long long *out, hipStream_t s)
 {
     exclusive_scan<long long, long long>(in, n, out, s);
@@ -504,12 +508,6 @@ __global__ void child_bounds_kernel(const uint32_t *__restrict__ keys, const uin
     natpos[nat] = lo;
 }
 
-__global__ void nonempty_kernel(const int *__restrict__ natpos, long long ncand, int *__restrict__ flag)
-{
-    long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (nat < ncand) flag[nat] = natpos[nat + 1] > natpos[nat] ? 1 : 0;
-}
-
 // stats[0] = number of non-empty children, stats[1] = largest count
 __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__restrict__ cid, long long ncand, int d,
                                    const uint32_t *__restrict__ prefix_prev, const float *__restrict__ ctr_prev,
@@ -557,13 +555,11 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     TreeLevel &prev = t.lev[k - 1];
     long long ncand = (long long)prev.nb << d;
     F3M_REQUIRE(ncand < (1ll << 31) - 2, 20, "too many candidate boxes at depth %d (%lld)", k, ncand);
-    DBuf<int> natpos((size_t)ncand + 1), flag((size_t)ncand), cid((size_t)ncand + 1);
+    DBuf<int> natpos((size_t)ncand + 1), cid((size_t)ncand + 1);
     F3M_LAUNCH(child_bounds_kernel, cdiv(ncand + 1, 256), 256, 0, s, t.keys.get(), prev.prefix.get(), prev.off.get(), ncand,
                d, shift, t.n, natpos.get());
     check_launch("child_bounds");
-    F3M_LAUNCH(nonempty_kernel, cdiv(ncand, 256), 256, 0, s, natpos.get(), ncand, flag.get());
-    check_launch("nonempty");
-    exclusive_scan_i32(flag.get(), ncand, cid.get(), s);
+    exclusive_scan_nonempty(natpos.get(), ncand, cid.get(), s);      // compact id = number of non-empty candidates before
     size_t bound = (size_t)std::min<long long>(ncand, t.n);
     TreeLevel cur;
     cur.depth = k;
@@ -572,7 +568,6 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     cur.ctr.reset(bound * d);
     cur.cell.reset(bound * d);
     prev.childstart.reset((size_t)prev.nb + 1);
-    F3M_HIP(hipMemsetAsync(dstats, 0, 2 * sizeof(int), s));
     float quarter = 0.25f * prev.edge;
     F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
                prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
@@ -797,11 +792,6 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     if (!WRITE && lane == 0) { cnt[bx] = c0; cnt[stride + bx] = c1; cnt[2 * stride + bx] = c2; }
 }
 
-__global__ void list_totals_kernel(const long long *__restrict__ pos, long long stride, long long *__restrict__ out)
-{
-    if (threadIdx.x < 3) out[threadIdx.x] = pos[threadIdx.x * stride + stride - 1];   // out[3]: outlier counter
-}
-
 // Row statistics of the small and the keep list of a level: out[4c .. 4c+3] (c = 0 small, 1 keep) += x
 // boxes with pairs, their points, their pieces of 128 and of 160 points (out is zero before).
 constexpr int kRowStatBlock = 256;
@@ -856,7 +846,6 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
     pend.active = false;
-    F3M_HIP(hipMemsetAsync(dtot, 0, 4 * sizeof(long long), s));
     if (keep_prev.n == 0) return;
     F3M_REQUIRE(keep_prev.n < (1ll << 31) - 2, 21, "keep list too long (%lld)", keep_prev.n);
     F3M_REQUIRE((1 << d) < (1 << 21), 21, "too many children per box");
@@ -875,8 +864,6 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
     exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
-    F3M_LAUNCH(list_totals_kernel, 1, 64, 0, s, pend.pos.get(), pend.stride, dtot);
-    check_launch("list_totals");
 }
 
 void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,

@@ -227,8 +227,23 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // two things per level, the box counts of the division and the list sizes; to wait only once per
     // level, the division of depth k+1 is started together with the list count of depth k whenever the
     // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
-    DBuf<int> dres(16);          // [0..7]: four 64-bit list totals, [8,9]: X tree stats, [10,11]: Y tree stats
+    // Host record of a level, in 32-bit words: [0..5] pairs of the small, far and keep list (64 bits each),
+    // [6,7] far pairs outside the M2L tables, [8,9] boxes and largest box of the X tree's new level,
+    // [10,11] of the Y tree's.  On the device the first three are the last entries of the list builder's
+    // scans; the counters behind [6..11] live in dres and are cleared by the readback that fetches them.
+    DBuf<int> dres(16);
+    F3M_HIP(hipMemsetAsync(dres.get(), 0, 16 * sizeof(int), s));
     alignas(8) int hres[16];
+    auto fetch_level = [&](const ListsPending *pend, bool division) {
+        memset(hres, 0, sizeof(hres));
+        ExportList L;
+        if (pend != nullptr && pend->active) {
+            for (int c = 0; c < 3; c++) L.add(pend->pos.get() + (c + 1) * pend->stride - 1, 2, 2 * c);
+            L.add(dres.get() + 6, 2, 6, true);
+        }
+        if (division) L.add(dres.get() + 8, sym ? 2 : 4, 8, true);
+        if (L.nseg > 0) fetch_segments(L, hres, s);
+    };
     // row statistics of the small and keep lists, 8 words per level; nothing at plan time depends on
     // them, so they are fetched once at the end instead of with the per-level wait
     constexpr int kMaxLevels = 40;
@@ -248,7 +263,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     };
     if (need_tree && wants_division()) {
         start_division();
-        fetch_small(hres, dres.get(), 16, s);
+        fetch_level(nullptr, true);
         finish_division();
         for (;;) {
             const int k = (int)P->tx.lev.size() - 1;
@@ -260,7 +275,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
             const bool ahead = wants_division();
             if (ahead) start_division();
-            fetch_small(hres, dres.get(), 16, s);
+            fetch_level(&pend, ahead);
             F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
                          drow.get() + 8 * (P->levels.size() - 1), s);

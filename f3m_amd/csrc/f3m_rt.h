@@ -157,9 +157,37 @@ inline void d2h(T *dst, const T *src, size_t n, hipStream_t s)
 // waiting for the stream (a stream wait costs some 15 us more, a copy into pageable memory a staged
 // copy command on top).  After kSpinLimitMs of watching the host falls back to the stream wait, which
 // also reports a failed kernel.  Pinned blocks are kept for the life of the process.
+// What one readback collects: up to kMaxExportSegs runs of 32-bit words from device memory, each to its
+// place in the host record; a run marked `clear` is zeroed after it is read (counters that the next
+// round of kernels adds to).
+constexpr int kMaxExportSegs = 8;
+struct ExportList {
+    struct Seg { unsigned *src; int nwords, dst, clear; } seg[kMaxExportSegs];
+    int nseg = 0, total = 0;
+    void add(void *src, int nwords, int dst_word, bool clear = false)
+    {
+        if (nseg >= kMaxExportSegs) throw Error(103, "too many readback segments");
+        seg[nseg++] = Seg{static_cast<unsigned *>(src), nwords, dst_word, clear ? 1 : 0};
+        if (dst_word + nwords > total) total = dst_word + nwords;
+    }
+};
+template <int BLOCK>
+__global__ void export_segments_kernel(ExportList L, unsigned *__restrict__ dst)
+{
+    for (int g = 0; g < L.nseg; g++)
+        for (int i = threadIdx.x; i < L.seg[g].nwords; i += BLOCK) {
+            dst[L.seg[g].dst + i] = L.seg[g].src[i];
+            if (L.seg[g].clear) L.seg[g].src[i] = 0;
+        }
+}
 #ifdef F3M_CPU_EMU
 template <typename T>
 inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s) { d2h(dst, src, n, s); }
+inline void fetch_segments(const ExportList &L, void *dst, hipStream_t s)
+{
+    F3M_LAUNCH((export_segments_kernel<64>), 1, 64, 0, s, L, static_cast<unsigned *>(dst));
+    F3M_HIP(hipStreamSynchronize(s));
+}
 #else
 constexpr size_t kPinnedBytes = 64 << 10, kPinnedHeader = 64;
 constexpr int kSpinLimitMs = 50;
@@ -214,6 +242,28 @@ inline void await_flag(const unsigned *flag, unsigned seq, hipStream_t s)
             return;
         }
     }
+}
+template <int BLOCK>
+__global__ void export_segments_flag_kernel(ExportList L, unsigned *__restrict__ dst, unsigned *flag, unsigned seq)
+{
+    for (int g = 0; g < L.nseg; g++)
+        for (int i = threadIdx.x; i < L.seg[g].nwords; i += BLOCK) {
+            dst[L.seg[g].dst + i] = L.seg[g].src[i];
+            if (L.seg[g].clear) L.seg[g].src[i] = 0;
+        }
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(flag, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+inline void fetch_segments(const ExportList &L, void *dst, hipStream_t s)
+{
+    if ((size_t)L.total * 4 > kPinnedBytes) throw Error(103, "readback record too large");
+    PinnedBlock blk;
+    const unsigned seq = blk.next_seq();
+    hipLaunchKernelGGL(export_segments_flag_kernel<64>, dim3(1), dim3(64), 0, s, L, static_cast<unsigned *>(blk.data()), blk.flag(), seq);
+    F3M_HIP(hipGetLastError());
+    await_flag(blk.flag(), seq, s);
+    memcpy(dst, blk.data(), (size_t)L.total * 4);
 }
 template <typename T>
 inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s)
