@@ -581,6 +581,20 @@ int f3m_plan_level_sizes(const f3m_plan *plan, int level, int64_t *sizes, float 
     });
 }
 
+int f3m_plan_list_rows(const f3m_plan *plan, int level, int64_t *rows)
+{
+    return guarded([&] {
+        check_level(plan, level);
+        F3M_REQUIRE(rows != nullptr, 1, "rows is NULL");
+        const PlanLevel &L = plan->levels[level - 1];
+        const PairList *l[2] = {&L.small_, &L.keep};
+        for (int c = 0; c < 2; c++) {
+            rows[4 * c + 0] = l[c]->rows, rows[4 * c + 1] = l[c]->row_points;
+            rows[4 * c + 2] = l[c]->items128, rows[4 * c + 3] = l[c]->items160;
+        }
+    });
+}
+
 int f3m_plan_level_copy(const f3m_plan *plan, int level, int which, void *dst, void *stream)
 {
     return guarded([&] {

@@ -145,6 +145,13 @@ class Plan:
         out["edge"] = np.float32(e.value)
         return out
 
+    def list_rows(self, level):
+        """[boxes with pairs, their points, their pieces of 128 and of 160 points] of the small list,
+        then the same of the keep list: what the near field sizes its launches with."""
+        r = (C.c_int64 * 8)()
+        capi.check(self._lib, self._lib.f3m_plan_list_rows(self._h, level, r))
+        return [int(v) for v in r]
+
     def level(self, level):
         """Host copies (numpy) of the tree level and its three lists; levels are 1..depth."""
         sz = self.level_sizes(level)

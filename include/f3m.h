@@ -69,6 +69,9 @@ int f3m_plan_depth(const f3m_plan *plan);                 /* number of divisions
 int f3m_plan_symmetric(const f3m_plan *plan);
 /* sizes[0..7] = boxes of X tree, boxes of Y tree, |far|, |small|, |keep|, nodes used, max count X, max count Y */
 int f3m_plan_level_sizes(const f3m_plan *plan, int level, int64_t *sizes, float *edge);
+/* rows[0..3] = x boxes with pairs in the small list, their points, their pieces of 128 and of 160 points;
+ * rows[4..7] = the same for the keep list (what the near field sizes its launches with) */
+int f3m_plan_list_rows(const f3m_plan *plan, int level, int64_t *rows);
 enum f3m_level_array {
     F3M_CENTERS_X = 0,   /* float (nbx,d) */
     F3M_CENTERS_Y = 1,

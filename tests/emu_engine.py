@@ -77,6 +77,11 @@ class Plan:
         out["edge"] = np.float32(e.value)
         return out
 
+    def list_rows(self, level):
+        r = (C.c_int64 * 8)()
+        capi.check(lib(), lib().f3m_plan_list_rows(self._h, level, r))
+        return [int(v) for v in r]
+
     def lookup_boxes(self, level, cells, tree="x"):
         cells = np.ascontiguousarray(np.asarray(cells, np.int32))
         ids = np.empty(cells.shape[0], np.int32)

@@ -32,3 +32,15 @@ def rel_l2(a, t):
     a = np.asarray(a, np.float64)
     t = np.asarray(t, np.float64)
     return float(np.linalg.norm(a - t) / np.linalg.norm(t))
+
+
+def expected_list_rows(level):
+    """row statistics of the small and keep list of a level (dict of Plan.level): boxes with pairs, their
+    points, their pieces of 128 and of 160 points"""
+    cnt = np.diff(np.asarray(level["offx"], np.int64))
+    out = []
+    for which in ("small", "keep"):
+        pairs = np.asarray(level[which]).reshape(-1, 2)
+        n = cnt[np.unique(pairs[:, 0])] if len(pairs) else np.zeros(0, np.int64)
+        out += [len(n), int(n.sum()), int(((n + 127) // 128).sum()), int(((n + 159) // 160).sum())]
+    return out

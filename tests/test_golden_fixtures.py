@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 import golden_fixtures as gf
-from parity_checks import rel_l2
+from parity_checks import rel_l2, expected_list_rows
 
 NAMES = gf.names()
 
@@ -35,4 +35,18 @@ def test_emulated_engine_matches_fixtures(monkeypatch, name):
     X, Y, b, prm = gf.case(fx, name)
     eng = ee.Plan(X, Y, **prm)
     gf.assert_plan_matches_fixture(eng, eng.depth, fx, name)
+    for k in range(1, eng.depth + 1):
+        assert eng.list_rows(k) == expected_list_rows(eng.level(k)), (name, k)
+    gf.assert_product_matches_fixture(eng.apply(b), fx, name)
+
+
+@pytest.mark.parametrize("name", ["d3_uniform", "d3_two_trees", "d3_lattice_duplicates", "d4_uniform"])
+def test_emulated_matrix_pipe_near_field_with_source_runs(monkeypatch, name):
+    """the matrix-pipe near field, whole lists per wavefront: source boxes under one parent cell form one run"""
+    import emu_engine as ee
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    fx = gf.load()
+    X, Y, b, prm = gf.case(fx, name)
+    eng = ee.Plan(X, Y, **prm)
     gf.assert_product_matches_fixture(eng.apply(b), fx, name)

@@ -5,7 +5,7 @@ product and no worse than 1.5x the oracle algorithm's own error)."""
 import numpy as np
 import pytest
 
-from parity_checks import assert_plan_matches_oracle, rel_l2
+from parity_checks import assert_plan_matches_oracle, expected_list_rows, rel_l2
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -73,9 +73,26 @@ def test_committed_oracle_fixtures(eng, fixture_name):
     X, Y, b, prm = gf.case(fx, fixture_name)
     plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
     gf.assert_plan_matches_fixture(plan, plan.depth, fx, fixture_name)
+    for k in range(1, plan.depth + 1):
+        assert plan.list_rows(k) == expected_list_rows(plan.level(k)), (fixture_name, k)
     gf.assert_product_matches_fixture(plan.apply(dev(b)).cpu().numpy(), fx, fixture_name)
     gf.assert_product_matches_fixture(eng.kmvm(dev(X), None if Y is None else dev(Y), dev(b), **prm).cpu().numpy(), fx,
                                       fixture_name)
+
+
+@pytest.mark.parametrize("fixture_name", __import__("golden_fixtures").names())
+def test_near_field_source_runs_on_matrix_pipe(eng, monkeypatch, fixture_name):
+    """The matrix-pipe near field with whole lists per wavefront (no slicing), where source boxes that
+    follow each other under one parent cell are taken as one run.  The lattice fixture has targets whose
+    -|x''|^2 is an exact tie between two f16 values: hi and lo of the split must come from one rounding."""
+    import golden_fixtures as gf
+    print("case fixture (matrix pipe, unsliced)", fixture_name, flush=True)
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    fx = gf.load()
+    X, Y, b, prm = gf.case(fx, fixture_name)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    gf.assert_product_matches_fixture(plan.apply(dev(b)).cpu().numpy(), fx, fixture_name)
 
 
 @pytest.mark.parametrize("name", NAMES)
