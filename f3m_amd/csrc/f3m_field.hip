@@ -296,7 +296,7 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 // is an inner product over the D+1 components (2y'_k, -|y'|^2) . (x'_k, 1) plus a per-target constant.
 // Every fp32 operand is split into two f16 values, v = hi + lo (|v - hi - lo| <= 2^-22 |v|), and the
 // products hi.hi + hi.lo + lo.hi of all components fill the 16 inner slots of one
-// v_mfma_f32_32x32x16_f16 (two instructions for D >= 5), accumulated in fp32 on top of C = -|x'|^2.
+// v_mfma_f32_32x32x16_f16 (two instructions for D >= 5), accumulated in fp32 from zero.
 // The f16 matrix pipe runs beside the vector ALU, which is left with one exp2 and one fused
 // multiply-add per pair.  A wavefront owns two tiles of 32 targets (lanes l and l+32 hold the same
 // target and different source rows; their partial sums are combined once at the end), a workgroup
@@ -306,17 +306,27 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 // lengthscale and otherwise launches near_kernel).
 
 
-// inner slot s of the matrix product: component s/3; s%3 = 0: hi.hi, 1: (source hi).(target lo), 2: (source lo).(target hi)
-template <int C>
+// Inner slots of the matrix product.  Coordinate k takes slots 3k..3k+2: hi.hi, (source hi).(target lo),
+// (source lo).(target hi).  The two scalars need two slots each, because their partner is exactly 1:
+// slots 3D, 3D+1 = (hi, lo of the source's -|y'|^2) . 1 and slots 3D+2, 3D+3 = 1 . (hi, lo of the
+// target's -|x''|^2).  3D+4 slots in all: one instruction of 16 up to D = 4.
+// hi/lo hold C = D+2 values: the coordinates, then on the source side (-|y'|^2, 1), on the target side (1, -|x''|^2).
+__host__ __device__ constexpr int near_slots(int D) { return 3 * D + 4; }
+__host__ __device__ constexpr int near_insts(int D) { return (near_slots(D) + 15) / 16; }
+template <int D>
 __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, int hh, bool source)
 {
     h8 v;
 #pragma unroll
     for (int e = 0; e < 8; e++) {
         const int slot = 16 * n + 8 * hh + e;
-        if (slot < 3 * C) {
+        if (slot < 3 * D) {
             const int c = slot / 3, tau = slot % 3;
             v[e] = source ? (tau == 2 ? lo[c] : hi[c]) : (tau == 1 ? lo[c] : hi[c]);
+        } else if (slot < near_slots(D)) {
+            const int sl = slot - 3 * D;
+            if (source) v[e] = sl == 0 ? hi[D] : (sl == 1 ? lo[D] : hi[D + 1]);
+            else v[e] = sl < 2 ? hi[D] : (sl == 2 ? hi[D + 1] : lo[D + 1]);
         } else {
             v[e] = to_half(0.f);
         }
@@ -349,7 +359,7 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
                                                                   const int *__restrict__ need, h8 *__restrict__ ops)
 {
     constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
-    constexpr int NS = (3 * C + 15) / 16;
+    constexpr int NS = near_insts(D);
     __shared__ int bounds[kOpsBlock];
     const int tid = threadIdx.x;
     const long long i0 = (long long)blockIdx.x * kOpsBlock, i = i0 + tid;
@@ -396,8 +406,8 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
     }
 #pragma unroll
     for (int n = 0; n < NS; n++) {
-        ops[(long long)(n * 2 + 0) * stride + i] = split_operand<C>(hi, lo, n, 0, true);
-        ops[(long long)(n * 2 + 1) * stride + i] = split_operand<C>(hi, lo, n, 1, true);
+        ops[(long long)(n * 2 + 0) * stride + i] = split_operand<D>(hi, lo, n, 0, true);
+        ops[(long long)(n * 2 + 1) * stride + i] = split_operand<D>(hi, lo, n, 1, true);
     }
 }
 
@@ -423,7 +433,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
     int stripe, int nsplit, float *__restrict__ part, int nitems)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
-    constexpr int NS = (3 * C + 15) / 16;
+    constexpr int NS = near_insts(D);
     const int lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     // Workgroups are handed to the 8 XCDs round-robin.  Work items are in Morton order of their x box
     // and neighbouring boxes share their source boxes, so the work items are cut into stripes of
@@ -544,7 +554,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
             }
 #pragma unroll
             for (int n = 0; n < NS; n++) {
-                h8 v0 = split_operand<C>(hi, lo, n, 0, false), v1 = split_operand<C>(hi, lo, n, 1, false);
+                h8 v0 = split_operand<D>(hi, lo, n, 0, false), v1 = split_operand<D>(hi, lo, n, 1, false);
                 bop[q][n] = half ? v1 : v0;
             }
         }
@@ -661,7 +671,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     if (use_mfma && list.rows >= 0) ntiles = (int)std::max<long long>(1, tpw == 5 ? list.items160 : list.items128);
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
-        const int C = d + 2, NS = (3 * C + 15) / 16;
+        const int NS = near_insts(d);
         const long long stride = ty.n + 32;
         // The operands of a level are kept in the plan.  only_list: this list is the only near list of
         // its level, so operands are needed for its source boxes only (at most levels a small part).
