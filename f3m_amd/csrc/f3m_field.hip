@@ -1266,7 +1266,7 @@ __device__ inline void sib_ext_digits(int e, int *dg)
 
 template <int D, int N>
 __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
-                                                        int R2, int GS, int nsub, const int *__restrict__ childstart,
+                                                        int R2, int GS, int nsub, int npass, const int *__restrict__ childstart,
                                                         const int *__restrict__ cell, const int *__restrict__ pairs,
                                                         const int *__restrict__ rowptr, const float *__restrict__ mom,
                                                         float *__restrict__ loc)
@@ -1274,13 +1274,17 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     constexpr int NCODE = sib_codes(D), NEXT = sib_ext_codes(D), NN = N * N, NB = N <= 3 ? 4 : (D >= 4 ? 1 : 2);
     F3M_DYN_SHARED(float, smem);
     const int tid = threadIdx.x, BD = blockDim.x, lane = tid & 63;
-    int *tby = reinterpret_cast<int *>(smem);                       // NCODE: y box of a table cell
-    unsigned *tmask = reinterpret_cast<unsigned *>(smem) + NCODE;   // NCODE: siblings that list it
-    int *xby = reinterpret_cast<int *>(smem) + 2 * NCODE;           // NEXT: the same for the extension cells
-    unsigned *xmask = reinterpret_cast<unsigned *>(smem) + 2 * NCODE + NEXT;
-    int *xord = reinterpret_cast<int *>(smem) + 2 * NCODE + 2 * NEXT;   // NEXT: extension cells in walking order
+    // The regular table is filled and walked in npass parts (slabs of the last dimension, which is the
+    // outermost of the walk), so that it takes NCODE / npass cells of LDS (the host asks for more than
+    // one part only where the whole table does not fit).
+    const int chunk = NCODE / npass;
+    int *tby = reinterpret_cast<int *>(smem);                       // chunk: y box of a table cell
+    unsigned *tmask = reinterpret_cast<unsigned *>(smem) + chunk;   // chunk: siblings that list it
+    int *xby = reinterpret_cast<int *>(smem) + 2 * chunk;           // NEXT: the same for the extension cells
+    unsigned *xmask = reinterpret_cast<unsigned *>(smem) + 2 * chunk + NEXT;
+    int *xord = reinterpret_cast<int *>(smem) + 2 * chunk + 2 * NEXT;   // NEXT: extension cells in walking order
     int *xkey = xord + NEXT;                                        // NEXT
-    float *xbuf = smem + 2 * NCODE + 4 * NEXT;                      // NN * BD: exchange buffer
+    float *xbuf = smem + 2 * chunk + 4 * NEXT;                      // NN * BD: exchange buffer
     float *tabg = xbuf + NN * BD;                                   // ntab: E_j[o][a][q], row length sm.NT
     float *tab01 = tabg + ((ntab + 3) & ~3);                        // 2 * 13 * N rows of 4: E_0, E_1 padded
     float *zrow = tab01 + 2 * kM2LOffsets * N * 4;                  // N rows of zeros
@@ -1288,7 +1292,6 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     const int px = blockIdx.x / nsub, sg = blockIdx.x % nsub;
     const int P = nm.P;
 
-    for (int e = tid; e < NCODE; e += BD) { tby[e] = 0; tmask[e] = 0u; }
     for (int e = tid; e < NEXT; e += BD) {
         xby[e] = 0; xmask[e] = 0u;
         int dg[D], key = 0, mul = 1;
@@ -1323,36 +1326,45 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
 #pragma unroll
     for (int j = 0; j < D; j++) pc[j] = 2 * (cell[(long long)c0 * D + j] >> 1) - 2;
     __syncthreads();
-    for (int sl = 0; sl < GS; sl++) {
-        const int bx = sib[sl];
-        if (bx < 0) continue;                              // uniform over the workgroup
-        const int m1 = rowptr[bx + 1];
-        for (int m = rowptr[bx] + tid; m < m1; m += BD) {
-            const int by = pairs[2 * (long long)m + 1];
-            int dg[D];
+    // fills part `pass` of the regular table (and, with part 0, the extension table) from the far rows
+    auto fill_tables = [&](int pass) {
+        for (int e = tid; e < chunk; e += BD) { tby[e] = 0; tmask[e] = 0u; }
+        __syncthreads();
+        for (int s2 = 0; s2 < GS; s2++) {
+            const int bx = sib[s2];
+            if (bx < 0) continue;                          // uniform over the workgroup
+            const int m1 = rowptr[bx + 1];
+            for (int m = rowptr[bx] + tid; m < m1; m += BD) {
+                const int by = pairs[2 * (long long)m + 1];
+                int dg[D];
 #pragma unroll
-            for (int j = 0; j < D; j++) dg[j] = cell[(long long)by * D + j] - pc[j];
-            const int code = sib_code<D>(dg);
-            if (code >= 0) { tby[code] = by; atomicOr(&tmask[code], 1u << sl); }
-            else if (code <= -2) { xby[-2 - code] = by; atomicOr(&xmask[-2 - code], 1u << sl); }
+                for (int j = 0; j < D; j++) dg[j] = cell[(long long)by * D + j] - pc[j];
+                const int code = sib_code<D>(dg);
+                if (code >= 0) {
+                    const int c = code - pass * chunk;
+                    if (c >= 0 && c < chunk) { tby[c] = by; atomicOr(&tmask[c], 1u << s2); }
+                } else if (code <= -2 && pass == 0) { xby[-2 - code] = by; atomicOr(&xmask[-2 - code], 1u << s2); }
+            }
         }
-    }
-    __syncthreads();
+        __syncthreads();
+    };
 
-    // this lane: sibling sl, position r2 among the nodes of dimensions >= 2
-    const int sl = tid / R2, r2 = tid % R2;
-    const bool valid = sl < GS;                            // lanes past the last sibling only keep step
+    // This lane: sibling sl, position r2 among the nodes of dimensions >= 2.  The siblings are the fast
+    // index: the GS lanes of one r2 read the same moments, so a wavefront's load touches 64/GS short
+    // runs of memory instead of 64 (the moment loads are what the level-1 cache has to carry here).
+    const int sl = tid % GS, r2 = tid / GS;
+    const bool valid = r2 < R2;                            // lanes past the last node only keep step
     const int mybox = valid ? sib[sl] : -1;
     const bool live = mybox >= 0;
     int cbit[D], dig[D], lstride[D];
     {
-        const int code = sg * GS + (valid ? sl : 0);
-        int rem = r2, st = 1;
+        const int code = sg * GS + sl;
+        int rem = valid ? r2 : 0, st = GS;
 #pragma unroll
         for (int j = 0; j < D; j++) {
-            cbit[j] = 2 + ((code >> j) & 1) + sm.omin[j];  // table index of dimension j = digit_j - cbit[j]
+            cbit[j] = 4 + ((code >> j) & 1) + sm.omin[j];  // table index of dimension j = (digit_j + 2) - cbit[j]
             dig[j] = 0; lstride[j] = 0;
-            if (j >= 2) { dig[j] = rem % nm.n[j]; rem /= nm.n[j]; lstride[j] = st; st *= nm.n[j]; }
+            if (j >= 2) { dig[j] = rem % nm.n[j]; rem /= nm.n[j]; lstride[j] = st; st *= nm.n[j]; }   // lstride: in lanes
         }
     }
     const float *mine = mom + (long long)NN * (live ? r2 : 0);
@@ -1362,16 +1374,18 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     for (int j = 0; j < D; j++)
 #pragma unroll
         for (int i = 0; i < NN; i++) acc[j][i] = 0.f;
-    int cur[D];
-#pragma unroll
-    for (int j = 0; j < D; j++) cur[j] = 0;
+    // The digits of a far cell travel as one word, four bits each, biased by 2 (extension cells reach
+    // -2): the walk is the same in every wavefront, so whatever it costs in scalar instructions per far
+    // box is paid by each of them on the compute unit's one scalar unit.
+    int curpk = 0;
     bool have = false;
+    auto digit2 = [](int pk, int j) { return (pk >> (4 * j)) & 15; };      // digit j + 2
 
     // applies factor l+1 to acc[l], adds the result to acc[l+1] and clears acc[l]
     auto flush = [&](auto level) {
         constexpr int l = decltype(level)::value, j = l + 1;
         if constexpr (j == 1) {
-            int oi = cur[1] - cbit[1];
+            int oi = digit2(curpk, 1) - cbit[1];
             oi = min(max(oi, 0), kM2LOffsets - 1);
             const float *T1 = tab01 + ((kM2LOffsets + oi) * N) * 4;
 #pragma unroll
@@ -1392,7 +1406,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
             for (int i = 0; i < NN; i++) xbuf[i * BD + tid] = acc[l][i];
             __syncthreads();
             if (valid) {
-                int oi = cur[j] - cbit[j];
+                int oi = digit2(curpk, j) - cbit[j];
                 oi = min(max(oi, 0), kM2LOffsets - 1);
                 const float *row = tabg + ((j * kM2LOffsets + oi) * sm.NT + dig[j]) * sm.NT;
                 for (int q = 0; q < nm.n[j]; q++) {
@@ -1412,19 +1426,16 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
         if constexpr (D > 3) { if (jt > 2) flush(std::integral_constant<int, 2>()); }
         if constexpr (D > 4) { if (jt > 3) flush(std::integral_constant<int, 3>()); }
     };
-    // one far box: dg = its digits (uniform), v = its moments at this lane's nodes
-    auto far_box = [&](const int *dg, unsigned smask, const fvec<NN> &v) {
+    // one far box: pk = its packed digits (uniform), v = its moments at this lane's nodes
+    auto far_box = [&](int pk, unsigned smask, const fvec<NN> &v) {
         if (have) {
-            int jt = 0;
-#pragma unroll
-            for (int j = 1; j < D; j++) if (dg[j] != cur[j]) jt = j;
-            flush_upto(jt);
+            const int diff = (pk ^ curpk) >> 4;             // digits 1.. that change
+            flush_upto(diff ? (31 - __builtin_clz(diff)) / 4 + 1 : 0);   // up to the highest of them
         }
-#pragma unroll
-        for (int j = 0; j < D; j++) cur[j] = dg[j];
+        curpk = pk;
         have = true;
         const bool part = live && ((smask >> sl) & 1u);
-        int oi = dg[0] - cbit[0];
+        int oi = digit2(pk, 0) - cbit[0];
         oi = min(max(oi, 0), kM2LOffsets - 1);
         const float *T0 = part ? tab01 + (oi * N) * 4 : zrow;
 #pragma unroll
@@ -1442,6 +1453,19 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     };
     // walks 64 table cells: ml, byl = this lane's cell; cellid = its id (regular code or extension entry)
     auto walk64 = [&](unsigned ml, int byl, int cellid, auto ext) {
+        int pkl = 0;                                       // packed digits of this lane's cell
+        {
+            int dg[D];
+            if constexpr (decltype(ext)::value) {
+                sib_ext_digits<D>(cellid, dg);
+            } else {
+                int rem = cellid;
+#pragma unroll
+                for (int j = 0; j < D; j++) { dg[j] = rem % kSibSpan; rem /= kSibSpan; }
+            }
+#pragma unroll
+            for (int j = 0; j < D; j++) pkl |= (dg[j] + 2) << (4 * j);
+        }
         unsigned long long bal = wave_ballot(ml != 0u);
         while (bal) {                                      // identical in every wavefront of the workgroup
             int ls[NB], cnt = 0;
@@ -1456,24 +1480,19 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
 #pragma unroll
             for (int u = 0; u < NB; u++) {
                 if (u >= cnt) break;                       // uniform
-                const int id = wave_readlane(cellid, ls[u]);
                 const unsigned smask = (unsigned)wave_readlane((int)ml, ls[u]);
-                int dg[D];
-                if constexpr (decltype(ext)::value) {
-                    sib_ext_digits<D>(id, dg);
-                } else {
-                    int rem = id;
-#pragma unroll
-                    for (int j = 0; j < D; j++) { dg[j] = rem % kSibSpan; rem /= kSibSpan; }
-                }
-                far_box(dg, smask, v[u]);
+                far_box(wave_readlane(pkl, ls[u]), smask, v[u]);
             }
         }
     };
 
-    for (int base = 0; base < NCODE; base += 64) {
-        const int idx = base + lane;
-        walk64(idx < NCODE ? tmask[idx] : 0u, idx < NCODE ? tby[idx] : 0, idx, std::false_type());
+    for (int pass = 0; pass < npass; pass++) {
+        if (pass > 0) __syncthreads();                     // every wavefront is done with the previous part
+        fill_tables(pass);
+        for (int base = 0; base < chunk; base += 64) {
+            const int idx = base + lane;
+            walk64(idx < chunk ? tmask[idx] : 0u, idx < chunk ? tby[idx] : 0, pass * chunk + idx, std::false_type());
+        }
     }
     if (have) flush_upto(D - 1);
     have = false;
@@ -1630,7 +1649,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         timer_begin(kM2L, s);
         const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
         // sibling-group kernel: one tree, 3 <= d <= 5, n0 = n1 in 2..4, every far pair inside the 6^d cells
-        int sibGS = 0, sibR2 = 0;
+        int sibGS = 0, sibR2 = 0, sibPass = 1;
         size_t shsib = 0;
         // (preferred to the per-box kernel for 4 x 4 x 4 nodes as well once a level has a few hundred
         // parents: 0.30 against 0.55 ms at depth 5 of N=1e7; with fewer parents the per-box kernel has
@@ -1644,8 +1663,18 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                 sibGS = 1 << d;
                 while (sibGS * sibR2 > 1024) sibGS >>= 1;
                 const int bd = ((sibGS * sibR2 + kWave - 1) / kWave) * kWave;
-                shsib = sizeof(float) * (2 * (size_t)sib_codes(d) + 4 * (size_t)sib_ext_codes(d) + (size_t)N * N * bd + (size_t)((ntab + 3) & ~3) +
-                                         2 * (size_t)kM2LOffsets * N * 4 + (size_t)N * 4) + sizeof(int) * (size_t)sibGS;
+                // table in 1, 2, 3 or 6 parts: the fewest that fit (a second workgroup per compute unit bought
+                // with two parts did not pay at 6^5 cells: 7.7 -> 8.2 ms; every part scans the far rows again)
+                int forced = 0;                                  // F3M_SIB_PASSES=1|2|3|6: testing aid
+                if (const char *e = getenv("F3M_SIB_PASSES")) forced = atoi(e);
+                for (int np : {1, 2, 3, 6}) {
+                    if (forced > 0 && np != forced && np != 6) continue;
+                    sibPass = np;
+                    shsib = sizeof(float) * (2 * (size_t)(sib_codes(d) / np) + 4 * (size_t)sib_ext_codes(d) + (size_t)N * N * bd +
+                                             (size_t)((ntab + 3) & ~3) + 2 * (size_t)kM2LOffsets * N * 4 + (size_t)N * 4) +
+                            sizeof(int) * (size_t)sibGS;
+                    if ((shsib <= 150 * 1024 && forced <= 0) || np == forced) break;
+                }
                 if (shsib > 150 * 1024) sibGS = 0;
             }
         }
@@ -1664,7 +1693,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     if (d == DD && ns.n[0] == NNODE) {                                                                                 \
         F3M_SIB_ATTR(DD, NNODE)                                                                                        \
         F3M_LAUNCH((m2l_sib_kernel<DD, NNODE>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2, sibGS,   \
-                   nsub, par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom, loc);            \
+                   nsub, sibPass, par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom, loc);   \
     }
             F3M_SIB(3, 2) F3M_SIB(3, 3) F3M_SIB(3, 4)
             F3M_SIB(4, 2) F3M_SIB(4, 3) F3M_SIB(4, 4)

@@ -190,6 +190,20 @@ def test_m2l_forms_agree(monkeypatch, d, n, P, mp):
     assert rel_l2(grouped, direct) < 3e-6
 
 
+@pytest.mark.parametrize("parts", [2, 6])
+def test_m2l_sibling_table_in_parts(monkeypatch, parts):
+    """the sibling-group M2L can fill and walk its table of far cells in several parts (for tables that do not fit LDS whole):
+    same sums as in one part, bit for bit, because the walking order does not change"""
+    rng = np.random.default_rng(4)
+    X = rng.random((3000, 3), dtype=f32)
+    b = rng.standard_normal((3000, 1)).astype(f32)
+    eng = ee.Plan(X, None, ls=0.6, min_points=60, nr_of_interpolation=27, small_field_points=37)
+    monkeypatch.setenv("F3M_SIB_PASSES", "1")
+    whole = eng.apply(b)
+    monkeypatch.setenv("F3M_SIB_PASSES", str(parts))
+    assert np.array_equal(whole, eng.apply(b))
+
+
 def test_mfma_near_field(oracle, monkeypatch):
     monkeypatch.setenv("F3M_NEAR", "mfma")
     rng = np.random.default_rng(5)

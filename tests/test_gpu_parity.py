@@ -226,6 +226,20 @@ def test_m2l_forms_agree(eng, monkeypatch, name):
     assert rel_l2(grouped, direct) < (2e-5 if name == "uniform5_1024" else 5e-6)
 
 
+@pytest.mark.parametrize("name,parts", [("C1_uniform3", 2), ("C1_uniform3", 3), ("uniform4", 6), ("uniform5_243", 2)])
+def test_m2l_sibling_table_in_parts(eng, monkeypatch, name, parts):
+    """The sibling-group M2L can fill and walk its table of far cells in parts (for tables that do not fit
+    LDS whole).  The walking order is the same, so the sums are the same bit for bit."""
+    print("case m2l table parts", name, parts, flush=True)
+    rng = np.random.default_rng(15)
+    X, Y, prm = clouds(name, rng)
+    b = rng.standard_normal((X.shape[0], 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, **prm)
+    default = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_SIB_PASSES", str(parts))
+    assert np.array_equal(default, plan.apply(dev(b)).cpu().numpy())
+
+
 def test_m2l_children_of_parent_pairs_kept_on_the_far_threshold(eng, monkeypatch):
     """A parent pair two cells apart along one axis is exactly 2 edges away; fp32 rounding of the centres
     decides whether the reference's predicate (F3M_src/1_d_conv.cu:936-941) calls it far.  Where it is
