@@ -292,19 +292,16 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 }
 
 // Near field with the exponent on the matrix pipe.  The exponent of a pair,
-//   t = 2x'.y' - |y'|^2 - |x'|^2   (x', y' shifted to the x-box centre and scaled by sqrt(lcs log2 e)),
-// is an inner product over the D+1 components (2y'_k, -|y'|^2) . (x'_k, 1) plus a per-target constant.
+//   t = 2x''.y' - |y'|^2 - |x''|^2   (x'', y' shifted to an anchor near the sources and scaled by sqrt(lcs log2 e)),
+// is an inner product over the components (2y'_k, -|y'|^2, 1) . (x''_k, 1, -|x''|^2).
 // Every fp32 operand is split into two f16 values, v = hi + lo (|v - hi - lo| <= 2^-22 |v|), and the
-// products hi.hi + hi.lo + lo.hi of all components fill the 16 inner slots of one
+// products hi.hi + hi.lo + lo.hi of all components fill the inner slots of one
 // v_mfma_f32_32x32x16_f16 (two instructions for D >= 5), accumulated in fp32 from zero.
 // The f16 matrix pipe runs beside the vector ALU, which is left with one exp2 and one fused
-// multiply-add per pair.  A wavefront owns two tiles of 32 targets (lanes l and l+32 hold the same
-// target and different source rows; their partial sums are combined once at the end), a workgroup
-// of four wavefronts 256 targets.  Sources of a y box are staged through LDS as ready-made matrix
-// operands, padded with zero-weight sources to a multiple of 32.
-// Valid while |x'|, |y'| stay small enough for the split (the host checks the box size against the
+// multiply-add per pair.  near_operands_kernel prepares the source side once per tree level,
+// near_g_kernel streams it against the targets of a wavefront.
+// Valid while |x''|, |y'| stay small enough for the split (the host checks the box size against the
 // lengthscale and otherwise launches near_kernel).
-
 
 // Inner slots of the matrix product.  Coordinate k takes slots 3k..3k+2: hi.hi, (source hi).(target lo),
 // (source lo).(target hi).  The two scalars need two slots each, because their partner is exactly 1:
@@ -412,9 +409,10 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
 }
 
 // Near field, matrix-pipe form.  One wavefront per TPW*32 targets of an x box (TPW tiles of 32; lanes
-// l and l+32 hold the same target and different source rows).  For every listed y box the targets are
-// re-expressed relative to the centre of that y box (x'' = sc (x - c_y)) and split into f16 pairs; the
-// per-target constant -|x''|^2 rides in two spare inner slots (against a source-side 1), so the
+// l and l+32 hold the same target and different source rows).  For every run of listed y boxes (boxes
+// that follow each other in memory under one parent cell) the targets are re-expressed relative to
+// the run's anchor, the centre of that parent cell (x'' = sc (x - anchor)), and split into f16 pairs;
+// the per-target constant -|x''|^2 rides in two inner slots (against a source-side 1), so the
 // accumulator starts from zero.  The source operands come ready-made from near_operands_kernel and
 // are streamed from global memory / L2 in 32-source tiles, together with their weights.  No LDS and
 // no barriers: wavefronts are independent.  Rows past the end of a box are neutralised by a zero
@@ -662,7 +660,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     check_launch("mark_rows");
     // target tiles of 32 per wavefront: 4 (2: 10.2 ms, 4: 9.2 ms, 5: 10.2 ms, 8: 9.4 ms at N=1e7, d=3, ten tiles
     // per box), but 5 where a typical box has five tiles and would otherwise be cut into 4 + 1
-    // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms)
+    // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms at the time)
     // Where the plan has counted the rows of the list, "typical" is the mean over the listed boxes and the
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
