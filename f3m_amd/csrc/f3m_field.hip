@@ -1262,14 +1262,17 @@ __device__ inline void sib_ext_digits(int e, int *dg)
     }
 }
 
-template <int D, int N>
+template <int D, int N, int H>
 __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
                                                         int R2, int GS, int nsub, int npass, const int *__restrict__ childstart,
                                                         const int *__restrict__ cell, const int *__restrict__ pairs,
                                                         const int *__restrict__ rowptr, const float *__restrict__ mom,
                                                         float *__restrict__ loc)
 {
-    constexpr int NCODE = sib_codes(D), NEXT = sib_ext_codes(D), NN = N * N, NB = N <= 3 ? 4 : (D >= 4 ? 1 : 2);
+    // H = 2: the n0 x n1 nodes of a lane are shared by two lanes, n1/2 values of a1 each (a workgroup of
+    // 2^D siblings x R2 lanes would otherwise fill half a wavefront in 3-D); NN = nodes of a lane
+    constexpr int NCODE = sib_codes(D), NEXT = sib_ext_codes(D), NN = N * N / H, NQ1 = N / H, NB = N <= 3 ? 4 : (D >= 4 ? 1 : 2);
+    static_assert(H == 1 || (H == 2 && N % 2 == 0), "the nodes of dimension 1 are split in halves");
     F3M_DYN_SHARED(float, smem);
     const int tid = threadIdx.x, BD = blockDim.x, lane = tid & 63;
     // The regular table is filled and walked in npass parts (slabs of the last dimension, which is the
@@ -1350,14 +1353,15 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     // This lane: sibling sl, position r2 among the nodes of dimensions >= 2.  The siblings are the fast
     // index: the GS lanes of one r2 read the same moments, so a wavefront's load touches 64/GS short
     // runs of memory instead of 64 (the moment loads are what the level-1 cache has to carry here).
-    const int sl = tid % GS, r2 = tid / GS;
-    const bool valid = r2 < R2;                            // lanes past the last node only keep step
+    const int sl = tid % GS, r2h = tid / GS;               // r2h = r2 * H + h: half h of the a1 range
+    const bool valid = r2h < R2;                           // lanes past the last node only keep step
+    const int r2 = r2h / H, h = r2h % H;
     const int mybox = valid ? sib[sl] : -1;
     const bool live = mybox >= 0;
     int cbit[D], dig[D], lstride[D];
     {
         const int code = sg * GS + sl;
-        int rem = valid ? r2 : 0, st = GS;
+        int rem = valid ? r2 : 0, st = GS * H;
 #pragma unroll
         for (int j = 0; j < D; j++) {
             cbit[j] = 4 + ((code >> j) & 1) + sm.omin[j];  // table index of dimension j = (digit_j + 2) - cbit[j]
@@ -1365,7 +1369,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
             if (j >= 2) { dig[j] = rem % nm.n[j]; rem /= nm.n[j]; lstride[j] = st; st *= nm.n[j]; }   // lstride: in lanes
         }
     }
-    const float *mine = mom + (long long)NN * (live ? r2 : 0);
+    const float *mine = mom + (long long)NN * (live ? r2h : 0);
 
     float acc[D][NN];
 #pragma unroll
@@ -1386,17 +1390,43 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
             int oi = digit2(curpk, 1) - cbit[1];
             oi = min(max(oi, 0), kM2LOffsets - 1);
             const float *T1 = tab01 + ((kM2LOffsets + oi) * N) * 4;
+            if constexpr (H == 1) {
 #pragma unroll
-            for (int a1 = 0; a1 < N; a1++) {
-                const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
-                const float ev[4] = {e.x, e.y, e.z, e.w};
+                for (int a1 = 0; a1 < N; a1++) {
+                    const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
+                    const float ev[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
-                for (int a0 = 0; a0 < N; a0++) {
-                    float t = acc[1][a0 + N * a1];
+                    for (int a0 = 0; a0 < N; a0++) {
+                        float t = acc[1][a0 + N * a1];
 #pragma unroll
-                    for (int q = 0; q < N; q++) t = fmaf(ev[q], acc[0][a0 + N * q], t);
-                    acc[1][a0 + N * a1] = t;
+                        for (int q = 0; q < N; q++) t = fmaf(ev[q], acc[0][a0 + N * q], t);
+                        acc[1][a0 + N * a1] = t;
+                    }
                 }
+            } else {
+                // this lane holds the q1 of its half: partial sums for every a1, then the half of them that
+                // belongs to the partner lane (GS lanes away) is traded for the partner's
+                float part[N * N];
+#pragma unroll
+                for (int a1 = 0; a1 < N; a1++) {
+                    const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
+                    const float ev[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+                    for (int a0 = 0; a0 < N; a0++) {
+                        float t = 0.f;
+#pragma unroll
+                        for (int q = 0; q < NQ1; q++) t = fmaf(h ? ev[NQ1 + q] : ev[q], acc[0][a0 + N * q], t);
+                        part[a0 + N * a1] = t;
+                    }
+                }
+#pragma unroll
+                for (int a1 = 0; a1 < NQ1; a1++)
+#pragma unroll
+                    for (int a0 = 0; a0 < N; a0++) {
+                        const float lo = part[a0 + N * a1], hi = part[a0 + N * (NQ1 + a1)];
+                        const float got = wave_shfl_xor_f(h ? lo : hi, GS);       // what the partner summed for my a1
+                        acc[1][a0 + N * a1] += (h ? hi : lo) + got;
+                    }
             }
         } else {
             __syncthreads();
@@ -1441,7 +1471,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
             const float4 e = *reinterpret_cast<const float4 *>(T0 + a0 * 4);
             const float ev[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
-            for (int q1 = 0; q1 < N; q1++) {
+            for (int q1 = 0; q1 < NQ1; q1++) {
                 float t = acc[0][a0 + N * q1];
 #pragma unroll
                 for (int q = 0; q < N; q++) t = fmaf(ev[q], v.v[q + N * q1], t);
@@ -1504,7 +1534,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
         fvec<NN> r;
 #pragma unroll
         for (int i = 0; i < NN; i++) r.v[i] = acc[D - 1][i];
-        *reinterpret_cast<fvec<NN> *>(loc + (long long)mybox * P + (long long)NN * r2) = r;
+        *reinterpret_cast<fvec<NN> *>(loc + (long long)mybox * P + (long long)NN * r2h) = r;
     }
 }
 
@@ -1627,6 +1657,8 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     int NT = 1;
     for (int j = 0; j < d; j++) NT = std::max(NT, ns.n[j]);
     const int ntab = d * kM2LOffsets * NT * NT;
+    const bool sib_forced = m2l_mode == 3;
+    if (sib_forced) m2l_mode = 0;
     const bool separable = m2l_mode == 2 || (m2l_mode == 0 && (size_t)(ntab + 2 * P) * sizeof(float) <= 48 * 1024);
     if (separable) {
         F3M_REQUIRE((size_t)(ntab + 2 * P) * sizeof(float) <= 64 * 1024, 31, "separable M2L tables do not fit in LDS");
@@ -1647,12 +1679,12 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         timer_begin(kM2L, s);
         const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
         // sibling-group kernel: one tree, 3 <= d <= 5, n0 = n1 in 2..4, every far pair inside the 6^d cells
-        int sibGS = 0, sibR2 = 0, sibPass = 1;
+        int sibGS = 0, sibR2 = 0, sibPass = 1, sibH = 1;
         size_t shsib = 0;
         // (preferred to the per-box kernel for 4 x 4 x 4 nodes as well once a level has a few hundred
         // parents: 0.30 against 0.55 ms at depth 5 of N=1e7; with fewer parents the per-box kernel has
         // more workgroups to offer)
-        const bool enough_parents = !q64 || (lx.depth >= 1 && tx.lev[lx.depth - 1].nb >= 256);
+        const bool enough_parents = sib_forced || !q64 || (lx.depth >= 1 && tx.lev[lx.depth - 1].nb >= 256);
         if (m2l_mode == 0 && enough_parents && &tx == &ty && d >= 3 && d <= 5 && ns.n[0] == ns.n[1] && ns.n[0] >= 2 && ns.n[0] <= 4 &&
             far.outliers == 0 && lx.depth >= 1) {
             const int N = ns.n[0];
@@ -1660,6 +1692,9 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             if (sibR2 <= 1024) {
                 sibGS = 1 << d;
                 while (sibGS * sibR2 > 1024) sibGS >>= 1;
+                // 3-D: 8 siblings x n2 lanes fill at most half a wavefront; two lanes then share a lane's nodes
+                const char *nosplit = getenv("F3M_SIB_SPLIT");   // F3M_SIB_SPLIT=0: testing aid
+                if (d == 3 && N % 2 == 0 && sibGS * sibR2 <= kWave / 2 && !(nosplit && atoi(nosplit) == 0)) { sibH = 2; sibR2 *= 2; }
                 const int bd = ((sibGS * sibR2 + kWave - 1) / kWave) * kWave;
                 // table in 1, 2, 3 or 6 parts: the fewest that fit (a second workgroup per compute unit bought
                 // with two parts did not pay at 6^5 cells: 7.7 -> 8.2 ms; every part scans the far rows again)
@@ -1668,7 +1703,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                 for (int np : {1, 2, 3, 6}) {
                     if (forced > 0 && np != forced && np != 6) continue;
                     sibPass = np;
-                    shsib = sizeof(float) * (2 * (size_t)(sib_codes(d) / np) + 4 * (size_t)sib_ext_codes(d) + (size_t)N * N * bd +
+                    shsib = sizeof(float) * (2 * (size_t)(sib_codes(d) / np) + 4 * (size_t)sib_ext_codes(d) + (size_t)(N * N / sibH) * bd +
                                              (size_t)((ntab + 3) & ~3) + 2 * (size_t)kM2LOffsets * N * 4 + (size_t)N * 4) +
                             sizeof(int) * (size_t)sibGS;
                     if ((shsib <= 150 * 1024 && forced <= 0) || np == forced) break;
@@ -1681,21 +1716,22 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             const int nsub = (1 << d) / sibGS;
             const int bd = ((sibGS * sibR2 + kWave - 1) / kWave) * kWave;
 #ifndef F3M_CPU_EMU
-#define F3M_SIB_ATTR(DD, NNODE)                                                                                        \
-    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE>),                            \
+#define F3M_SIB_ATTR(DD, NNODE, HH)                                                                                    \
+    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE, HH>),                        \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shsib));
 #else
-#define F3M_SIB_ATTR(DD, NNODE)
+#define F3M_SIB_ATTR(DD, NNODE, HH)
 #endif
-#define F3M_SIB(DD, NNODE)                                                                                             \
-    if (d == DD && ns.n[0] == NNODE) {                                                                                 \
-        F3M_SIB_ATTR(DD, NNODE)                                                                                        \
-        F3M_LAUNCH((m2l_sib_kernel<DD, NNODE>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2, sibGS,   \
-                   nsub, sibPass, par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom, loc);   \
+#define F3M_SIB(DD, NNODE, HH)                                                                                         \
+    if (d == DD && ns.n[0] == NNODE && sibH == HH) {                                                                   \
+        F3M_SIB_ATTR(DD, NNODE, HH)                                                                                    \
+        F3M_LAUNCH((m2l_sib_kernel<DD, NNODE, HH>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2,      \
+                   sibGS, nsub, sibPass, par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom,  \
+                   loc);                                                                                               \
     }
-            F3M_SIB(3, 2) F3M_SIB(3, 3) F3M_SIB(3, 4)
-            F3M_SIB(4, 2) F3M_SIB(4, 3) F3M_SIB(4, 4)
-            F3M_SIB(5, 2) F3M_SIB(5, 3) F3M_SIB(5, 4)
+            F3M_SIB(3, 2, 2) F3M_SIB(3, 3, 1) F3M_SIB(3, 4, 2) F3M_SIB(3, 2, 1) F3M_SIB(3, 4, 1)
+            F3M_SIB(4, 2, 1) F3M_SIB(4, 3, 1) F3M_SIB(4, 4, 1)
+            F3M_SIB(5, 2, 1) F3M_SIB(5, 3, 1) F3M_SIB(5, 4, 1)
 #undef F3M_SIB
 #undef F3M_SIB_ATTR
         } else if (q64) {

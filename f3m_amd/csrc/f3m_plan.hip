@@ -329,9 +329,11 @@ static void check_level(const f3m_plan *P, int level)
 
 static int m2l_mode_env()
 {
-    // F3M_M2L=direct|separable forces one form of the M2L kernel (default: separable when its tables fit)
+    // F3M_M2L=direct|separable forces one form of the M2L kernel (default: separable when its tables fit);
+    // F3M_M2L=sibling takes the sibling-group kernel wherever it applies, also at levels with few parents
     int mode = 0;
-    if (const char *e = getenv("F3M_M2L")) mode = !strcmp(e, "direct") ? 1 : (!strcmp(e, "separable") ? 2 : 0);
+    if (const char *e = getenv("F3M_M2L"))
+        mode = !strcmp(e, "direct") ? 1 : (!strcmp(e, "separable") ? 2 : (!strcmp(e, "sibling") ? 3 : 0));
     return mode;
 }
 

@@ -204,6 +204,25 @@ def test_m2l_sibling_table_in_parts(monkeypatch, parts):
     assert np.array_equal(whole, eng.apply(b))
 
 
+@pytest.mark.parametrize("P", [8, 64])
+def test_m2l_sibling_nodes_shared_by_two_lanes(monkeypatch, P):
+    """3-D sibling-group M2L: two lanes share the n0 x n1 nodes of a lane (full wavefronts); same sums as the
+    one-lane form up to the order of two additions"""
+    rng = np.random.default_rng(6)
+    n, mp = (2500, 60) if P == 8 else (6000, 150)
+    X = rng.random((n, 3), dtype=f32)
+    b = rng.standard_normal((n, 1)).astype(f32)
+    eng = ee.Plan(X, None, ls=0.6, min_points=mp, nr_of_interpolation=P, small_field_points=P + 10)
+    assert any(eng.level_sizes(k)["nfar"] for k in range(1, eng.depth + 1))
+    monkeypatch.setenv("F3M_M2L", "sibling")               # also at levels with few parents
+    shared = eng.apply(b)
+    monkeypatch.setenv("F3M_SIB_SPLIT", "0")
+    single = eng.apply(b)
+    assert 0 < rel_l2(shared, single) < 1e-6
+    monkeypatch.setenv("F3M_M2L", "direct")
+    assert rel_l2(shared, eng.apply(b)) < 3e-6
+
+
 def test_mfma_near_field(oracle, monkeypatch):
     monkeypatch.setenv("F3M_NEAR", "mfma")
     rng = np.random.default_rng(5)

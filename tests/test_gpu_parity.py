@@ -240,6 +240,24 @@ def test_m2l_sibling_table_in_parts(eng, monkeypatch, name, parts):
     assert np.array_equal(default, plan.apply(dev(b)).cpu().numpy())
 
 
+@pytest.mark.parametrize("nodes", [8, 64])
+def test_m2l_sibling_nodes_shared_by_two_lanes(eng, monkeypatch, nodes):
+    """3-D sibling-group M2L with two lanes per n0 x n1 node set (default) against one lane per set and
+    against the direct form of the reference (F3M_src/1_d_conv.cu:741-817)."""
+    print("case m2l shared nodes", nodes, flush=True)
+    rng = np.random.default_rng(16)
+    X = rng.random((400000, 3), dtype=f32)
+    b = rng.standard_normal((400000, 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, ls=1.0, nr_of_interpolation=nodes, min_points=150, small_field_points=100)
+    assert plan.depth == 4 and plan.level_sizes(4)["nfar"] > 0     # 512 parents at the deepest level
+    shared = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_SIB_SPLIT", "0")
+    single = plan.apply(dev(b)).cpu().numpy()
+    assert 0 < rel_l2(shared, single) < 1e-6
+    monkeypatch.setenv("F3M_M2L", "direct")
+    assert rel_l2(shared, plan.apply(dev(b)).cpu().numpy()) < 5e-6
+
+
 def test_m2l_children_of_parent_pairs_kept_on_the_far_threshold(eng, monkeypatch):
     """A parent pair two cells apart along one axis is exactly 2 edges away; fp32 rounding of the centres
     decides whether the reference's predicate (F3M_src/1_d_conv.cu:936-941) calls it far.  Where it is
