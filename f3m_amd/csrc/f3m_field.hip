@@ -423,7 +423,7 @@ struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floa
 // NC right-hand sides at once: the exponential of a pair is computed once and multiplies NC weights
 // (columns of bs, bstride apart; results to NC columns of outs, ostride apart).
 template <int D, int TPW, int NC>
-__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 2) near_g_kernel(
+__global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 && NC == 1) ? 5 : 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
@@ -664,7 +664,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // Where the plan has counted the rows of the list, "typical" is the mean over the listed boxes and the
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
-    const int tpw = ((avg_points + 31) / 32 == 5 && nc == 1) ? 5 : 4;
+    int tpw = ((avg_points + 31) / 32 == 5 && nc == 1) ? 5 : 4;
+    if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
     int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? tpw * 32 : bd * T, tileoff, s);
     if (use_mfma && list.rows >= 0) ntiles = (int)std::max<long long>(1, tpw == 5 ? list.items160 : list.items128);
     float sc = sqrtf(lcs * kLog2e);
