@@ -954,6 +954,90 @@ __global__ void __launch_bounds__(1024) p2m_kernel(const float *__restrict__ ys,
     if (tid < nm.P) partial[(long long)blockIdx.x * nm.P + tid] = acc;
 }
 
+// P2M for the 4 x 4 x 4 grid: one wavefront per (box, chunk of points).  64 points at a time: every lane
+// prepares one point -- its twelve 1-D basis values in registers, then l0[0..3] and the 16 products
+// w[a1 + 4 a2] = l1[a1] l2[a2] b to LDS -- and then lane (g, q), g = lane / 16, adds the points
+// 16 g .. 16 g + 15 to its four moments (a0, q): one multiply-add per node and point, where the
+// lane-per-node form spends two multiplications and three LDS reads as well.  The four partial sums
+// of a node are added across the wavefront at the end.  Same partial-sum layout as p2m_kernel.
+__device__ inline void basis4(float t, const float (&nt)[4], const float (&nw)[4], float (&out)[4], float scale)
+{
+    float sum = 0.f;
+    int hit = -1;
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+        const float diff = t - nt[a];
+        if (diff == 0.f) hit = a;
+        out[a] = nw[a] * fast_rcp(diff);
+        sum += out[a];
+    }
+    const float inv = scale * fast_rcp(sum);
+#pragma unroll
+    for (int a = 0; a < 4; a++) out[a] = hit >= 0 ? (a == hit ? scale : 0.f) : out[a] * inv;
+}
+
+__global__ void __launch_bounds__(64) p2m_q64_kernel(const float *__restrict__ ys, long long M, const float *__restrict__ bs,
+                                                      const int *__restrict__ off, const float *__restrict__ ctr,
+                                                      const int *__restrict__ tileoff, int nb, const float *__restrict__ nt,
+                                                      const float *__restrict__ nw, float factor, float *__restrict__ partial)
+{
+    // w of point p at 16 p + 16 (p / 16): the four groups of the accumulation read different banks
+    __shared__ __align__(16) float sl0[64 * 4];
+    __shared__ __align__(16) float sw[64 * 16 + 64];
+    const int lane = threadIdx.x;
+    if ((int)blockIdx.x >= tileoff[nb]) return;     // launched with an upper bound of the chunk count
+    const int box = find_box(tileoff, nb, blockIdx.x);
+    const int chunk = blockIdx.x - tileoff[box];
+    const int p0 = off[box] + chunk * kP2MChunk;
+    const int p1 = min(off[box + 1], p0 + kP2MChunk);
+    float tn[3][4], tw[3][4], c[3];
+#pragma unroll
+    for (int k = 0; k < 3; k++) {
+        c[k] = ctr[(long long)box * 3 + k];
+#pragma unroll
+        for (int a = 0; a < 4; a++) { tn[k][a] = nt[4 * k + a]; tw[k][a] = nw[4 * k + a]; }
+    }
+    const int g = lane >> 4, q = lane & 15;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = p0; s0 < p1; s0 += 64) {
+        const int i = s0 + lane;
+        const bool in = i < p1;
+        float l[3][4];
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            const float t = in ? factor * (ys[(long long)k * M + i] - c[k]) : 0.f;
+            basis4(t, tn[k], tw[k], l[k], 1.f);
+        }
+        const float b = in ? bs[i] : 0.f;            // lanes past the end add nothing
+        __syncthreads();                             // the previous round has been read
+        *reinterpret_cast<float4 *>(sl0 + 4 * lane) = make_float4(l[0][0], l[0][1], l[0][2], l[0][3]);
+        float *wrow = sw + 16 * lane + 16 * (lane >> 4);
+#pragma unroll
+        for (int a2 = 0; a2 < 4; a2++) {
+            const float lb = l[2][a2] * b;
+            *reinterpret_cast<float4 *>(wrow + 4 * a2) = make_float4(l[1][0] * lb, l[1][1] * lb, l[1][2] * lb, l[1][3] * lb);
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int pt = 0; pt < 16; pt++) {
+            const int pp = 16 * g + pt;
+            const float4 l0 = *reinterpret_cast<const float4 *>(sl0 + 4 * pp);
+            const float w = sw[16 * pp + 16 * g + q];
+            acc[0] = fmaf(l0.x, w, acc[0]);
+            acc[1] = fmaf(l0.y, w, acc[1]);
+            acc[2] = fmaf(l0.z, w, acc[2]);
+            acc[3] = fmaf(l0.w, w, acc[3]);
+        }
+    }
+#pragma unroll
+    for (int a = 0; a < 4; a++) {
+        acc[a] += wave_shfl_xor_f(acc[a], 16);
+        acc[a] += wave_shfl_xor_f(acc[a], 32);
+    }
+    if (g == 0)                                      // node a0 + 4 q
+        *reinterpret_cast<float4 *>(partial + (long long)blockIdx.x * 64 + 4 * q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+}
+
 __global__ void p2m_reduce_kernel(const float *__restrict__ partial, const int *__restrict__ tileoff, int nb, int P,
                                   float *__restrict__ mom)
 {
@@ -1632,7 +1716,11 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
                    ly.nb, nm, ns.dt.get(), ns.dw.get(), factor, partial.get());                                        \
         break;
     timer_begin(kP2M, s);
-    if (nty > 0) {
+    if (nty > 0 && d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4) {
+        F3M_LAUNCH(p2m_q64_kernel, nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(), ly.nb,
+                   ns.dt.get(), ns.dw.get(), factor, partial.get());
+        check_launch("p2m_q64");
+    } else if (nty > 0) {
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
             F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
