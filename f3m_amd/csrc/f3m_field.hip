@@ -2007,6 +2007,65 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restr
     outs[i] += acc;
 }
 
+// The same for other tensor grids of N nodes per dimension: the weights of the nodes of dimensions >= 1
+// are formed once per point, the expansion is read in rows of N.
+template <int D, int N>
+__global__ void __launch_bounds__(kL2PBlock) l2p_tensor_kernel(const float *__restrict__ xs, long long NP, float *__restrict__ outs,
+                                                                const int *__restrict__ off, const float *__restrict__ ctr,
+                                                                int nb, const float *__restrict__ nt,
+                                                                const float *__restrict__ nw, float factor,
+                                                                const float *__restrict__ loc)
+{
+    constexpr int Q = ipow(N, D - 1), P = Q * N;
+    __shared__ int bounds[kL2PBlock];
+    const int tid = threadIdx.x;
+    const long long i0 = (long long)blockIdx.x * kL2PBlock;
+    int lo = 0, hi = nb;                            // box of the first point: last b with off[b] <= i0
+    while (hi - lo > 1) {
+        int mid = lo + ((hi - lo) >> 1);
+        if (off[mid] <= i0) lo = mid; else hi = mid;
+    }
+    const int b0 = lo;
+    bounds[tid] = off[min(b0 + 1 + tid, nb)];      // starts of the next boxes (off[nb] = NP closes the list)
+    __syncthreads();
+    const long long i = i0 + tid;
+    if (i >= NP) return;
+    int a = 0, b = kL2PBlock;                       // number of those starts that are <= i
+    while (a < b) {
+        int mid = (a + b) >> 1;
+        if (bounds[mid] <= i) a = mid + 1; else b = mid;
+    }
+    const int box = b0 + a;
+    float l[D][N];
+#pragma unroll
+    for (int k = 0; k < D; k++) {
+        const float t = factor * (xs[(long long)k * NP + i] - ctr[(long long)box * D + k]);
+        basis_1d(t, nt + N * k, nw + N * k, N, l[k], 1.f);
+    }
+    float w[Q];                                     // w[j] = prod_{k >= 1} l_k[digit_k(j)], dimension 1 fastest
+    w[0] = 1.f;
+    int len = 1;
+#pragma unroll
+    for (int k = D - 1; k >= 1; k--) {
+#pragma unroll
+        for (int j = len - 1; j >= 0; j--)
+#pragma unroll
+            for (int e = N - 1; e >= 0; e--) w[j * N + e] = w[j] * l[k][e];
+        len *= N;
+    }
+    const float *lp = loc + (long long)box * P;
+    float acc = 0.f;
+#pragma unroll
+    for (int j = 0; j < Q; j++) {
+        const fvec<N> r = *reinterpret_cast<const fvec<N> *>(lp + N * j);
+        float inner = l[0][0] * r.v[0];
+#pragma unroll
+        for (int e = 1; e < N; e++) inner = fmaf(l[0][e], r.v[e], inner);
+        acc = fmaf(w[j], inner, acc);
+    }
+    outs[i] += acc;
+}
+
 void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
                hipStream_t s)
 {
@@ -2020,6 +2079,30 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
                    lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_q64");
+        return;
+    }
+    if (flag == nullptr && d == 4 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH((l2p_tensor_kernel<4, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_tensor");
+        return;
+    }
+    if (flag == nullptr && d == 5 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3 && ns.n[4] == 3) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH((l2p_tensor_kernel<5, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_tensor");
+        return;
+    }
+    if (flag == nullptr && d == 3 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH((l2p_tensor_kernel<3, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_tensor");
         return;
     }
     DBuf<int> tilex;
