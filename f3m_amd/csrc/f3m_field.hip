@@ -1038,18 +1038,19 @@ __global__ void __launch_bounds__(64) p2m_q64_kernel(const float *__restrict__ y
         *reinterpret_cast<float4 *>(partial + (long long)blockIdx.x * 64 + 4 * q) = make_float4(acc[0], acc[1], acc[2], acc[3]);
 }
 
-// The same scheme for other tensor grids of N nodes per dimension with Q = N^(D-1) <= 64: lane (g, q),
-// g = lane / Q < G = 64 / Q, adds the points of its group to the N moments (a0, q).
+// The same scheme for other tensor grids of N nodes per dimension: a lane holds the N^R moments of the
+// first R dimensions for one combination q of the others, Q = N^(D-R) <= 64; lane (g, q), g = lane / Q <
+// G = 64 / Q, adds the points of its group.
 __host__ __device__ constexpr int ipow(int b, int e) { return e == 0 ? 1 : b * ipow(b, e - 1); }
-template <int D, int N>
+template <int D, int N, int R>
 __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict__ ys, long long M, const float *__restrict__ bs,
                                                          const int *__restrict__ off, const float *__restrict__ ctr,
                                                          const int *__restrict__ tileoff, int nb, const float *__restrict__ nt,
                                                          const float *__restrict__ nw, float factor, float *__restrict__ partial)
 {
-    constexpr int Q = ipow(N, D - 1), G = 64 / Q, PG = (64 + G - 1) / G, QS = Q | 1, P = Q * N;   // QS: odd row stride
-    static_assert(Q <= 64, "one wavefront holds the nodes of dimensions >= 1");
-    __shared__ float sl0[64 * N];
+    constexpr int NR = ipow(N, R), Q = ipow(N, D - R), G = 64 / Q, PG = (64 + G - 1) / G, QS = Q | 1, P = Q * NR;   // QS: odd row stride
+    static_assert(Q <= 64 && NR <= QS, "one wavefront holds the nodes of the last D-R dimensions");
+    __shared__ float sh[64 * NR];
     __shared__ float sw[64 * QS];
     const int lane = threadIdx.x;
     if ((int)blockIdx.x >= tileoff[nb]) return;     // launched with an upper bound of the chunk count
@@ -1058,9 +1059,9 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
     const int p0 = off[box] + chunk * kP2MChunk;
     const int p1 = min(off[box + 1], p0 + kP2MChunk);
     const int g = lane / Q, q = lane % Q;
-    float acc[N];
+    float acc[NR];
 #pragma unroll
-    for (int a = 0; a < N; a++) acc[a] = 0.f;
+    for (int a = 0; a < NR; a++) acc[a] = 0.f;
     for (int s0 = p0; s0 < p1; s0 += 64) {
         const int i = s0 + lane;
         const bool in = i < p1;
@@ -1072,20 +1073,30 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
         }
         const float b = in ? bs[i] : 0.f;            // lanes past the end add nothing
         __syncthreads();                             // the previous round has been read
-#pragma unroll
-        for (int a = 0; a < N; a++) sl0[N * lane + a] = l[0][a];
-        // w[j] = b prod_{k >= 1} l_k[digit_k(j)], built dimension by dimension from the last
-        float w[Q];
+        // products over a range of dimensions, built dimension by dimension from the last (first one fastest)
+        float h[NR], w[Q];
+        h[0] = 1.f;
         w[0] = b;
         int len = 1;
 #pragma unroll
-        for (int k = D - 1; k >= 1; k--) {
+        for (int k = R - 1; k >= 0; k--) {
+#pragma unroll
+            for (int j = len - 1; j >= 0; j--)
+#pragma unroll
+                for (int a = N - 1; a >= 0; a--) h[j * N + a] = h[j] * l[k][a];
+            len *= N;
+        }
+        len = 1;
+#pragma unroll
+        for (int k = D - 1; k >= R; k--) {
 #pragma unroll
             for (int j = len - 1; j >= 0; j--)
 #pragma unroll
                 for (int a = N - 1; a >= 0; a--) w[j * N + a] = w[j] * l[k][a];
             len *= N;
         }
+#pragma unroll
+        for (int a = 0; a < NR; a++) sh[NR * lane + a] = h[a];
 #pragma unroll
         for (int j = 0; j < Q; j++) sw[QS * lane + j] = w[j];
         __syncthreads();
@@ -1095,21 +1106,21 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
                 if (pp >= 64) break;
                 const float wv = sw[QS * pp + q];
 #pragma unroll
-                for (int a = 0; a < N; a++) acc[a] = fmaf(sl0[N * pp + a], wv, acc[a]);
+                for (int a = 0; a < NR; a++) acc[a] = fmaf(sh[NR * pp + a], wv, acc[a]);
             }
         }
     }
     // add the groups: lanes q, Q + q, 2Q + q, ... hold partial sums of the same nodes
     __syncthreads();
 #pragma unroll
-    for (int a = 0; a < N; a++) sw[lane * N + a] = g < G ? acc[a] : 0.f;
+    for (int a = 0; a < NR; a++) sw[lane * NR + a] = g < G ? acc[a] : 0.f;
     __syncthreads();
     if (lane < Q) {
 #pragma unroll
-        for (int a = 0; a < N; a++) {
+        for (int a = 0; a < NR; a++) {
             float t = 0.f;
-            for (int gg = 0; gg < G; gg++) t += sw[(gg * Q + lane) * N + a];
-            partial[(long long)blockIdx.x * P + a + N * lane] = t;
+            for (int gg = 0; gg < G; gg++) t += sw[(gg * Q + lane) * NR + a];
+            partial[(long long)blockIdx.x * P + a + NR * lane] = t;
         }
     }
 }
@@ -1797,11 +1808,15 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
                    ns.dt.get(), ns.dw.get(), factor, partial.get());
         check_launch("p2m_q64");
     } else if (nty > 0 && d == 4 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3) {
-        F3M_LAUNCH((p2m_tensor_kernel<4, 3>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
+        F3M_LAUNCH((p2m_tensor_kernel<4, 3, 1>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
+                   ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
+        check_launch("p2m_tensor");
+    } else if (nty > 0 && d == 5 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3 && ns.n[4] == 3) {
+        F3M_LAUNCH((p2m_tensor_kernel<5, 3, 2>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
                    ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
         check_launch("p2m_tensor");
     } else if (nty > 0 && d == 3 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3) {
-        F3M_LAUNCH((p2m_tensor_kernel<3, 3>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
+        F3M_LAUNCH((p2m_tensor_kernel<3, 3, 1>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
                    ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
         check_launch("p2m_tensor");
     } else if (nty > 0) {
