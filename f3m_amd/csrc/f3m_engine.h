@@ -31,6 +31,9 @@ struct TreeLevel {
     mutable float nearops_sc = 0.f;
     mutable bool nearops_partial = false;   // built for the source boxes of one list only
     // grid key -> box id table of this level (built on first use by lookup_boxes)
+    // box of every 32nd point (npoints/32 + 2 entries, built on first use by box_table): kernels that
+    // take points in fixed-size pieces start from here instead of searching the offsets
+    mutable DBuf<int> box32;
     mutable DBuf<uint32_t> hashtab;      // hashcap pairs (key, value), empty = 0xffffffff
     mutable uint32_t hashcap = 0;
 };

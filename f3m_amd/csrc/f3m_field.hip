@@ -196,6 +196,28 @@ __device__ inline int find_box(const int *__restrict__ tileoff, int nb, int tile
     return lo;
 }
 
+// box32[k] = box of point 32 k (the last box for k past the end).  A workgroup that owns a fixed-size
+// piece of the points would otherwise open with a binary search over the offsets, some 17 dependent
+// loads that take longer than the piece's own work.
+__global__ void box_table_kernel(const int *__restrict__ off, int nb, long long npoints, int nent, int *__restrict__ box32)
+{
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= nent) return;
+    const long long p = min((long long)k * 32, npoints - 1);
+    box32[k] = find_box(off, nb, (int)max(0ll, p));
+}
+
+static const int *box_table(const TreeLevel &lev, long long npoints, hipStream_t s)
+{
+    const int nent = (int)(npoints / 32) + 2;
+    if (lev.box32.size() != (size_t)nent) {
+        lev.box32.reset((size_t)nent);
+        F3M_LAUNCH(box_table_kernel, cdiv(nent, 256), 256, 0, s, lev.off.get(), lev.nb, npoints, nent, lev.box32.get());
+        check_launch("box_table");
+    }
+    return lev.box32.get();
+}
+
 // ------------------------------------------------------------------------------------------------
 // near field (F3M_src/1_d_conv.cu:255-335): out_i += sum over the y boxes listed for the box of i of
 // sum_j exp(-|x_i-y_j|^2 lcs) b_j.  One workgroup per (x box, tile of targets); the sources of a y
@@ -353,7 +375,8 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
                                                                   const int *__restrict__ off, int nb,
                                                                   const int *__restrict__ cell, Geo geo, float edge,
                                                                   float sc, long long stride,
-                                                                  const int *__restrict__ need, h8 *__restrict__ ops)
+                                                                  const int *__restrict__ need, const int *__restrict__ box32,
+                                                                  h8 *__restrict__ ops)
 {
     constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
     constexpr int NS = near_insts(D);
@@ -361,8 +384,10 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
     const int tid = threadIdx.x;
     const long long i0 = (long long)blockIdx.x * kOpsBlock, i = i0 + tid;
     // boxes of the first point of this workgroup and of the point 31 before it (uniform)
-    const int b0 = find_box(off, nb, (int)min(i0, M - 1));
-    const int b0m = find_box(off, nb, (int)max(0ll, min(i0, M - 1) - 31));
+    const long long pm = max(0ll, min(i0, M - 1) - 31);
+    int b0 = box32[min(i0, M - 1) / 32], b0m = box32[pm / 32];
+    while (off[b0 + 1] <= min(i0, M - 1)) b0++;      // at most the boxes that start inside 32 points
+    while (off[b0m + 1] <= pm) b0m++;
     bounds[tid] = off[min(b0 + 1 + tid, nb)];       // starts of the following boxes; off[nb] = M closes the list
     __syncthreads();
     if (i >= stride) return;
@@ -687,11 +712,12 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                 need.reset((size_t)ly.nb + 1);
                 exclusive_scan_i32(fy.get(), ly.nb, need.get(), s);
             }
+            const int *box32 = box_table(ly, ty.n, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
         F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
                    ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
-                   only_list ? need.get() : (const int *)nullptr,                                                     \
+                   only_list ? need.get() : (const int *)nullptr, box32,                                              \
                    reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
         break;
             switch (d) {
@@ -1977,20 +2003,14 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 // 1-D basis values in registers.
 __global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restrict__ xs, long long N, float *__restrict__ outs,
                                                              const int *__restrict__ off, const float *__restrict__ ctr,
-                                                             int nb, const float *__restrict__ nt,
-                                                             const float *__restrict__ nw, float factor,
-                                                             const float *__restrict__ loc)
+                                                             int nb, const int *__restrict__ box32,
+                                                             const float *__restrict__ nt, const float *__restrict__ nw,
+                                                             float factor, const float *__restrict__ loc)
 {
     __shared__ int bounds[kL2PBlock];
     const int tid = threadIdx.x;
     const long long i0 = (long long)blockIdx.x * kL2PBlock;
-    // box of the first point: last b with off[b] <= i0
-    int lo = 0, hi = nb;
-    while (hi - lo > 1) {
-        int mid = lo + ((hi - lo) >> 1);
-        if (off[mid] <= i0) lo = mid; else hi = mid;
-    }
-    const int b0 = lo;
+    const int b0 = box32[i0 / 32];                  // box of the first point (i0 is a multiple of 32)
     bounds[tid] = off[min(b0 + 1 + tid, nb)];      // starts of the next boxes (off[nb] = N closes the list)
     __syncthreads();
     const long long i = i0 + tid;
@@ -2027,20 +2047,15 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restr
 template <int D, int N>
 __global__ void __launch_bounds__(kL2PBlock) l2p_tensor_kernel(const float *__restrict__ xs, long long NP, float *__restrict__ outs,
                                                                 const int *__restrict__ off, const float *__restrict__ ctr,
-                                                                int nb, const float *__restrict__ nt,
-                                                                const float *__restrict__ nw, float factor,
-                                                                const float *__restrict__ loc)
+                                                                int nb, const int *__restrict__ box32,
+                                                                const float *__restrict__ nt, const float *__restrict__ nw,
+                                                                float factor, const float *__restrict__ loc)
 {
     constexpr int Q = ipow(N, D - 1), P = Q * N;
     __shared__ int bounds[kL2PBlock];
     const int tid = threadIdx.x;
     const long long i0 = (long long)blockIdx.x * kL2PBlock;
-    int lo = 0, hi = nb;                            // box of the first point: last b with off[b] <= i0
-    while (hi - lo > 1) {
-        int mid = lo + ((hi - lo) >> 1);
-        if (off[mid] <= i0) lo = mid; else hi = mid;
-    }
-    const int b0 = lo;
+    const int b0 = box32[i0 / 32];                  // box of the first point (i0 is a multiple of 32)
     bounds[tid] = off[min(b0 + 1 + tid, nb)];      // starts of the next boxes (off[nb] = NP closes the list)
     __syncthreads();
     const long long i = i0 + tid;
@@ -2091,7 +2106,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4) {
         timer_begin(kL2P, s);
         F3M_LAUNCH(l2p_q64_kernel, cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_q64");
         return;
@@ -2099,7 +2114,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 4 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<4, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2107,7 +2122,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 5 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3 && ns.n[4] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<5, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2115,7 +2130,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<3, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
