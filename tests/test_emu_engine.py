@@ -204,6 +204,18 @@ def test_m2l_sibling_table_in_parts(monkeypatch, parts):
     assert np.array_equal(whole, eng.apply(b))
 
 
+def test_m2l_sibling_parents_longest_first(monkeypatch):
+    """the sibling-group M2L may start the parents with the longest far rows first: the same sums, bit for bit"""
+    rng = np.random.default_rng(8)
+    X = rng.random((3000, 3), dtype=f32)
+    b = rng.standard_normal((3000, 1)).astype(f32)
+    eng = ee.Plan(X, None, ls=0.6, min_points=60, nr_of_interpolation=27, small_field_points=37)
+    monkeypatch.setenv("F3M_SIB_ORDER", "0")
+    plain = eng.apply(b)
+    monkeypatch.setenv("F3M_SIB_ORDER", "1")
+    assert np.array_equal(plain, eng.apply(b))
+
+
 @pytest.mark.parametrize("P", [8, 64])
 def test_m2l_sibling_nodes_shared_by_two_lanes(monkeypatch, P):
     """3-D sibling-group M2L: two lanes share the n0 x n1 nodes of a lane (full wavefronts); same sums as the

@@ -240,6 +240,21 @@ def test_m2l_sibling_table_in_parts(eng, monkeypatch, name, parts):
     assert np.array_equal(default, plan.apply(dev(b)).cpu().numpy())
 
 
+@pytest.mark.parametrize("name", ["C1_uniform3", "uniform4", "uniform5_243"])
+def test_m2l_sibling_parents_longest_first(eng, monkeypatch, name):
+    """The sibling-group M2L may start the parents with the longest far rows first (default in d >= 4 when
+    there are few parents): the same sums, bit for bit."""
+    print("case m2l parent order", name, flush=True)
+    rng = np.random.default_rng(17)
+    X, Y, prm = clouds(name, rng)
+    b = rng.standard_normal((X.shape[0], 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, **prm)
+    monkeypatch.setenv("F3M_SIB_ORDER", "0")
+    plain = plan.apply(dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_SIB_ORDER", "1")
+    assert np.array_equal(plain, plan.apply(dev(b)).cpu().numpy())
+
+
 @pytest.mark.parametrize("nodes", [8, 64])
 def test_m2l_sibling_nodes_shared_by_two_lanes(eng, monkeypatch, nodes):
     """3-D sibling-group M2L with two lanes per n0 x n1 node set (default) against one lane per set and
