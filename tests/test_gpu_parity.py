@@ -255,6 +255,22 @@ def test_m2l_sibling_parents_longest_first(eng, monkeypatch, name):
     assert np.array_equal(plain, plan.apply(dev(b)).cpu().numpy())
 
 
+def test_near_field_longest_lists_first(eng, monkeypatch):
+    """The matrix-pipe near field may take the boxes with the longest lists first (default from five
+    dimensions on): the same sums for every target, bit for bit."""
+    print("case near order", flush=True)
+    rng = np.random.default_rng(18)
+    X = rng.random((3_000_000, 3), dtype=f32)
+    b = rng.standard_normal((3_000_000, 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, ls=1.0, min_points=200)              # depth 5, ~92 points per box: 32768 work items
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_NEAR_ORDER", "0")
+    plain = plan.near_level(plan.depth, "small", dev(b)).cpu().numpy()
+    monkeypatch.setenv("F3M_NEAR_ORDER", "1")
+    assert plan.list_rows(plan.depth)[2] >= 16384                      # not sliced: the order applies
+    assert np.array_equal(plain, plan.near_level(plan.depth, "small", dev(b)).cpu().numpy())
+
+
 @pytest.mark.parametrize("nodes", [8, 64])
 def test_m2l_sibling_nodes_shared_by_two_lanes(eng, monkeypatch, nodes):
     """3-D sibling-group M2L with two lanes per n0 x n1 node set (default) against one lane per set and
