@@ -1520,18 +1520,6 @@ __global__ void sib_class_count_kernel(const int *__restrict__ childstart, const
     cls[p] = c;
     atomicAdd(&hist[c], 1);
 }
-__global__ void sib_class_place_kernel(const int *__restrict__ cls, int npar, int *__restrict__ hist, int *__restrict__ order)
-{
-    __shared__ int start[256];
-    if (threadIdx.x == 0) {                          // 256 classes: a serial scan is enough
-        int run = 0;
-        for (int c = 0; c < 256; c++) { start[c] = run; run += hist[c]; }
-    }
-    __syncthreads();
-    // one workgroup places every parent: the cursors live in LDS
-    for (int p = threadIdx.x; p < npar; p += blockDim.x) order[atomicAdd(&start[cls[p]], 1)] = p;
-}
-
 template <int D, int N, int H>
 __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
                                                         int R2, int GS, int nsub, int npass, const int *__restrict__ order,
@@ -2020,7 +2008,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                 F3M_LAUNCH(sib_class_count_kernel, cdiv(par.nb, 256), 256, 0, s, par.childstart.get(), far.rowptr.get(), par.nb,
                            unit, cls.get(), hist.get());
                 check_launch("sib_class_count");
-                F3M_LAUNCH(sib_class_place_kernel, 1, 1024, 0, s, cls.get(), par.nb, hist.get(), sibOrder.get());
+                F3M_LAUNCH(class_place_kernel, 1, 1024, 0, s, cls.get(), par.nb, hist.get(), sibOrder.get());
                 check_launch("sib_class_place");
             }
             const int *sibOrd = ordered ? sibOrder.get() : (const int *)nullptr;
