@@ -19,7 +19,7 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak
 # HBM bytes moved by one near-field launch of the default workload, from the rocprofv3 FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/ (None until measured)
-NEAR_TRAFFIC_BYTES = 6.073e9
+NEAR_TRAFFIC_BYTES = 6.072e9
 
 
 def cpu_baseline(X, Y, b, ls, budget_s=15.0):
