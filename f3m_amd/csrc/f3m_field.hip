@@ -692,10 +692,10 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                 bool only_list)
 {
     if (list.n == 0) return;
-    F3M_REQUIRE(nc == 1 || nc == 4, 34, "near field takes 1 or 4 columns at a time");
+    F3M_REQUIRE(nc == 1 || nc == 2 || nc == 4, 34, "near field takes 1, 2 or 4 columns at a time");
     // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to about
-    // 2^-22 times the largest term, |x''|^2 <= 30 d (sc edge)^2 (listed targets lie within 5.5 edges per
-    // dimension of the source box centre); it is used while that bound stays below 1e-4 (box edge up to
+    // 2^-22 times the largest term, |x''|^2 <= 30 d (sc edge)^2 (listed targets lie within 5 edges per
+    // dimension of the anchor of their sources); it is used while that bound stays below 1e-4 (box edge up to
     // ~2 lengthscales in 3-D), otherwise the all-vector kernel.
     // F3M_NEAR=valu|mfma overrides the choice.
     const float sc_edge = sqrtf(lcs * kLog2e) * lx.edge;
@@ -800,6 +800,11 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
         else if (nc == 4)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
+                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
+        else if (nc == 2)                                                                                             \
+            F3M_LAUNCH((near_g_kernel<DD, 4, 2>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \

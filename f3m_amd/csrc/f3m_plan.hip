@@ -412,8 +412,8 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         F3M_HIP(hipStreamSynchronize(s));
         return;
     }
-    // Columns are taken four at a time when at least two are left (the near field then computes every
-    // exponential once for the four), else one at a time.  bs columns are padded by one tile:
+    // Columns are taken four at a time while at least three are left (the near field then computes every
+    // exponential once for the four), two at a time when two are left, else one.  bs columns are padded by one tile:
     // near_g_kernel reads whole tiles.
     const long long bstride = P->M + 32, ostride = P->N;
     const int width = c >= 2 ? 4 : 1;
@@ -424,7 +424,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     const bool per_level = fe && !strcmp(fe, "levels");
     for (int col = 0; col < c;) {
         const int left = c - col;
-        const int nc = left >= 2 ? 4 : 1;          // columns processed in this pass (past `left`: zero weights)
+        const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);   // columns of this pass (past `left`: zero weights)
         const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
