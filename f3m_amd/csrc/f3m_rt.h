@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <chrono>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
@@ -231,17 +232,17 @@ __global__ void export_kernel(const T *__restrict__ src, T *__restrict__ dst, in
 // waits until the GPU has stored seq into *flag
 inline void await_flag(const unsigned *flag, unsigned seq, hipStream_t s)
 {
+    // F3M_SPIN_LIMIT_MS overrides the limit; 0 goes straight to the stream wait (test of that path)
+    int limit = kSpinLimitMs;
+    if (const char *e = getenv("F3M_SPIN_LIMIT_MS")) limit = atoi(e);
     const auto t0 = std::chrono::steady_clock::now();
-    for (unsigned spins = 1;; spins++) {
+    for (unsigned spins = 1; limit > 0; spins++) {
         if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) == seq) return;
         __builtin_ia32_pause();
-        if ((spins & 0xfff) == 0 &&
-            std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(kSpinLimitMs)) {
-            F3M_HIP(hipStreamSynchronize(s));
-            if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) throw Error(102, "result of a device kernel did not arrive");
-            return;
-        }
+        if ((spins & 0xfff) == 0 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(limit)) break;
     }
+    F3M_HIP(hipStreamSynchronize(s));
+    if (__atomic_load_n(flag, __ATOMIC_ACQUIRE) != seq) throw Error(102, "result of a device kernel did not arrive");
 }
 template <int BLOCK>
 __global__ void export_segments_flag_kernel(ExportList L, unsigned *__restrict__ dst, unsigned *flag, unsigned seq)

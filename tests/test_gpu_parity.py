@@ -255,6 +255,17 @@ def test_m2l_sibling_parents_longest_first(eng, monkeypatch, name):
     assert np.array_equal(plain, plan.apply(dev(b)).cpu().numpy())
 
 
+def test_plan_with_stream_wait_instead_of_watching_pinned_memory(eng, oracle, monkeypatch):
+    """The host normally watches a sequence number in pinned memory for the per-level results; with the
+    spin limit at zero it takes the fallback, a stream wait.  Same plan either way."""
+    print("case spin limit 0", flush=True)
+    rng = np.random.default_rng(19)
+    X, Y, prm = clouds("clustered_xy", rng)
+    monkeypatch.setenv("F3M_SPIN_LIMIT_MS", "0")
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    assert_plan_matches_oracle(plan, oracle.Plan(X, Y, **prm))
+
+
 def test_near_field_longest_lists_first(eng, monkeypatch):
     """The matrix-pipe near field may take the boxes with the longest lists first (default from five
     dimensions on): the same sums for every target, bit for bit."""
