@@ -727,7 +727,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     const int *ord = nullptr;
     bool want_order = d >= 5;
     if (const char *e = getenv("F3M_NEAR_ORDER")) want_order = atoi(e) != 0;
-    if (use_mfma && want_order && items_exact >= 16384) {
+    if (use_mfma && want_order && items_exact >= 16384 && lx.nb <= 65536) {      // one workgroup places the boxes
         DBuf<int> cls((size_t)lx.nb), hist(256);
         orderbuf.reset((size_t)lx.nb);
         F3M_HIP(hipMemsetAsync(hist.get(), 0, 256 * sizeof(int), s));
