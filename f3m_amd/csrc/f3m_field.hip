@@ -693,13 +693,17 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 {
     if (list.n == 0) return;
     F3M_REQUIRE(nc == 1 || nc == 2 || nc == 4, 34, "near field takes 1, 2 or 4 columns at a time");
-    // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent accurate to about
-    // 2^-22 times the largest term, |x''|^2 <= 30 d (sc edge)^2 (listed targets lie within 5 edges per
-    // dimension of the anchor of their sources); it is used while that bound stays below 1e-4 (box edge up to
-    // ~2 lengthscales in 3-D), otherwise the all-vector kernel.
-    // F3M_NEAR=valu|mfma overrides the choice.
+    // The matrix-pipe kernel splits operands into f16 pairs, which keeps the exponent of a pair accurate to
+    // about 2^-22 times the products that enter it, (|x''| + |y'|)^2.  Sources lie within one edge per
+    // dimension of their anchor, |y'| <= S sqrt(d) with S = sc edge, and a target at scaled distance r of a
+    // source within r + S sqrt(d): a pair that matters (2^(-r^2) not negligible, r of order 1) has an
+    // exponent error of about 2^-22 4 S^2 d, and pairs with larger errors have targets several boxes away
+    // whose kernel values vanish against the others as S grows.  The kernel is used while 30 d S^2 <= 1200,
+    // i.e. a relative error of a term below 3e-5 (box edge up to ~3.6 lengthscales in 3-D; the N(0,I) cloud
+    // with ls = 0.1 has the same error against the fp64 product, 1.3968e-3, with either kernel at every
+    // level), otherwise the all-vector kernel.  F3M_NEAR=valu|mfma overrides the choice.
     const float sc_edge = sqrtf(lcs * kLog2e) * lx.edge;
-    bool use_mfma = 30.f * (float)d * sc_edge * sc_edge <= 400.f;
+    bool use_mfma = 30.f * (float)d * sc_edge * sc_edge <= 1200.f;
     if (const char *env = getenv("F3M_NEAR")) use_mfma = !strcmp(env, "mfma") ? true : (!strcmp(env, "valu") ? false : use_mfma);
     constexpr int T = 1;
     // all-vector kernel: whole boxes per workgroup where possible (multiple of the wave size, <= 512 lanes)
