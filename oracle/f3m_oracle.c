@@ -600,7 +600,7 @@ static inline float fo_rbf(int d, const float *x, const float *y, float lcs)
 /* exact block sums over a box-pair list sorted by bx (1_d_conv.cu:255-335): one accumulator per
  * target over the whole list of its box, then out += acc */
 static void fo_near(const fo_plan *P, const fo_level *L, const int *list, long nlist,
-                    const float *b, int c, float *out)
+                    const float *b, int c, float *out, const char *rowsel)
 {
     int d = P->d;
     long ngroups = 0;
@@ -612,6 +612,7 @@ static void fo_near(const fo_plan *P, const fo_level *L, const int *list, long n
         int bx = list[2 * gstart[g]];
         for (int ii = L->offx[bx]; ii < L->offx[bx + 1]; ii++) {
             int i = L->permx[ii];
+            if (rowsel && !rowsel[i]) continue;     /* rows that the caller did not ask for stay untouched */
             const float *xi = P->X + (long)i * d;
             for (int col = 0; col < c; col++) {
                 float acc = 0.f;
@@ -631,9 +632,13 @@ static void fo_near(const fo_plan *P, const fo_level *L, const int *list, long n
 
 /* far field of one level (n_tree.cu:489-593): P2M (1_d_conv.cu:451-552), M2L (:741-817),
  * L2P (:554-659).  Optional outputs mom/loc receive the moments of every Y box / local
- * expansions of every X box (zeros for boxes outside the far list). */
+ * expansions of every X box (zeros for boxes outside the far list).
+ * rowsel (nullable, one flag per row of X): the same sums restricted to the flagged target rows --
+ * M2L only for the X boxes that hold a flagged row, L2P only for flagged rows; everything else of
+ * out and loc stays zero/untouched.  (Sized for clouds whose complete M2L, far pairs x P^2 kernel
+ * evaluations, would take minutes on a CPU.) */
 static void fo_far(const fo_plan *P, const fo_level *L, const float *b, int c, float *out,
-                   float *mom_out, float *loc_out)
+                   float *mom_out, float *loc_out, const char *rowsel)
 {
     int d = P->d;
     int per_dim[FO_MAXD];
@@ -655,6 +660,12 @@ static void fo_far(const fo_plan *P, const fo_level *L, const float *b, int c, f
 
     char *uy = (char *)calloc(L->nby, 1), *ux = (char *)calloc(L->nbx, 1);
     for (long t = 0; t < L->nfar; t++) { ux[L->far[2 * t]] = 1; uy[L->far[2 * t + 1]] = 1; }
+    if (rowsel)
+        for (long bx = 0; bx < L->nbx; bx++) {
+            char any = 0;
+            for (int ii = L->offx[bx]; ii < L->offx[bx + 1] && !any; ii++) any = rowsel[L->permx[ii]];
+            if (!any) ux[bx] = 0;
+        }
     float *mom = (float *)calloc((size_t)L->nby * Pn * c, sizeof(float));
     float *loc = (float *)calloc((size_t)L->nbx * Pn * c, sizeof(float));
 
@@ -681,6 +692,7 @@ static void fo_far(const fo_plan *P, const fo_level *L, const float *b, int c, f
 #pragma omp parallel for schedule(dynamic, 4)
     for (long g = 0; g < ngroups; g++) {
         int bx = L->far[2 * gstart[g]];
+        if (!ux[bx]) continue;
         float xi[FO_MAXD], ym[FO_MAXD];
         for (int i = 0; i < Pn; i++) {
             for (int k = 0; k < d; k++) xi[k] = noff[i * d + k] + L->cx[(long)bx * d + k];  /* 1_d_conv.cu:776 */
@@ -704,6 +716,7 @@ static void fo_far(const fo_plan *P, const fo_level *L, const float *b, int c, f
         if (!ux[bx]) continue;
         for (int ii = L->offx[bx]; ii < L->offx[bx + 1]; ii++) {
             int i = L->permx[ii];
+            if (rowsel && !rowsel[i]) continue;
             fo_bprep bp;
             fo_basis_prepare(d, P->X + (long)i * d, L->cx + bx * d, factor, per_dim, nodes, w, &bp);
             for (int col = 0; col < c; col++) {
@@ -770,7 +783,7 @@ void fo_exact_f64(int d, const double *X, long N, const double *Y, long M, const
 }
 
 /* whole product from a plan (n_tree.cu:1075-1094 / 1099-1120) */
-int fo_plan_apply(const fo_plan *P, const float *b, int c, float *out)
+static int fo_apply_rows(const fo_plan *P, const float *b, int c, float *out, const char *rowsel)
 {
     if (P->status) return P->status;
     memset(out, 0, sizeof(float) * (size_t)P->N * c);
@@ -779,39 +792,56 @@ int fo_plan_apply(const fo_plan *P, const float *b, int c, float *out)
          * (n_tree.cu:1075,1092-1093); the defined behaviour chosen here is the exact product */
         float lcs = P->lcs;
 #pragma omp parallel for schedule(static)
-        for (long i = 0; i < P->N; i++)
+        for (long i = 0; i < P->N; i++) {
+            if (rowsel && !rowsel[i]) continue;
             for (int col = 0; col < c; col++) {
                 float acc = 0.f;
                 for (long j = 0; j < P->M; j++)
                     acc += fo_rbf(P->d, P->X + i * P->d, P->Y + j * P->d, lcs) * b[j * c + col];
                 out[i * c + col] = acc;
             }
+        }
         return 0;
     }
     for (int k = 0; k < P->nlevels; k++) {
         const fo_level *L = &P->lev[k];
-        if (L->nsmall > 0) fo_near(P, L, L->small_, L->nsmall, b, c, out);     /* n_tree.cu:1018-1020 */
-        if (L->nfar > 0) fo_far(P, L, b, c, out, NULL, NULL);                  /* n_tree.cu:1021-1051 */
+        if (L->nsmall > 0) fo_near(P, L, L->small_, L->nsmall, b, c, out, rowsel);     /* n_tree.cu:1018-1020 */
+        if (L->nfar > 0) fo_far(P, L, b, c, out, NULL, NULL, rowsel);                  /* n_tree.cu:1021-1051 */
     }
     const fo_level *L = &P->lev[P->nlevels - 1];
-    if (L->nkeep > 0) fo_near(P, L, L->keep, L->nkeep, b, c, out);             /* n_tree.cu:1092-1094 */
+    if (L->nkeep > 0) fo_near(P, L, L->keep, L->nkeep, b, c, out, rowsel);             /* n_tree.cu:1092-1094 */
     return 0;
+}
+int fo_plan_apply(const fo_plan *P, const float *b, int c, float *out) { return fo_apply_rows(P, b, c, out, NULL); }
+/* the same product for the target rows flagged in rowsel (N flags) only; the other rows of out are zero */
+int fo_plan_apply_rows(const fo_plan *P, const float *b, int c, float *out, const char *rowsel)
+{
+    return fo_apply_rows(P, b, c, out, rowsel);
 }
 
 /* single stages, exported so the GPU stages can be checked one by one */
-int fo_plan_far_level(const fo_plan *P, int k, const float *b, int c, float *out_accum, float *mom, float *loc)
+int fo_plan_far_level_rows(const fo_plan *P, int k, const float *b, int c, float *out_accum, float *mom, float *loc,
+                           const char *rowsel)
 {
     if (k < 0 || k >= P->nlevels) return 1;
-    fo_far(P, &P->lev[k], b, c, out_accum, mom, loc);
+    fo_far(P, &P->lev[k], b, c, out_accum, mom, loc, rowsel);
+    return 0;
+}
+int fo_plan_far_level(const fo_plan *P, int k, const float *b, int c, float *out_accum, float *mom, float *loc)
+{
+    return fo_plan_far_level_rows(P, k, b, c, out_accum, mom, loc, NULL);
+}
+int fo_plan_near_level_rows(const fo_plan *P, int k, int which, const float *b, int c, float *out_accum, const char *rowsel)
+{
+    if (k < 0 || k >= P->nlevels) return 1;
+    const fo_level *L = &P->lev[k];
+    if (which == 0) fo_near(P, L, L->small_, L->nsmall, b, c, out_accum, rowsel);
+    else fo_near(P, L, L->keep, L->nkeep, b, c, out_accum, rowsel);
     return 0;
 }
 int fo_plan_near_level(const fo_plan *P, int k, int which, const float *b, int c, float *out_accum)
 {
-    if (k < 0 || k >= P->nlevels) return 1;
-    const fo_level *L = &P->lev[k];
-    if (which == 0) fo_near(P, L, L->small_, L->nsmall, b, c, out_accum);
-    else fo_near(P, L, L->keep, L->nkeep, b, c, out_accum);
-    return 0;
+    return fo_plan_near_level_rows(P, k, which, b, c, out_accum, NULL);
 }
 
 /* M2L block between two boxes: K (P x P) with K[i][m] = exp(-|(n_i+cx)-(n_m+cy)|^2 lcs) */

@@ -57,6 +57,9 @@ def lib():
         L.fo_plan_apply.argtypes = [C.c_void_p, fp, C.c_int, fp]
         L.fo_plan_far_level.argtypes = [C.c_void_p, C.c_int, fp, C.c_int, fp, fp, fp]
         L.fo_plan_near_level.argtypes = [C.c_void_p, C.c_int, C.c_int, fp, C.c_int, fp]
+        L.fo_plan_apply_rows.argtypes = [C.c_void_p, fp, C.c_int, fp, C.c_char_p]
+        L.fo_plan_far_level_rows.argtypes = [C.c_void_p, C.c_int, fp, C.c_int, fp, fp, fp, C.c_char_p]
+        L.fo_plan_near_level_rows.argtypes = [C.c_void_p, C.c_int, C.c_int, fp, C.c_int, fp, C.c_char_p]
         L.fo_exact_f32.argtypes = [C.c_int, fp, C.c_long, fp, C.c_long, fp, C.c_int, C.c_float, fp]
         L.fo_exact_grad_f32.argtypes = [C.c_int, fp, C.c_long, fp, C.c_long, fp, C.c_int, C.c_float, fp]
         L.fo_exact_f64.argtypes = [C.c_int, dp, C.c_long, dp, C.c_long, dp, C.c_int, C.c_double, dp]
@@ -202,19 +205,30 @@ class Plan:
             "keep": grab("keep", (nkeep, 2), np.int32),
         }
 
-    def apply(self, b):
+    def _rowsel(self, rows):
+        """Flags (bytes, one per row of X) of the target rows in `rows`, or None for every row."""
+        if rows is None:
+            return None
+        sel = np.zeros(self.N, np.uint8)
+        sel[np.asarray(rows, np.int64)] = 1
+        return sel.tobytes()
+
+    def apply(self, b, rows=None):
+        """The product; with `rows` (indices into X) only those rows are computed, the others stay zero
+        (the same sums: M2L only for the boxes that hold a requested row)."""
         b = _f32(b)
         if b.ndim == 1:
             b = b[:, None]
         assert b.shape[0] == self.M
         out = np.zeros((self.N, b.shape[1]), np.float32)
-        rc = lib().fo_plan_apply(self._h, _fp(b), b.shape[1], _fp(out))
+        rc = lib().fo_plan_apply_rows(self._h, _fp(b), b.shape[1], _fp(out), self._rowsel(rows))
         if rc:
             raise RuntimeError("oracle apply failed")
         return out
 
-    def far_level(self, k, b):
-        """-> (out contribution, moments (nby,P,c), locals (nbx,P,c)) of level k's far field."""
+    def far_level(self, k, b, rows=None):
+        """-> (out contribution, moments (nby,P,c), locals (nbx,P,c)) of level k's far field; with `rows`
+        the local expansions of boxes without a requested row, and the other rows of out, stay zero."""
         b = _f32(b)
         if b.ndim == 1:
             b = b[:, None]
@@ -224,15 +238,16 @@ class Plan:
         out = np.zeros((self.N, c), np.float32)
         mom = np.zeros((lv["cy"].shape[0], P, c), np.float32)
         loc = np.zeros((lv["cx"].shape[0], P, c), np.float32)
-        lib().fo_plan_far_level(self._h, k, _fp(b), c, _fp(out), _fp(mom), _fp(loc))
+        lib().fo_plan_far_level_rows(self._h, k, _fp(b), c, _fp(out), _fp(mom), _fp(loc), self._rowsel(rows))
         return out, mom, loc
 
-    def near_level(self, k, which, b):
+    def near_level(self, k, which, b, rows=None):
         b = _f32(b)
         if b.ndim == 1:
             b = b[:, None]
         out = np.zeros((self.N, b.shape[1]), np.float32)
-        lib().fo_plan_near_level(self._h, k, 0 if which == "small" else 1, _fp(b), b.shape[1], _fp(out))
+        lib().fo_plan_near_level_rows(self._h, k, 0 if which == "small" else 1, _fp(b), b.shape[1], _fp(out),
+                                      self._rowsel(rows))
         return out
 
 

@@ -45,6 +45,17 @@ def cases():
     yield "d3_var_compression", rng.random((512, 3), dtype=f32), None, dict(base, ls=3.0, var_compression=True,
                                                                             eff_var_limit=0.3, min_points=30,
                                                                             small_field_points=12)
+    # Larger clouds whose box pairs hold at least 2 * nr_of_interpolation points, so that pairs two or more
+    # boxes apart are FAR (interpolated) instead of falling under the first "small" rule:
+    # the default 4 x 4 x 4 grid in 3-D, far pairs at depth 2;
+    yield "d3_uniform_64nodes_far", rng.random((8000, 3), dtype=f32), None, dict(base, ls=0.8, nr_of_interpolation=64,
+                                                                               min_points=200, small_field_points=80)
+    # the 3^5 grid in 5-D: the 32 boxes of depth 1, far across the diagonals of the hypercube;
+    yield "d5_uniform_243nodes_far", rng.random((8192, 5), dtype=f32), None, dict(base, ls=1.0, nr_of_interpolation=243,
+                                                                                min_points=1000, small_field_points=200)
+    # and a thin slab (two long dimensions), 16 boxes at depth 2 with far pairs up to three cells apart.
+    yield "d5_slab_243nodes_far", (rng.random((4800, 5)) * np.array([1, 1, .1, .1, .1])).astype(f32), None, \
+        dict(base, ls=0.7, nr_of_interpolation=243, min_points=500, small_field_points=200)
 
 
 def main():

@@ -5,7 +5,7 @@ product and no worse than 1.5x the oracle algorithm's own error)."""
 import numpy as np
 import pytest
 
-from parity_checks import assert_plan_matches_oracle, expected_list_rows, rel_l2
+from parity_checks import assert_plan_matches_oracle, canonical_box_of_point, expected_list_rows, rel_l2
 
 pytestmark = pytest.mark.gpu
 f32 = np.float32
@@ -40,9 +40,14 @@ def clouds(name, rng):
     if name == "uniform5":
         return rng.random((60000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=32, min_points=100,
                                                               small_field_points=40)
-    if name == "uniform5_243":       # config 4: 3^5 nodes per box
-        return rng.random((200000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=243, min_points=1000,
+    if name == "uniform5_243":       # config 4: 3^5 nodes per box; 390 points per box at depth 2, so pairs of boxes
+        # there hold more than 2 * 243 points and are far wherever they are two or more boxes apart
+        return rng.random((400000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=243, min_points=1000,
                                                                small_field_points=300)
+    if name in ("uniform3_ls0.1", "uniform3_ls10"):      # config 2 in miniature: lengthscales 0.1 and 10
+        return rng.random((100000, 3), dtype=f32), None, dict(ls=float(name.split("ls")[1]))
+    if name in ("normal3_ls0.1", "normal3_ls10"):
+        return rng.standard_normal((60000, 3)).astype(f32), None, dict(ls=float(name.split("ls")[1]))
     if name == "uniform5_1024":      # 4^5 nodes: the siblings of a box do not fit one workgroup and are split in two
         return rng.random((1500000, 5), dtype=f32), None, dict(ls=1.5, nr_of_interpolation=1024, min_points=1000,
                                                                 small_field_points=300)
@@ -59,8 +64,19 @@ def clouds(name, rng):
     raise KeyError(name)
 
 
-NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "uniform2", "uniform1", "lattice_faces_dups",
-         "uniform3_varcomp"]
+NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "uniform5_243", "uniform2", "uniform1",
+         "lattice_faces_dups", "uniform3_varcomp"]
+# Clouds whose complete far field would keep the CPU oracle busy for minutes (far pairs x 243^2 kernel
+# evaluations): the oracle computes the target rows of a few boxes only (same sums, restricted to those rows)
+# and the GPU results are compared on them.
+ROW_BOXES = {"uniform5_243": [0, 17, 333, 512, 800, 1023]}
+
+
+def selected_rows(name, level):
+    """rows of X that lie in the boxes ROW_BOXES[name] of the deepest level, or None for every row"""
+    if name not in ROW_BOXES:
+        return None
+    return np.concatenate([level["permx"][level["offx"][bx]:level["offx"][bx + 1]] for bx in ROW_BOXES[name]])
 
 
 @pytest.mark.parametrize("fixture_name", __import__("golden_fixtures").names())
@@ -93,6 +109,64 @@ def test_near_field_source_runs_on_matrix_pipe(eng, monkeypatch, fixture_name):
     X, Y, b, prm = gf.case(fx, fixture_name)
     plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
     gf.assert_product_matches_fixture(plan.apply(dev(b)).cpu().numpy(), fx, fixture_name)
+
+
+@pytest.mark.parametrize("fixture_name", __import__("golden_fixtures").names())
+def test_near_field_all_vector_kernel_on_fixtures(eng, monkeypatch, fixture_name):
+    """The all-vector near-field kernel (LDS-staged sources, fp32 throughout), which the library takes by
+    itself only where boxes are large against the lengthscale, forced on every fixture."""
+    import golden_fixtures as gf
+    print("case fixture (all-vector near field)", fixture_name, flush=True)
+    monkeypatch.setenv("F3M_NEAR", "valu")
+    fx = gf.load()
+    X, Y, b, prm = gf.case(fx, fixture_name)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    gf.assert_product_matches_fixture(plan.apply(dev(b)).cpu().numpy(), fx, fixture_name)
+
+
+@pytest.mark.parametrize("d,n,boxes", [(3, 40000, None), (5, 200000, [0, 100, 341, 682, 900, 1023])])
+@pytest.mark.parametrize("side", ["below", "above"])
+def test_near_field_kernel_switch_at_its_threshold(eng, oracle, monkeypatch, d, n, boxes, side):
+    """The library sums near pairs on the matrix pipe (split-f16 operands) while 30 d (sc edge)^2 <= 1200,
+    sc = sqrt(log2(e) / (2 ls^2)), and with the all-vector kernel beyond.  Lengthscales that put the boxes of
+    the deepest level 1 % below and 1 % above that switch: the matrix-pipe kernel must stay within 3e-5 of
+    the oracle's sums (the bound the switch is derived from) below it, the all-vector kernel within 1e-5 on
+    both sides, and the library's own choice must be the matrix pipe below and the all-vector kernel above."""
+    print("case near switch d=%d %s" % (d, side), flush=True)
+    rng = np.random.default_rng(21)
+    X = rng.random((n, d), dtype=f32)
+    b = rng.standard_normal((n, 2)).astype(f32)
+    prm = dict(min_points=1000, nr_of_interpolation=64 if d == 3 else 32)
+    probe = eng.Plan(dev(X), None, ls=1.0, **prm)                       # the box edge does not depend on ls
+    depth = probe.depth
+    edge = float(probe.level_sizes(depth)["edge"])
+    probe.close()
+    s_edge = np.sqrt(1200.0 / (30.0 * d)) * (0.99 if side == "below" else 1.01)      # sc * edge aimed at
+    ls = float(np.sqrt(np.log2(np.e) / 2.0) * edge / s_edge)
+    plan = eng.Plan(dev(X), None, ls=ls, **prm)
+    ora = oracle.Plan(X, None, ls=ls, **prm)
+    assert plan.depth == depth and ora.nlevels == depth
+    sc_edge = np.sqrt(float(ora.lcs) * np.log2(np.e)) * edge
+    assert (30 * d * sc_edge ** 2 <= 1200) == (side == "below")
+    L = ora.level(depth - 1)
+    which = "small" if len(L["small"]) else "keep"
+    rows = None if boxes is None else np.concatenate([L["permx"][L["offx"][bx]:L["offx"][bx + 1]] for bx in boxes])
+    sel = slice(None) if rows is None else rows
+    want = ora.near_level(depth - 1, which, b, rows=rows)[sel]
+    assert np.abs(want).max() > 0
+    auto = plan.near_level(depth, which, dev(b)).cpu().numpy()[sel]
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    mfma = plan.near_level(depth, which, dev(b)).cpu().numpy()[sel]
+    monkeypatch.setenv("F3M_NEAR", "valu")
+    valu = plan.near_level(depth, which, dev(b)).cpu().numpy()[sel]
+    e_mfma, e_valu = rel_l2(mfma, want), rel_l2(valu, want)
+    print("sc*edge %.4f  rel-L2 vs oracle: matrix pipe %.3e, all-vector %.3e" % (sc_edge, e_mfma, e_valu), flush=True)
+    assert e_valu < 1e-5
+    if side == "below":
+        assert e_mfma < 3e-5
+        assert np.array_equal(auto, mfma)
+    else:
+        assert np.array_equal(auto, valu)
 
 
 @pytest.mark.parametrize("name", NAMES)
@@ -154,40 +228,59 @@ def test_exact_kernels(eng, oracle, d):
     assert rel_l2(eng.exact_grad_f32(dev(X), dev(Y), dev(b), ls).cpu().numpy(), oracle.exact_grad_f32(X, Y, b, ls)) < 1e-5
 
 
-@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform5_243",
+                                  "uniform3_varcomp"])
 def test_stages_against_oracle(eng, oracle, name):
     print("case stages", name, flush=True)
     rng = np.random.default_rng(7)
     X, Y, prm = clouds(name, rng)
-    X = X[:30000]
-    Y = None if Y is None else Y[:12000]
+    if name not in ("uniform5", "uniform5_243"):          # the 5-D clouds need their points to have far pairs
+        X = X[:30000]
+        Y = None if Y is None else Y[:12000]
     M = X.shape[0] if Y is None else Y.shape[0]
     b = rng.standard_normal((M, 2)).astype(f32)
     plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
     ora = oracle.Plan(X, Y, **prm)
     assert_plan_matches_oracle(plan, ora)
-    did_far = False
+    rows = selected_rows(name, ora.level(ora.nlevels - 1))
+    sel = slice(None) if rows is None else rows
+    far_levels = 0
     for k in range(1, plan.depth + 1):
         sz = plan.level_sizes(k)
         if sz["nsmall"]:
             got = plan.near_level(k, "small", dev(b)).cpu().numpy()
-            assert rel_l2(got, ora.near_level(k - 1, "small", b)) < 1e-5          # fp32 summation order only
+            assert rel_l2(got[sel], ora.near_level(k - 1, "small", b, rows=rows)[sel]) < 1e-5   # fp32 summation order only
         if sz["nfar"]:
-            did_far = True
+            far_levels += 1
             out, mom, loc = plan.far_level(k, dev(b), want_expansions=True)
-            o_out, o_mom, o_loc = ora.far_level(k - 1, b)
+            o_out, o_mom, o_loc = ora.far_level(k - 1, b, rows=rows)
+            loc = loc.cpu().numpy()
+            o_loc = np.moveaxis(o_loc, 2, 0)
+            if rows is not None:                         # local expansions of the boxes that hold a selected row
+                L = ora.level(k - 1)
+                boxes = np.unique(canonical_box_of_point(L, "x")[rows])
+                assert np.abs(o_loc[:, boxes]).max() > 0
+                loc, o_loc = loc[:, boxes], o_loc[:, boxes]
             assert rel_l2(mom.cpu().numpy(), np.moveaxis(o_mom, 2, 0)) < 1e-4     # P2M
-            assert rel_l2(loc.cpu().numpy(), np.moveaxis(o_loc, 2, 0)) < 1e-4     # M2L
-            assert rel_l2(out.cpu().numpy(), o_out) < 1e-4                        # L2P
-    assert did_far or name == "uniform5"
+            assert rel_l2(loc, o_loc) < 1e-4                                      # M2L
+            assert rel_l2(out.cpu().numpy()[sel], o_out[sel]) < 1e-4              # L2P
+    assert far_levels >= (2 if name == "uniform5_243" else 1)
     if plan.level_sizes(plan.depth)["nkeep"]:
         got = plan.near_level(plan.depth, "keep", dev(b)).cpu().numpy()
-        assert rel_l2(got, ora.near_level(plan.depth - 1, "keep", b)) < 1e-5
+        assert rel_l2(got[sel], ora.near_level(plan.depth - 1, "keep", b, rows=rows)[sel]) < 1e-5
     got = plan.apply(dev(b)).cpu().numpy()
-    assert rel_l2(got, ora.apply(b)) < 1e-5
+    assert rel_l2(got[sel], ora.apply(b, rows=rows)[sel]) < 1e-5
 
 
-@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform4"])
+PRODUCT_NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5_243", "uniform3_ls0.1", "uniform3_ls10",
+                 "normal3_ls0.1", "normal3_ls10"]
+# Where the reference algorithm itself (the oracle, same nodes and lengthscale) misses the 1e-3 of the
+# north star, the engine cannot meet it either; these are the clouds where that is expected, with the
+# oracle's error as measured (the engine must still stay within 1.5x of it).
+ORACLE_ABOVE_1E3 = {"uniform3_ls0.1"}
+
+
+@pytest.mark.parametrize("name", PRODUCT_NAMES)
 def test_product_error_vs_fp64_exact(eng, oracle, name):
     print("case product", name, flush=True)
     rng = np.random.default_rng(9)
@@ -198,12 +291,19 @@ def test_product_error_vs_fp64_exact(eng, oracle, name):
     got = eng.kmvm(Xd, Yd, bd, **prm).cpu().numpy()
     Ys = X if Y is None else Y
     exact = eng.exact_f64(dev(X.astype(np.float64)), dev(Ys.astype(np.float64)), dev(b.astype(np.float64)), prm["ls"]).cpu().numpy()
+    ora = oracle.Plan(X, Y, **prm)
+    rows = selected_rows(name, ora.level(ora.nlevels - 1))
+    sel = slice(None) if rows is None else rows
     err = rel_l2(got, exact)
-    err_oracle = rel_l2(oracle.kmvm(X, Y, b, **prm), exact)
-    print("rel-L2 engine %.3e oracle %.3e" % (err, err_oracle), flush=True)
-    assert err <= 1.5 * err_oracle + 1e-7                # no worse than 1.5x the reference algorithm
-    # north-star tolerance, wherever the reference algorithm itself reaches it at these parameters
-    assert err <= 1e-3 or err_oracle > 1e-3 / 1.5, (err, err_oracle)
+    err_sel = rel_l2(got[sel], exact[sel])
+    err_oracle = rel_l2(ora.apply(b, rows=rows)[sel], exact[sel])
+    print("rel-L2 engine %.3e (compared rows %.3e) oracle %.3e" % (err, err_sel, err_oracle), flush=True)
+    assert err_sel <= 1.5 * err_oracle + 1e-7            # no worse than 1.5x the reference algorithm
+    # north-star tolerance 1e-3 against the fp64 product, on every row
+    if name in ORACLE_ABOVE_1E3:
+        assert err_oracle > 1e-3 / 1.5 and err <= 1.5 * err_oracle, (err, err_oracle)
+    else:
+        assert err <= 1e-3, (err, err_oracle)
 
 
 @pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform5_1024", "uniform3_varcomp"])
