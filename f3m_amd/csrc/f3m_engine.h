@@ -36,6 +36,10 @@ struct TreeLevel {
     mutable DBuf<int> box32;
     mutable DBuf<uint32_t> hashtab;      // hashcap pairs (key, value), empty = 0xffffffff
     mutable uint32_t hashcap = 0;
+    // work items of P2M and of the general L2P over every box of this level (chunk offsets per box,
+    // built on first use): they depend on the tree only
+    mutable DBuf<int> p2m_tiles, l2p_tiles;
+    mutable int p2m_bound = -1, l2p_bound = -1;
 };
 
 struct Tree {
@@ -46,6 +50,13 @@ struct Tree {
     int sorted_from = 0;
     DBuf<int> perm;      // sorted position -> original row
     std::vector<TreeLevel> lev;   // lev[0] is the root
+};
+
+// work items of the near field over one list: offsets of the target tiles per x box (in the order
+// `order`, if any), and the launch bound that goes with them
+struct TileTable {
+    DBuf<int> tileoff, order;
+    int bound = 0;
 };
 
 struct PairList {
@@ -59,6 +70,12 @@ struct PairList {
     // x boxes with a non-empty row, their points, and the work items they make when cut into pieces of
     // 128 and of 160 targets (near-field launch shapes); rows = -1: not counted
     long long rows = -1, row_points = 0, items128 = 0, items160 = 0;
+    // Tables that depend on the plan only, built on first use and kept: near-field tile tables by
+    // (targets per work item) * 2 + (longest lists first); for far lists the separable M2L tables of the
+    // level and the order of the parents for the sibling-group kernel.
+    mutable std::map<int, TileTable> near_tiles;
+    mutable DBuf<float> m2l_tab;
+    mutable DBuf<int> m2l_order;
 };
 
 struct ClassifyParams {

@@ -236,6 +236,7 @@ static const int *box_table(const TreeLevel &lev, long long npoints, hipStream_t
 {
     const int nent = (int)(npoints / 32) + 2;
     if (lev.box32.size() != (size_t)nent) {
+        require_tables_may_be_built("the box table of a level");
         lev.box32.reset((size_t)nent);
         F3M_LAUNCH(box_table_kernel, cdiv(nent, 256), 256, 0, s, lev.off.get(), lev.nb, npoints, nent, lev.box32.get());
         check_launch("box_table");
@@ -245,10 +246,13 @@ static const int *box_table(const TreeLevel &lev, long long npoints, hipStream_t
 
 // ------------------------------------------------------------------------------------------------
 // near field (F3M_src/1_d_conv.cu:255-335): out_i += sum over the y boxes listed for the box of i of
-// sum_j exp(-|x_i-y_j|^2 lcs) b_j.  One workgroup per (x box, tile of targets); the sources of a y
-// box are staged through LDS already shifted to the x box centre and scaled by sqrt(lcs*log2 e), in
-// the form (2y', -|y'|^2, b), so that a pair costs D fused multiply-adds, one add, one exp2 and one
-// fused multiply-add:  exp2(2x'.y' - |y'|^2 - |x'|^2) b.
+// sum_j exp(-|x_i-y_j|^2 lcs) b_j.  All-vector form: one workgroup per (x box, tile of targets); the
+// sources of a y box are staged through LDS already shifted to the x box centre and scaled by
+// sqrt(lcs*log2 e), together with their weights, and a pair costs D subtractions, D multiply-adds, one
+// exp2 and one multiply-add:  exp2(-|x' - y'|^2) b.  The exponent is formed from the coordinate
+// differences (not from 2x'.y' - |y'|^2 - |x'|^2, whose cancellation costs about 2^-24 (|x'|^2 + |y'|^2)):
+// this is the kernel for boxes that are large against the lengthscale, where those squares reach
+// hundreds.
 
 constexpr int kNearCap = 512;   // sources per LDS tile
 
@@ -260,9 +264,8 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
                                                     const int *__restrict__ rowptr, const int *__restrict__ tileoff,
                                                     int nbx, float sc)
 {
-    constexpr int NV = (D + 1 + 3) / 4;
+    constexpr int NV = (D + 1 + 3) / 4;             // float4 slots per source: D coordinates and the weight
     __shared__ float4 sv[NV][kNearCap];
-    __shared__ float sb[kNearCap];
     const int tid = threadIdx.x, BD = blockDim.x;
     if ((int)blockIdx.x >= tileoff[nbx]) return;    // launched with an upper bound of the tile count
     const int bx = find_box(tileoff, nbx, blockIdx.x);
@@ -271,17 +274,15 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
     float cx[D];
 #pragma unroll
     for (int k = 0; k < D; k++) cx[k] = ctrx[(long long)bx * D + k];
-    float x[T][D], nx2[T], acc[T];
+    float x[T][D], acc[T];
 #pragma unroll
     for (int r = 0; r < T; r++) {
         int i = x0 + r * BD + tid;
-        nx2[r] = 0.f;
         acc[r] = 0.f;
 #pragma unroll
         for (int k = 0; k < D; k++) {
             float v = (i < x1) ? xs[(long long)k * N + i] : cx[k];
             x[r][k] = sc * (v - cx[k]);
-            nx2[r] -= x[r][k] * x[r][k];
         }
     }
     // a wavefront whose lanes all lie past the end of the box only helps with staging
@@ -295,19 +296,13 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
             __syncthreads();
             for (int jj = tid; jj < cnt; jj += BD) {
                 float v[NV * 4];
-                float ny2 = 0.f;
 #pragma unroll
-                for (int k = 0; k < D; k++) {
-                    float y = sc * (ys[(long long)k * M + base + jj] - cx[k]);
-                    v[k] = 2.f * y;
-                    ny2 -= y * y;
-                }
-                v[D] = ny2;
+                for (int k = 0; k < D; k++) v[k] = sc * (ys[(long long)k * M + base + jj] - cx[k]);
+                v[D] = bs[base + jj];
 #pragma unroll
                 for (int k = D + 1; k < NV * 4; k++) v[k] = 0.f;
 #pragma unroll
                 for (int q = 0; q < NV; q++) sv[q][jj] = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
-                sb[jj] = bs[base + jj];
             }
             __syncthreads();
             if (!wave_live) continue;
@@ -319,14 +314,12 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
                     float4 f = sv[q][jj];
                     v[4 * q] = f.x; v[4 * q + 1] = f.y; v[4 * q + 2] = f.z; v[4 * q + 3] = f.w;
                 }
-                const float bj = sb[jj];
 #pragma unroll
                 for (int r = 0; r < T; r++) {
-                    float t = v[D];
+                    float r2 = 0.f;
 #pragma unroll
-                    for (int k = 0; k < D; k++) t = fmaf(x[r][k], v[k], t);
-                    t += nx2[r];
-                    acc[r] = fmaf(fast_exp2(t), bj, acc[r]);
+                    for (int k = 0; k < D; k++) { const float df = x[r][k] - v[k]; r2 = fmaf(df, df, r2); }
+                    acc[r] = fmaf(fast_exp2(-r2), v[D], acc[r]);
                 }
             }
         }
@@ -710,9 +703,6 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     int bd = ((lx.maxcount + kWave - 1) / kWave) * kWave;
     if (bd > 512) bd = 256;
     if (bd < kWave) bd = kWave;
-    DBuf<int> flag((size_t)lx.nb), tileoff;
-    F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
-    check_launch("mark_rows");
     // target tiles of 32 per wavefront: 4 (2: 10.2 ms, 4: 9.2 ms, 5: 10.2 ms, 8: 9.4 ms at N=1e7, d=3, ten tiles
     // per box), but 5 where a typical box has five tiles and would otherwise be cut into 4 + 1
     // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms at the time)
@@ -727,22 +717,33 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
     // the time of the ordering itself: 11.7 -> 11.8 ms, 10.5 -> 10.8 ms per product).  Lists that are not
     // sliced only.  F3M_NEAR_ORDER=0|1 overrides.
-    DBuf<int> orderbuf;
-    const int *ord = nullptr;
     bool want_order = d >= 5;
     if (const char *e = getenv("F3M_NEAR_ORDER")) want_order = atoi(e) != 0;
-    if (use_mfma && want_order && items_exact >= 16384 && lx.nb <= 65536) {      // one workgroup places the boxes
-        DBuf<int> cls((size_t)lx.nb), hist(256);
-        orderbuf.reset((size_t)lx.nb);
-        F3M_HIP(hipMemsetAsync(hist.get(), 0, 256 * sizeof(int), s));
-        const int unit = (int)std::max<long long>(1, list.n / std::max<long long>(1, list.rows) / 64);   // mean row = class 64
-        F3M_LAUNCH(row_class_count_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, unit, cls.get(), hist.get());
-        check_launch("row_class_count");
-        F3M_LAUNCH(class_place_kernel, 1, 1024, 0, s, cls.get(), lx.nb, hist.get(), orderbuf.get());
-        check_launch("class_place");
-        ord = orderbuf.get();
+    const bool ordered = use_mfma && want_order && items_exact >= 16384 && lx.nb <= 65536;   // one workgroup places the boxes
+    // The tile table of this list (offsets of the work items per box, in launch order) depends on the plan
+    // only and is kept with the list.
+    const int tilesize = use_mfma ? tpw * 32 : bd * T;
+    TileTable &tt = list.near_tiles[tilesize * 2 + (ordered ? 1 : 0)];
+    if (tt.tileoff.size() == 0) {
+        require_tables_may_be_built("the near-field tile table of a list");
+        DBuf<int> flag((size_t)lx.nb);
+        F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());
+        check_launch("mark_rows");
+        if (ordered) {
+            DBuf<int> cls((size_t)lx.nb), hist(256);
+            tt.order.reset((size_t)lx.nb);
+            dev_fill(hist.get(), 0, 256 * sizeof(int), s);
+            const int unit = (int)std::max<long long>(1, list.n / std::max<long long>(1, list.rows) / 64);   // mean row = class 64
+            F3M_LAUNCH(row_class_count_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, unit, cls.get(), hist.get());
+            check_launch("row_class_count");
+            F3M_LAUNCH(class_place_kernel, 1, 1024, 0, s, cls.get(), lx.nb, hist.get(), tt.order.get());
+            check_launch("class_place");
+        }
+        tt.bound = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, tilesize, tt.tileoff, s, ordered ? tt.order.get() : nullptr);
     }
-    int ntiles = build_tiles(lx.off.get(), flag.get(), lx.nb, tx.n, use_mfma ? tpw * 32 : bd * T, tileoff, s, ord);
+    const int *ord = ordered ? tt.order.get() : nullptr;
+    const DBuf<int> &tileoff = tt.tileoff;
+    int ntiles = tt.bound;
     if (use_mfma && items_exact >= 0) ntiles = (int)std::max<long long>(1, items_exact);
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
@@ -751,13 +752,14 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         // The operands of a level are kept in the plan.  only_list: this list is the only near list of
         // its level, so operands are needed for its source boxes only (at most levels a small part).
         if (ly.nearops.size() == 0 || ly.nearops_sc != sc || (ly.nearops_partial && !only_list)) {
+            require_tables_may_be_built("the near-field source operands of a level");
             ly.nearops.reset((size_t)NS * 2 * stride * 16);
             ly.nearops_sc = sc;
             ly.nearops_partial = only_list;
             DBuf<int> need;
             if (only_list) {
                 DBuf<int> fy((size_t)ly.nb);
-                F3M_HIP(hipMemsetAsync(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s));
+                dev_fill(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s);
                 F3M_LAUNCH(mark_cols_kernel, cdiv(list.n, 256), 256, 0, s, list.pairs.get(), list.n, fy.get());
                 check_launch("mark_cols");
                 need.reset((size_t)ly.nb + 1);
@@ -1871,7 +1873,7 @@ void mark_far_boxes(const PairList &far, int nbx, int nby, int *fx, int *fy, hip
     // participating boxes: x boxes with a non-empty far row, y boxes that occur in the far list
     F3M_LAUNCH(mark_rows_kernel, cdiv(nbx, 256), 256, 0, s, far.rowptr.get(), nbx, fx);
     check_launch("mark_rows");
-    F3M_HIP(hipMemsetAsync(fy, 0, sizeof(int) * (size_t)nby, s));
+    dev_fill(fy, 0, sizeof(int) * (size_t)nby, s);
     if (far.n > 0) {
         F3M_LAUNCH(mark_cols_kernel, cdiv(far.n, 256), 256, 0, s, far.pairs.get(), far.n, fy);
         check_launch("mark_cols");
@@ -1890,8 +1892,19 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
     const int P = ns.P;
     NodeMeta nm = meta_of(ns);
     const float factor = 2 / ly.edge;                  // F3M_src/1_d_conv.cu:473
-    DBuf<int> tiley;
-    int nty = build_tiles(ly.off.get(), flag, ly.nb, ty.n, kP2MChunk, tiley, s);
+    // chunks of every box: kept with the level (they depend on the tree only); chunks of flagged boxes: per call
+    DBuf<int> tiles_flagged;
+    int nty;
+    if (flag == nullptr) {
+        if (ly.p2m_bound < 0) {
+            require_tables_may_be_built("the chunk table of a level");
+            ly.p2m_bound = build_tiles(ly.off.get(), nullptr, ly.nb, ty.n, kP2MChunk, ly.p2m_tiles, s);
+        }
+        nty = ly.p2m_bound;
+    } else {
+        nty = build_tiles(ly.off.get(), flag, ly.nb, ty.n, kP2MChunk, tiles_flagged, s);
+    }
+    const DBuf<int> &tiley = flag == nullptr ? ly.p2m_tiles : tiles_flagged;
     DBuf<float> partial((size_t)std::max(1, nty) * P);
     int bdp = ((P + kWave - 1) / kWave) * kWave;
     size_t shp = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)kP2MSub * ns.S1);
@@ -1938,7 +1951,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
     const int P = ns.P;
     NodeMeta nm = meta_of(ns);
     int bdp = ((P + kWave - 1) / kWave) * kWave;
-    F3M_HIP(hipMemsetAsync(loc, 0, sizeof(float) * (size_t)lx.nb * P, s));
+    dev_fill(loc, 0, sizeof(float) * (size_t)lx.nb * P, s);
     if (far.n == 0) return;
     int NT = 1;
     for (int j = 0; j < d; j++) NT = std::max(NT, ns.n[j]);
@@ -1957,10 +1970,15 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             sg.delta[j] = (double)ty.geo.origin[j] - (double)tx.geo.origin[j];
             sm.omin[j] = sg.omin[j] = (int)std::floor(-5.0 - sg.delta[j] / edge) - 1;
         }
-        DBuf<float> dtab((size_t)ntab);
-        F3M_LAUNCH(sep_tables_kernel, cdiv(ntab, 256), 256, 0, s, nm, d, NT, kM2LOffsets, ns.dt.get(), edge, (double)lcs, sg,
-                   dtab.get());
-        check_launch("sep_tables");
+        // the tables of the level depend on the plan only (nodes, edge, lengthscale, origins) and are kept with its far list
+        DBuf<float> &dtab = far.m2l_tab;
+        if (dtab.size() != (size_t)ntab) {
+            require_tables_may_be_built("the M2L tables of a level");
+            dtab.reset((size_t)ntab);
+            F3M_LAUNCH(sep_tables_kernel, cdiv(ntab, 256), 256, 0, s, nm, d, NT, kM2LOffsets, ns.dt.get(), edge, (double)lcs, sg,
+                       dtab.get());
+            check_launch("sep_tables");
+        }
         size_t shs = sizeof(float) * ((size_t)ntab + 2 * (size_t)P);
         timer_begin(kM2L, s);
         const bool q64 = d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4 && m2l_mode != 2;
@@ -2008,11 +2026,12 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             // workgroup).  F3M_SIB_ORDER=0|1 overrides.
             bool ordered = d >= 4 && par.nb <= 16384;
             if (const char *e = getenv("F3M_SIB_ORDER")) ordered = atoi(e) != 0;
-            DBuf<int> sibOrder;
-            if (ordered) {
+            DBuf<int> &sibOrder = far.m2l_order;
+            if (ordered && sibOrder.size() != (size_t)par.nb) {
+                require_tables_may_be_built("the M2L parent order of a level");
                 DBuf<int> cls((size_t)par.nb), hist(256);
                 sibOrder.reset((size_t)par.nb);
-                F3M_HIP(hipMemsetAsync(hist.get(), 0, 256 * sizeof(int), s));
+                dev_fill(hist.get(), 0, 256 * sizeof(int), s);
                 const int unit = (int)std::max<long long>(1, far.n / std::max(1, par.nb) / 64);    // mean row = class 64
                 F3M_LAUNCH(sib_class_count_kernel, cdiv(par.nb, 256), 256, 0, s, par.childstart.get(), far.rowptr.get(), par.nb,
                            unit, cls.get(), hist.get());
@@ -2227,8 +2246,18 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
         check_launch("l2p_tensor");
         return;
     }
-    DBuf<int> tilex;
-    int ntx = build_tiles(lx.off.get(), flag, lx.nb, tx.n, kL2PBlock, tilex, s);
+    DBuf<int> tiles_flagged;
+    int ntx;
+    if (flag == nullptr) {
+        if (lx.l2p_bound < 0) {
+            require_tables_may_be_built("the chunk table of a level");
+            lx.l2p_bound = build_tiles(lx.off.get(), nullptr, lx.nb, tx.n, kL2PBlock, lx.l2p_tiles, s);
+        }
+        ntx = lx.l2p_bound;
+    } else {
+        ntx = build_tiles(lx.off.get(), flag, lx.nb, tx.n, kL2PBlock, tiles_flagged, s);
+    }
+    const DBuf<int> &tilex = flag == nullptr ? lx.l2p_tiles : tiles_flagged;
     size_t shl = sizeof(float) * (2 * (size_t)ns.S1 + (size_t)P + (size_t)kL2PBlock * (ns.S1 | 1));
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \

@@ -661,7 +661,7 @@ void lookup_boxes(const Tree &t, const TreeLevel &lev, const int *cells, long lo
         uint32_t cap = 1024;
         while (cap < 2u * (uint32_t)lev.nb) cap <<= 1;
         lev.hashtab.reset(2 * (size_t)cap);
-        F3M_HIP(hipMemsetAsync(lev.hashtab.get(), 0xff, sizeof(uint32_t) * 2 * (size_t)cap, s));
+        dev_fill(lev.hashtab.get(), 0xff, sizeof(uint32_t) * 2 * (size_t)cap, s);
         F3M_LAUNCH(hash_insert_kernel, cdiv(lev.nb, 256), 256, 0, s, lev.cell.get(), lev.nb, d, lev.depth, lev.hashtab.get(),
                    cap);
         check_launch("hash_insert");

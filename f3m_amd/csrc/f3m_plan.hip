@@ -98,6 +98,7 @@ struct f3m_plan {
         auto key = std::make_pair(nodes_parent, nodes_child);
         auto it = shift_tabs.find(key);
         if (it == shift_tabs.end()) {
+            require_tables_may_be_built("a table that moves expansions between levels");
             std::unique_ptr<DBuf<float>> t(new DBuf<float>());
             make_shift_tables(nodeset(nodes_parent, s), nodeset(nodes_child, s), *t, s);
             it = shift_tabs.emplace(key, std::move(t)).first;
@@ -108,6 +109,7 @@ struct f3m_plan {
     {
         auto it = nodes.find(num_nodes);
         if (it == nodes.end()) {
+            require_tables_may_be_built("a node set");
             std::unique_ptr<NodeSet> ns(new NodeSet());
             make_nodes(*ns, d, num_nodes, s);
             it = nodes.emplace(num_nodes, std::move(ns)).first;
@@ -218,7 +220,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     PairList root;
     root.n = 1;
     root.pairs.reset(2);
-    F3M_HIP(hipMemsetAsync(root.pairs.get(), 0, 2 * sizeof(int), s));     // the root pair (0,0)
+    dev_fill(root.pairs.get(), 0, 2 * sizeof(int), s);     // the root pair (0,0)
     build_rowptr(root, 1, s);
     const PairList *keep = &root;
     P->levels.reserve(64);   // `keep` points into this vector: it must not reallocate
@@ -232,7 +234,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // [10,11] of the Y tree's.  On the device the first three are the last entries of the list builder's
     // scans; the counters behind [6..11] live in dres and are cleared by the readback that fetches them.
     DBuf<int> dres(16);
-    F3M_HIP(hipMemsetAsync(dres.get(), 0, 16 * sizeof(int), s));
+    dev_fill(dres.get(), 0, 16 * sizeof(int), s);
     alignas(8) int hres[16];
     auto fetch_level = [&](const ListsPending *pend, bool division) {
         memset(hres, 0, sizeof(hres));
@@ -248,7 +250,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // them, so they are fetched once at the end instead of with the per-level wait
     constexpr int kMaxLevels = 40;
     DBuf<long long> drow((size_t)8 * kMaxLevels);
-    F3M_HIP(hipMemsetAsync(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s));
+    dev_fill(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s);
     auto wants_division = [&]() {
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
@@ -399,6 +401,18 @@ static void far_tree(f3m_plan *P, const float *bs, float *outs, hipStream_t s)
     l2p_level(d, P->tx, P->tx.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s);
 }
 
+// waits for the stream, except while it is being captured into a graph (where a wait is an error and
+// the work has not run anyway)
+static void finish_stream(hipStream_t s)
+{
+#ifndef F3M_CPU_EMU
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) return;
+    (void)hipGetLastError();
+#endif
+    F3M_HIP(hipStreamSynchronize(s));
+}
+
 static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s)
 {
     F3M_REQUIRE(P != nullptr, 1, "plan is NULL");
@@ -409,7 +423,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         const float *Yp = P->symmetric ? P->Xraw.get() : P->Yraw.get();
         Scope sc(kNear, s);
         exact_f32(P->d, P->Xraw.get(), P->N, Yp, P->M, b, c, P->prm.ls, false, out, s);
-        F3M_HIP(hipStreamSynchronize(s));
+        finish_stream(s);
         return;
     }
     // Columns are taken four at a time while at least three are left (the near field then computes every
@@ -428,9 +442,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
-            if (nc > ncol) F3M_HIP(hipMemsetAsync(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s));
+            if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
             for (int q = 0; q < ncol; q++) gather_column(b, P->ty->perm.get(), P->M, c, col + q, bs.get() + q * bstride, s);
-            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s));
+            dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
         }
         for (int k = 1; k <= depth; k++) {
             PlanLevel &L = P->levels[k - 1];
@@ -452,7 +466,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         }
         col += ncol;
     }
-    F3M_HIP(hipStreamSynchronize(s));
+    finish_stream(s);
 }
 
 template <typename F>
@@ -632,7 +646,7 @@ int f3m_plan_far_level(f3m_plan *plan, int level, const float *b, int c, float *
         int P = L.far.n ? plan->nodeset(L.num_nodes, s).P : 0;
         for (int col = 0; col < c; col++) {
             gather_column(b, plan->ty->perm.get(), plan->M, c, col, bs.get(), s);
-            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)plan->N, s));
+            dev_fill(outs.get(), 0, sizeof(float) * (size_t)plan->N, s);
             far_level(plan, level, bs.get(), outs.get(),
                       mom ? mom + (size_t)col * plan->ty->lev[level].nb * P : nullptr,
                       loc ? loc + (size_t)col * plan->tx.lev[level].nb * P : nullptr, s);
@@ -653,7 +667,7 @@ int f3m_plan_near_level(f3m_plan *plan, int level, int which, const float *b, in
         PlanLevel &L = plan->levels[level - 1];
         for (int col = 0; col < c; col++) {
             gather_column(b, plan->ty->perm.get(), plan->M, c, col, bs.get(), s);
-            F3M_HIP(hipMemsetAsync(outs.get(), 0, sizeof(float) * (size_t)plan->N, s));
+            dev_fill(outs.get(), 0, sizeof(float) * (size_t)plan->N, s);
             near_field(plan->d, plan->tx, plan->tx.lev[level], *plan->ty, plan->ty->lev[level],
                        which == F3M_LIST_SMALL ? L.small_ : L.keep, bs.get(), outs.get(), plan->lcs, s);
             scatter_column(outs.get(), plan->tx.perm.get(), plan->N, c, col, out, s);

@@ -13,6 +13,7 @@
 #define F3M_DYN_SHARED(type, name) extern __shared__ __align__(16) unsigned char name##_raw[]; type *name = reinterpret_cast<type *>(name##_raw)
 #endif
 
+#include <algorithm>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -63,6 +64,32 @@ inline std::string fmt(const char *f, ...)
 // calls make no hipMalloc.  All work of one call runs on one stream and every C-ABI entry point
 // synchronises that stream before it returns, so a released block is idle when it is handed out
 // again.
+//
+// While the calling thread has an Arena installed (ArenaScope), every request is carved out of that
+// fixed block of device memory instead, in order, and nothing is given back until the scope ends:
+// a call that must not allocate takes its temporaries from there.  Tables that outlive the call
+// (kept in a plan) cannot come from an arena; code that is about to build one calls
+// require_tables_may_be_built() first.
+struct Arena {
+    char *base = nullptr;
+    size_t cap = 0, used = 0;
+    const char *owner = "";
+};
+inline thread_local Arena *g_arena = nullptr;
+struct ArenaScope {
+    Arena *prev;
+    explicit ArenaScope(Arena *a) : prev(g_arena) { g_arena = a; }
+    ~ArenaScope() { g_arena = prev; }
+    ArenaScope(const ArenaScope &) = delete;
+    ArenaScope &operator=(const ArenaScope &) = delete;
+};
+inline void require_tables_may_be_built(const char *what)
+{
+    if (g_arena != nullptr)
+        throw Error(41, fmt("%s: %s of this plan is not built yet; apply the plan once through f3m_plan_apply with the same "
+                            "number of columns first (that call builds the plan's tables)", g_arena->owner, what));
+}
+
 class Pool {
 public:
     static Pool &get() { static Pool p; return p; }
@@ -70,6 +97,14 @@ public:
     {
         if (bytes == 0) bytes = 256;
         bytes = (bytes + 255) & ~size_t(255);
+        if (Arena *a = g_arena) {
+            if (bytes > a->cap - a->used)
+                throw Error(42, fmt("%s: the product needs more than the %zu MiB of static scratch memory (request of %zu bytes "
+                                    "after %zu in use)", a->owner, a->cap >> 20, bytes, a->used));
+            void *p = a->base + a->used;
+            a->used += bytes;
+            return p;
+        }
         int dev = 0;
         (void)hipGetDevice(&dev);                   // blocks are cached per device
         std::lock_guard<std::mutex> g(mu_);
@@ -292,6 +327,27 @@ inline void check_launch(const char *what)
 {
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) throw Error(102, fmt("launch of %s failed: %s", what, hipGetErrorString(e)));
+}
+
+// Fills device memory with a byte value, as a kernel (a memset node recorded into a captured graph has
+// given wrong results on replays on this GPU pool, and the engine's fills are small or sit next to
+// kernels of the same stream anyway).  p and bytes are multiples of 4.
+template <int BLOCK>
+__global__ void __launch_bounds__(BLOCK) fill_words_kernel(unsigned *__restrict__ p, size_t n32, unsigned word)
+{
+    size_t i = (size_t)blockIdx.x * BLOCK + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * BLOCK;
+    for (; i < n32; i += step) p[i] = word;
+}
+inline void dev_fill(void *p, int byte, size_t bytes, hipStream_t s)
+{
+    if (bytes == 0) return;
+    if ((reinterpret_cast<uintptr_t>(p) | bytes) & 3) throw Error(104, "fill of a range that is not a multiple of 4 bytes");
+    const unsigned b = (unsigned)byte & 255u, word = b * 0x01010101u;
+    const size_t n32 = bytes / 4;
+    const unsigned grid = (unsigned)std::min<size_t>((n32 + 255) / 256, 8192);
+    F3M_LAUNCH((fill_words_kernel<256>), grid, 256, 0, s, static_cast<unsigned *>(p), n32, word);
+    check_launch("fill");
 }
 
 // ---- wave helpers ---------------------------------------------------------------------------
