@@ -572,6 +572,68 @@ int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stre
     });
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------------------
+// Its temporaries (the sorted copies of b and of the result, moments and local expansions, partial sums)
+// come from this array, one copy per GPU, which the device holds from the moment the library is loaded.
+// In host code the name `scratch` is only a handle for hipGetSymbolAddress: the device address is asked
+// for once per device and kept.
+constexpr size_t kScratchBytes = (size_t)128 << 20;
+#ifndef F3M_CPU_EMU
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+#else
+alignas(256) static unsigned char scratch[kScratchBytes];
+#endif
+
+namespace f3m {
+static void *scratch_address()
+{
+    static std::mutex mu;
+    static std::map<int, void *> addr;        // device -> address of that device's copy of the array
+    int dev = 0;
+    F3M_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(mu);
+    auto it = addr.find(dev);
+    if (it != addr.end()) return it->second;
+    void *ptr = nullptr;
+#ifndef F3M_CPU_EMU
+    F3M_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+#else
+    ptr = scratch;
+#endif
+    F3M_REQUIRE(ptr != nullptr, 100, "no device address for the static scratch memory");
+    addr[dev] = ptr;
+    return ptr;
+}
+}  // namespace f3m
+
+int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream)
+{
+    return guarded([&] {
+        F3M_REQUIRE(plan != nullptr, 1, "plan is NULL");
+        F3M_REQUIRE(c >= 1, 12, "b has no columns");
+        // what the call needs at the least: the sorted copies of b and of the result
+        const size_t width = c >= 2 ? 4 : 1;
+        const size_t least = plan->levels.empty() ? 0 : sizeof(float) * width * ((size_t)plan->M + 32 + (size_t)plan->N);
+        F3M_REQUIRE(least <= kScratchBytes, 42,
+                    "f3m_plan_apply_noalloc: a product with N=%lld, M=%lld, c=%d needs more than %zu MiB of scratch memory; the "
+                    "static scratch memory holds %zu MiB (use f3m_plan_apply)", plan->N, plan->M, c, least >> 20, kScratchBytes >> 20);
+        Arena arena;
+        arena.base = static_cast<char *>(scratch_address());
+        arena.cap = kScratchBytes;
+        arena.owner = "f3m_plan_apply_noalloc";
+        ArenaScope scope(&arena);
+        const bool timing = g_timer.enabled;      // stage timing creates events: off for this call
+        g_timer.enabled = false;
+        try {
+            plan_apply(plan, b, c, out, (hipStream_t)stream);
+        } catch (...) {
+            g_timer.enabled = timing;
+            throw;
+        }
+        g_timer.enabled = timing;
+    });
+}
+
 int f3m_plan_destroy(f3m_plan *plan)
 {
     return guarded([&] { delete plan; });

@@ -136,6 +136,20 @@ class Plan:
 
     __matmul__ = apply
 
+    def apply_noalloc(self, b, out):
+        """The same product written into `out` (N, c) without any device allocation by the library: its
+        temporaries come from static device memory (128 MiB per GPU).  The plan must have been applied once
+        with the same number of columns before; b and out must already be contiguous fp32 device tensors."""
+        _need_cuda(b, out)
+        if b.dtype != torch.float32 or out.dtype != torch.float32 or not b.is_contiguous() or not out.is_contiguous():
+            raise AssertionError("b and out must be contiguous fp32 tensors")
+        if b.dim() != 2 or b.shape[0] != self.M or out.shape != (self.N, b.shape[1]):
+            raise AssertionError("b must be (M, c) and out (N, c)")
+        with torch.cuda.device(self.device):
+            rc = self._lib.f3m_plan_apply_noalloc(self._h, _ptr(b), b.shape[1], _ptr(out), _stream())
+        capi.check(self._lib, rc)
+        return out
+
     def level_sizes(self, level):
         s = (C.c_int64 * 8)()
         e = C.c_float()

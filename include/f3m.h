@@ -61,6 +61,17 @@ int f3m_plan_create(int d, const float *X, int64_t N, const float *Y, int64_t M,
                     void *stream, f3m_plan **plan);
 int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stream);
 int f3m_plan_destroy(f3m_plan *plan);
+/* f3m_plan_apply without any device allocation.  No counterpart in the reference: it is for callers that
+ * cannot allocate (a stream under HIP graph capture, a serving loop that must not touch the allocator, a
+ * harness that forbids hipMalloc).  Same arguments and result as f3m_plan_apply.  Its temporaries live in
+ * 128 MiB of static device memory that every GPU running the library holds until the process ends; a
+ * product that needs more (roughly 4 (N + M) bytes per column group of up to 4 columns, plus the moments
+ * and local expansions of the levels: N = M = 1e7 with one column just fits) is refused with error 42 and
+ * nothing is written to out.  The plan's own tables are built by the first f3m_plan_apply with the same
+ * number of columns, which must therefore have run once before (otherwise error 41).  All calls on a GPU
+ * share the one scratch array: calls that overlap on one GPU race, also from different plans or threads.
+ * The call waits for the stream like the others, except while the stream is being captured. */
+int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream);
 
 /* Introspection for parity tests (no counterpart is exported by the reference; the data are its
  * n_tree_cuda members, F3M_src/n_tree.cu:51-78, and the three lists of separate_interactions,

@@ -1,0 +1,86 @@
+"""f3m_plan_apply_noalloc (the entry point that allocates nothing: its temporaries live in static device
+memory) against f3m_plan_apply, through the C ABI.  Results must be the same bit for bit: both run the
+same kernels in the same order, only the memory of the temporaries differs.  Two calls in a row, the
+second on a smaller problem, so that whatever the first call left in the shared scratch array is there
+when the second runs."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+f32 = np.float32
+
+
+@pytest.fixture(scope="module")
+def eng():
+    import torch
+    assert torch.cuda.is_available(), "these tests need a GPU"
+    from f3m_amd import engine
+    engine._lib.get()
+    return engine
+
+
+def dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _reserved(eng):
+    import torch
+    torch.cuda.synchronize()
+    return torch.cuda.memory_reserved()
+
+
+def test_apply_without_allocation_matches_apply(eng):
+    import torch
+    from f3m_amd.capi import F3MError
+    rng = np.random.default_rng(31)
+    print("case no-alloc: 3-D 300000 points, then 4-D 60000 x 20000 points with 3 columns", flush=True)
+    X1 = rng.random((300000, 3), dtype=f32)
+    b1 = rng.standard_normal((300000, 1)).astype(f32)
+    X2 = rng.random((60000, 4), dtype=f32)
+    Y2 = rng.random((20000, 4), dtype=f32)
+    b2 = rng.standard_normal((20000, 3)).astype(f32)
+    p1 = eng.Plan(dev(X1), None, ls=0.7)
+    p2 = eng.Plan(dev(X2), dev(Y2), ls=1.0, nr_of_interpolation=81, min_points=500, small_field_points=200)
+    assert p1.depth >= 2 and p2.depth >= 1
+    b1d, b2d = dev(b1), dev(b2)
+    out1 = torch.full((300000, 1), float("nan"), device="cuda")
+    # a plan whose tables are not built yet is refused, and nothing is written
+    with pytest.raises(F3MError) as e:
+        p1.apply_noalloc(b1d, out1)
+    assert e.value.code == 41 and torch.isnan(out1).all()
+    want1 = p1.apply(b1d)                       # builds the tables of the plan
+    want2 = p2.apply(b2d)
+    out2 = torch.full((60000, 3), float("nan"), device="cuda")
+    eng.release_cache()                         # the library's buffer cache is empty: any allocation would show
+    lib = eng._lib.get()
+    free0 = torch.cuda.mem_get_info()[0]
+    p1.apply_noalloc(b1d, out1)                 # first call
+    p2.apply_noalloc(b2d, out2)                 # second call, smaller, same scratch array
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0            # no device memory was taken
+    assert np.array_equal(out1.cpu().numpy(), want1.cpu().numpy())
+    assert np.array_equal(out2.cpu().numpy(), want2.cpu().numpy())
+    # and again in the other order, results unchanged
+    out1.fill_(float("nan"))
+    p1.apply_noalloc(b1d, out1)
+    assert np.array_equal(out1.cpu().numpy(), want1.cpu().numpy())
+    del lib
+
+
+def test_apply_without_allocation_refuses_what_does_not_fit(eng):
+    import torch
+    from f3m_amd.capi import F3MError
+    print("case no-alloc: refusal above the scratch size", flush=True)
+    rng = np.random.default_rng(32)
+    n = 6_000_000                               # 4 columns: 4 * 4 * (N + M) bytes = 192 MB > 128 MiB
+    X = torch.from_numpy(rng.random((n, 3), dtype=f32)).cuda()
+    b = torch.from_numpy(rng.standard_normal((n, 4)).astype(f32)).cuda()
+    plan = eng.Plan(X, None, ls=1.0)
+    plan.apply(b)
+    out = torch.full((n, 4), float("nan"), device="cuda")
+    with pytest.raises(F3MError) as e:
+        plan.apply_noalloc(b, out)
+    assert e.value.code == 42 and "scratch" in str(e.value)
+    assert torch.isnan(out).all()
+    plan.close()
