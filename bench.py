@@ -1,25 +1,38 @@
 #!/usr/bin/env python3
 """Benchmark of the F3M kernel-matrix-vector product on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--dist uniform|normal] [--ls LS]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--n N] [--config NAME] [--no-extra]
 
-A step is one complete product out = K(X,X) b through the C ABI (box division + interaction lists +
+A step is one complete product out = K(X,Y) b through the C ABI (box division + interaction lists +
 near field + far field), inputs resident in HBM, like one `FFM(X) @ b` of the reference
-(experiments/experiments.py:72-77).  Prints one JSON line.
+(experiments/experiments.py:72-77).  Prints one JSON line: the headline configuration (N = 1e7 uniform in
+[0,1]^3, ls = 1, 64 nodes per box) with the roofline of its dominant kernel and the CPU baseline, and under
+"extra" the time, error and near-field roofline fraction of every other benchmark configuration.
 """
 import argparse
 import json
 import os
+import re
+import statistics
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak
-# HBM bytes moved by one near-field launch of the default workload, from the rocprofv3 FETCH_SIZE and
-# WRITE_SIZE counter runs summarised in profiles/ (None until measured)
-NEAR_TRAFFIC_BYTES = 6.072e9
+PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak (vector or matrix pipe)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "near_g_kernel_n1e7_uniform3d_counters.md")
+
+
+def near_traffic_bytes():
+    """HBM bytes per near-field launch of the headline workload and the range seen over the profiled runs,
+    from the line `traffic_bytes_per_launch: V (range LO - HI)` of the rocprofv3 counter summary."""
+    try:
+        m = re.search(r"traffic_bytes_per_launch:\s*([0-9.e+]+)\s*\(range\s*([0-9.e+]+)\s*-\s*([0-9.e+]+)\)",
+                      open(TRAFFIC_PROFILE).read())
+        return (float(m.group(1)), [float(m.group(2)), float(m.group(3))]) if m else (None, None)
+    except OSError:
+        return None, None
 
 
 def cpu_baseline(X, Y, b, ls, budget_s=15.0):
@@ -43,21 +56,65 @@ def cpu_baseline(X, Y, b, ls, budget_s=15.0):
             "host_cpu_count": os.cpu_count()}
 
 
+def run_config(name, n, steps, warmup, subsample, keep_inputs=False):
+    """Times `steps` products of one configuration; returns its record (and the inputs if asked)."""
+    import numpy as np
+    import torch
+    from f3m_amd import engine, workloads
+    X, Y, b, prm = workloads.make(name, n, seed=1)
+    d = X.shape[1]
+    engine.set_timing(True)
+    for _ in range(warmup):
+        out = engine.kmvm(X, Y, b, **prm)
+    torch.cuda.synchronize()
+    per_step, stage, near_t, near_n = [], {}, 0.0, 0
+    t_all = time.perf_counter()
+    for _ in range(steps):
+        t0 = time.perf_counter()
+        out = engine.kmvm(X, Y, b, **prm)        # synchronous: the stream is idle on return
+        per_step.append(time.perf_counter() - t0)
+        tm = engine.get_timing()
+        near_t += tm["near"][0]
+        near_n += tm["near"][1]
+        for k, v in tm.items():
+            stage[k] = stage.get(k, 0.0) + v[0]
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t_all
+    plan = engine.Plan(X, Y, **prm)
+    work = plan.work()
+    depth = plan.depth
+    nbx = plan.level_sizes(depth)["nbx"] if depth else 1
+    plan.close()
+    F = 3 * d + 3                                  # flops per kernel evaluation (d sub, d mul, d-1 add, scale, exp, fma)
+    achieved = F * work["near_pairs"] * steps / max(near_t, 1e-12) / 1e12
+    rec = {"ms_per_step": dt / steps * 1e3, "ms_per_step_median": statistics.median(per_step) * 1e3,
+           "points_per_s": n / (dt / steps), "tree_depth": depth, "boxes": nbx,
+           "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stage.items()},
+           "near": {"achieved_tflops": achieved, "frac": achieved / PEAK_FP32_TFLOPS, "launches_per_step": near_n // max(steps, 1),
+                    "ms_per_step": near_t / steps * 1e3, "flops_per_pair": F},
+           "work": work}
+    if subsample:
+        rows = torch.from_numpy(np.random.default_rng(1).choice(n, min(subsample, n), replace=False)).cuda()
+        exact = engine.exact_f64(X[rows].double(), (X if Y is None else Y).double(), b.double(), prm["ls"])
+        rec["rel_l2_error"] = float((out[rows].double() - exact).norm() / exact.norm())
+        rec["rel_l2_rows"] = int(rows.numel())
+        rec["meets_1e-3"] = rec["rel_l2_error"] <= 1e-3
+        rec["algorithm_error_at_this_config"] = workloads.ALGORITHM_ERROR_N1E7.get(name) if n == 10_000_000 else None
+    return (rec, (X, Y, b, prm)) if keep_inputs else rec
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--n", type=int, default=10_000_000)
-    ap.add_argument("--d", type=int, default=3)
-    ap.add_argument("--dist", default="uniform", choices=["uniform", "normal", "clustered"],
-                    help="clustered = the asymmetric benchmark configuration: X from 50 anisotropic Gaussians, Y (n/10 points) uniform over "
-                         "X's bounding box, two trees")
-    ap.add_argument("--ls", type=float, default=1.0)
-    ap.add_argument("--nodes", type=int, default=64)
+    ap.add_argument("--config", default="uniform3_ls1", help="headline configuration (a name of f3m_amd.workloads.CONFIGS)")
     ap.add_argument("--subsample", type=int, default=100_000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-accuracy", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
+    ap.add_argument("--extra-steps", type=int, default=3)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy (a kernel of known HBM traffic, to scale rocprof counters)")
     args = ap.parse_args()
@@ -66,28 +123,14 @@ def main():
               "Run with --gpus 1." % args.gpus, file=sys.stderr)
         sys.exit(2)
 
-    import numpy as np
     import torch
-    from f3m_amd import engine
+    from f3m_amd import workloads
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    g = torch.Generator().manual_seed(1)
-    N, d = args.n, args.d
-    Y = None
-    if args.dist == "clustered":
-        mu, sd = 10 * torch.rand(50, d, generator=g), 0.05 + 0.45 * torch.rand(50, d, generator=g)
-        comp = torch.arange(N) % 50
-        X = (mu[comp] + sd[comp] * torch.randn(N, d, generator=g)).cuda()
-        lo, hi = X.min(0).values.cpu(), X.max(0).values.cpu()
-        Y = (lo + (hi - lo) * torch.rand(N // 10, d, generator=g)).cuda()
-        dist_name = "X: 50 anisotropic Gaussians, Y: %d uniform over the bounding box" % (N // 10)
-    else:
-        X = (torch.rand(N, d, generator=g) if args.dist == "uniform" else torch.randn(N, d, generator=g)).cuda()
-        dist_name = "uniform [0,1]^%d" % d if args.dist == "uniform" else "N(0,I)"
-    M = N if Y is None else Y.shape[0]
-    b = torch.randn(M, 1, generator=g).cuda()
-    prm = dict(ls=args.ls, min_points=1000, nr_of_interpolation=args.nodes, small_field_points=1000)
+    N, name = args.n, args.config
+    cfg = workloads.CONFIGS[name]
+    d = cfg["d"]
 
     if args.copy_probe:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
@@ -97,62 +140,54 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    engine.set_timing(True)
-    for _ in range(args.warmup):
-        out = engine.kmvm(X, Y, b, **prm)
-    torch.cuda.synchronize()
-    near_t, near_n, stage = 0.0, 0, {}
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = engine.kmvm(X, Y, b, **prm)
-        tm = engine.get_timing()
-        near_t += tm["near"][0]
-        near_n += tm["near"][1]
-        for k, v in tm.items():
-            stage[k] = stage.get(k, 0.0) + v[0]
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms = dt / args.steps * 1e3
-
-    plan = engine.Plan(X, Y, **prm)
-    work = plan.work()
-    depth = plan.depth
-    nbx = plan.level_sizes(depth)["nbx"] if depth else 1
-    tiles_per_wave = 5 if (N // max(nbx, 1) + 31) // 32 == 5 else 4     # the library's choice (near_field)
-    plan.close()
-    F = 3 * d + 3                                  # flops per kernel evaluation (d sub, d mul, d-1 add, scale, exp, fma)
-    near_flops = F * work["near_pairs"]
-    near_per_launch_s = near_t / max(near_n, 1)
-    achieved = near_flops * args.steps / max(near_t, 1e-12) / 1e12
-    roofline = {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / PEAK_FP32_TFLOPS, "traffic": NEAR_TRAFFIC_BYTES if (N == 10_000_000 and d == 3) else None,
+    rec, (X, Y, b, prm) = run_config(name, N, args.steps, args.warmup, 0 if args.no_accuracy else args.subsample, keep_inputs=True)
+    M = N if Y is None else Y.shape[0]
+    tiles_per_wave = 5 if (N // max(rec["boxes"], 1) + 31) // 32 == 5 else 4     # the library's choice (near_field)
+    traffic, traffic_range = near_traffic_bytes() if (N == 10_000_000 and name == "uniform3_ls1") else (None, None)
+    near = rec["near"]
+    roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
                 "kernel": "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
-                "note": "near field: exponents on the f16 matrix pipe (hi/lo-split operands, fp32 accumulate), exp2 + FMA on "
-                        "the fp32 vector ALU; priced against the fp32 peak; %d launches/step, %.3f ms per launch, "
-                        "%.3e kernel evaluations/step x %d flops; traffic = HBM bytes per launch from rocprofv3 "
-                        "FETCH_SIZE + WRITE_SIZE (profiles/)" % (near_n // max(args.steps, 1), near_per_launch_s * 1e3,
-                                                               work["near_pairs"], F)}
+                "note": "near field, bound by fp32 vector-ALU issue (one exp2 and one FMA per pair; the exponents come from the "
+                        "f16 matrix pipe with hi/lo-split operands, fp32 accumulate); achieved = %d flops x kernel evaluations / "
+                        "HIP-event time of the launch, priced against the fp32 peak; %d launches/step, %.3f ms per step, "
+                        "%.3e kernel evaluations/step; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE "
+                        "(profiles/near_g_kernel_n1e7_uniform3d_counters.md)"
+                        % (near["flops_per_pair"], near["launches_per_step"], near["ms_per_step"], rec["work"]["near_pairs"])}
     res = {
         "metric": "KMVM points/sec at N=1e7 3D Gaussian (1 GPU); rel-L2 error vs fp64 exact",
-        "value": N / (dt / args.steps), "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
-        "data": "synthetic",
-        "config": {"workload": "%dD Gaussian KMVM %s, N=%d %s, b~N(0,1) (%d,1), ls=%g, %d nodes/box, cutoff 1000 "
-                               "(BASELINE.json configs[%d])" % (d, "X=Y" if Y is None else "X!=Y", N, dist_name, M, args.ls,
-                                                               args.nodes, 2 if Y is not None else (1 if d == 3 else 3)),
-                   "N": N, "d": d, "ls": args.ls, "nodes": args.nodes, "tree_depth": depth},
+        "value": rec["points_per_s"], "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": rec["ms_per_step"], "ms_per_step_median": rec["ms_per_step_median"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%dD Gaussian KMVM, %s, b~N(0,1) (%d,1), ls=%g, %d nodes/box, cutoff 1000 (BASELINE.json configs[%d])"
+                               % (d, workloads.describe(name, N), M, cfg["ls"], cfg["nodes"],
+                                  2 if Y is not None else (1 if d == 3 else 3)),
+                   "name": name, "N": N, "d": d, "ls": cfg["ls"], "nodes": cfg["nodes"], "tree_depth": rec["tree_depth"]},
         "roofline": roofline,
-        "stage_ms_per_step": {k: v / args.steps * 1e3 for k, v in stage.items()},
-        "work": work,
+        "stage_ms_per_step": rec["stage_ms_per_step"],
+        "work": rec["work"],
     }
-    if not args.no_accuracy:
-        rows = torch.from_numpy(np.random.default_rng(1).choice(N, min(args.subsample, N), replace=False)).cuda()
-        exact = engine.exact_f64(X[rows].double(), (X if Y is None else Y).double(), b.double(), args.ls)
-        diff = (out[rows].double() - exact)
-        res["rel_l2_error"] = float(diff.norm() / exact.norm())
-        res["rel_l2_rows"] = int(rows.numel())
+    for k in ("rel_l2_error", "rel_l2_rows"):
+        if k in rec:
+            res[k] = rec[k]
     if not args.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(X, Y, b, args.ls)
+        res["cpu_baseline"] = cpu_baseline(X, Y, b, cfg["ls"])
+    del X, Y, b
+    if not args.no_extra:
+        # every other benchmark configuration at the same N: fewer steps, error on 1e4 seeded rows
+        extra = {}
+        for other in workloads.CONFIGS:
+            if other == name:
+                continue
+            torch.cuda.empty_cache()
+            r = run_config(other, N, args.extra_steps, 1, 0 if args.no_accuracy else 10_000)
+            extra[other] = {"ms_per_step": r["ms_per_step"], "ms_per_step_median": r["ms_per_step_median"],
+                            "rel_l2_error": r.get("rel_l2_error"), "meets_1e-3": r.get("meets_1e-3"),
+                            "algorithm_error_at_this_config": r.get("algorithm_error_at_this_config"),
+                            "near_frac": r["near"]["frac"], "near_ms": r["near"]["ms_per_step"],
+                            "near_launches": r["near"]["launches_per_step"], "tree_depth": r["tree_depth"],
+                            "stage_ms_per_step": r["stage_ms_per_step"], "steps": args.extra_steps}
+        res["extra"] = extra
     print(json.dumps(res))
 
 

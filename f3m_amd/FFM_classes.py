@@ -11,7 +11,7 @@ def _check_shapes(X, Y, b):
         assert Y.shape[1] == X.shape[1]
         assert Y.shape[0] == b.shape[0]
     except AssertionError:
-        print('hey check the shapes of your tensor X,Y and b they dont match up!')
+        print('shape mismatch: X and Y need the same number of columns, b one row per row of Y')
         raise AssertionError
 
 

@@ -6,6 +6,8 @@
 #pragma once
 #include "f3m_rt.h"
 
+#include <cmath>
+
 namespace f3m {
 
 struct Geo {
@@ -63,6 +65,10 @@ struct PairList {
     long long n = 0;
     DBuf<int> pairs;     // (n,2) int32: (bx, by), sorted by (bx, by)
     DBuf<int> rowptr;    // nbx+1: range of each x box
+    // far lists: pairs whose cell offset lies outside the 13 offsets per dimension that the M2L tables of a
+    // level hold (m2l_table_omin .. +12).  Cannot happen (a far pair's parents were closer than 2 parent
+    // edges); plan creation counts them and fails if there is one, so the M2L kernels never meet one.
+    long long beyond_tables = 0;
     // far lists of one tree only: pairs whose y box is neither a child of one of the 3^d parents around
     // the parent of the x box nor a child of a parent two cells away along one axis (a parent pair
     // exactly on the far threshold, kept by rounding); -1 = not counted.  Expected to be 0.
@@ -79,12 +85,24 @@ struct PairList {
 };
 
 struct ClassifyParams {
+    int omin[kMaxD];     // m2l_table_omin per dimension (set by lists_launch)
     int nr_interp;
     int small_limit;
     int var_comp;
     int do_init, en_pair, en_all;
     float crit, lcs, edge;
 };
+
+// Lowest cell offset (y cell - x cell) along one dimension in the separable M2L tables of a level.
+// Centres of a far pair are less than 5 edges apart along every dimension (their parents were closer
+// than 2 parent edges), so offset * edge + (origin_y - origin_x) lies in (-5 edge, 5 edge): at most 11
+// integers from ceil(-5 - delta/edge) on; the tables hold 13 from here.
+constexpr int kM2LOffsets = 13;
+inline int m2l_table_omin(float origin_x, float origin_y, float edge)
+{
+    const double delta = (double)origin_y - (double)origin_x;
+    return (int)std::floor(-5.0 - delta / (double)edge) - 1;
+}
 
 struct PlanLevel {
     PairList far, small_, keep;
@@ -111,8 +129,8 @@ void divide_finish(Tree &t, const int *hstats);
 void divide_discard(Tree &t);
 // The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts and scans (the
 // sizes of the small, far and keep list are then the last entries pos[(c+1)*stride - 1] of the three
-// scans; the number of far pairs outside the M2L tables is added to dtot[3], which the caller keeps
-// zero between levels), lists_finish allocates from the fetched totals htot[0..3] and writes.
+// scans; the number of far pairs outside the sibling-group tables is added to dtot[3] and of those outside
+// the M2L tables of the level to dtot[6], which the caller keeps zero between levels), lists_finish allocates from the fetched totals htot[0..3] and writes.
 // divide_launch likewise adds to dstats[0..1], zero on entry.
 struct ListsPending {
     DBuf<long long> pos;
@@ -120,7 +138,7 @@ struct ListsPending {
     unsigned grid = 0;
     bool active = false;
 };
-void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
                   ListsPending &pend, long long *dtot, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
                   const ClassifyParams &cp, PlanLevel &out, long long *drow /* 8 zeroed words or null */, hipStream_t s);

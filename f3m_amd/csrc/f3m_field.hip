@@ -1273,7 +1273,8 @@ __global__ void __launch_bounds__(1024) m2l_direct_kernel(const float *__restric
 // The tables (a few KB, built on the host in fp64) live in LDS; the moment vector ping-pongs between
 // two LDS buffers.  Same sums as m2l_direct_kernel up to rounding.
 
-constexpr int kM2LOffsets = 13;   // cell offsets per dimension that a far pair can have (|dc| < 5 edge)
+// kM2LOffsets (f3m_engine.h) = cell offsets per dimension held by the tables; plan creation has checked
+// that no far pair lies outside them, the clamps below only keep a table index in bounds whatever happens
 
 struct SepMeta {
     int omin[kMaxD];
@@ -1968,7 +1969,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         for (int j = 0; j < kMaxD; j++) { sm.omin[j] = 0; sg.omin[j] = 0; sg.delta[j] = 0; }
         for (int j = 0; j < d; j++) {
             sg.delta[j] = (double)ty.geo.origin[j] - (double)tx.geo.origin[j];
-            sm.omin[j] = sg.omin[j] = (int)std::floor(-5.0 - sg.delta[j] / edge) - 1;
+            sm.omin[j] = sg.omin[j] = m2l_table_omin(tx.geo.origin[j], ty.geo.origin[j], lx.edge);
         }
         // the tables of the level depend on the plan only (nodes, edge, lengthscale, origins) and are kept with its far list
         DBuf<float> &dtab = far.m2l_tab;

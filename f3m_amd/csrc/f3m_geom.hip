@@ -714,7 +714,8 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     int nbx, const int *__restrict__ csx, int nbx_prev, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
     const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
     const float *__restrict__ ctrx, const float *__restrict__ ctry, int d, ClassifyParams cp,
-    const int *__restrict__ cellx, const int *__restrict__ celly, unsigned long long *__restrict__ outliers,
+    const int *__restrict__ cellx, const int *__restrict__ celly, bool one_tree, unsigned long long *__restrict__ outliers,
+    unsigned long long *__restrict__ beyond,
     long long *__restrict__ cnt /* 3 arrays of nbx+1 */, const long long *__restrict__ pos /* 3 arrays of nbx+1 */,
     int *__restrict__ out_small, int *__restrict__ out_far, int *__restrict__ out_keep, int *__restrict__ rp_small,
     int *__restrict__ rp_far, int *__restrict__ rp_keep)
@@ -764,7 +765,16 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
             if (there) {
                 const int size = nx + (offy[by + 1] - offy[by]);
                 c = classify_pair(cx, ctry + (long long)by * d, d, size, cp);
-                if (!WRITE && c == 1 && cellx != nullptr) {
+                if (!WRITE && c == 1) {
+                    // the cell offset of a far pair must lie inside the M2L tables of the level
+                    bool outside = false;
+                    for (int j = 0; j < d; j++) {
+                        const int o = celly[(long long)by * d + j] - cellx[(long long)bx * d + j] - cp.omin[j];
+                        outside = outside || o < 0 || o >= kM2LOffsets;
+                    }
+                    if (outside) atomicAdd(beyond, 1ull);
+                }
+                if (!WRITE && c == 1 && one_tree) {
                     // regular: every offset from twice the parent's cell in -2..3; or a child of a parent two
                     // cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere
                     int nout = 0, nmid = 0, nbad = 0;
@@ -839,7 +849,7 @@ void build_rowptr(PairList &l, int nbx, hipStream_t s)
     check_launch("rowptr");
 }
 
-void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, const ClassifyParams &cp,
+void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
                   ListsPending &pend, long long *dtot, hipStream_t s)
 {
     const int d = tx.geo.d;
@@ -855,12 +865,14 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     pend.stride = (long long)nbx + 1;
     DBuf<long long> cnt((size_t)(3 * pend.stride));
     pend.pos.reset((size_t)(3 * pend.stride));
-    const int *cellx = one_tree ? lx.cell.get() : (const int *)nullptr;
+    for (int j = 0; j < kMaxD; j++) cp.omin[j] = j < d ? m2l_table_omin(tx.geo.origin[j], ty.geo.origin[j], lx.edge) : 0;
+    const int *cellx = lx.cell.get();
     unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
+    unsigned long long *beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
     pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
     F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cell.get(), outl, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
+               cellx, ly.cell.get(), one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
     exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
@@ -878,6 +890,9 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     const int nbx = lx.nb;
     for (int c = 0; c < 3; c++) F3M_REQUIRE(tot[c] < (1ll << 31) - 2, 22, "interaction list too long (%lld)", tot[c]);
     out.far.outliers = one_tree ? tot[3] : -1;
+    out.far.beyond_tables = tot[6];
+    F3M_REQUIRE(tot[6] == 0, 24, "%lld far pairs of depth %d lie outside the M2L tables (cell offsets beyond %d per dimension)",
+                tot[6], k, kM2LOffsets);
     out.small_.n = tot[0];
     out.far.n = tot[1];
     out.keep.n = tot[2];
@@ -887,10 +902,11 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     out.small_.rowptr.reset((size_t)pend.stride);
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
-    const int *cellx = one_tree ? lx.cell.get() : (const int *)nullptr;
+    const int *cellx = lx.cell.get();
     F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cell.get(), (unsigned long long *)nullptr, (long long *)nullptr, (const long long *)pend.pos.get(),
+               cellx, ly.cell.get(), one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr, (long long *)nullptr,
+               (const long long *)pend.pos.get(),
                out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
                out.far.rowptr.get(), out.keep.rowptr.get());
     check_launch("lists_write");

@@ -230,8 +230,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // level, the division of depth k+1 is started together with the list count of depth k whenever the
     // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
     // Host record of a level, in 32-bit words: [0..5] pairs of the small, far and keep list (64 bits each),
-    // [6,7] far pairs outside the M2L tables, [8,9] boxes and largest box of the X tree's new level,
-    // [10,11] of the Y tree's.  On the device the first three are the last entries of the list builder's
+    // [6,7] far pairs outside the sibling-group M2L tables, [8,9] boxes and largest box of the X tree's new level,
+    // [10,11] of the Y tree's, [12,13] far pairs outside the M2L tables of the level (must be none).  On the device the first three are the last entries of the list builder's
     // scans; the counters behind [6..11] live in dres and are cleared by the readback that fetches them.
     DBuf<int> dres(16);
     dev_fill(dres.get(), 0, 16 * sizeof(int), s);
@@ -242,6 +242,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         if (pend != nullptr && pend->active) {
             for (int c = 0; c < 3; c++) L.add(pend->pos.get() + (c + 1) * pend->stride - 1, 2, 2 * c);
             L.add(dres.get() + 6, 2, 6, true);
+            L.add(dres.get() + 12, 2, 12, true);
         }
         if (division) L.add(dres.get() + 8, sym ? 2 : 4, 8, true);
         if (L.nseg > 0) fetch_segments(L, hres, s);
@@ -272,7 +273,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             const float e = P->tx.lev[k].edge;
             P->levels.emplace_back();
             PlanLevel &L = P->levels.back();
-            const ClassifyParams cp = classify_params(*P, e);
+            ClassifyParams cp = classify_params(*P, e);
             ListsPending pend;
             lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
             const bool ahead = wants_division();

@@ -1,0 +1,65 @@
+"""Seeded synthetic point clouds of the benchmark configurations (CPU generators, torch.manual_seed-style
+streams), shared by bench.py and the full-size GPU tests so that both measure the same inputs.
+
+Every entry of CONFIGS: name -> dict(d, dist, ls, nodes, m_ratio) with
+  dist "uniform"   X = rand(N, d)                                  (X = Y)
+       "normal"    X = randn(N, d)                                 (X = Y)
+       "clustered" X from 50 anisotropic Gaussians, means 10 rand(50, d), per-dimension std 0.05 + 0.45 rand,
+                   Y = N / m_ratio points uniform over X's bounding box (two trees)
+The reference draws its benchmark clouds the same way (experiments/experiments.py:45-60,115: seed 1, uniform
+and normal clouds, b ~ N(0,1))."""
+import torch
+
+CONFIGS = {
+    "uniform3_ls1": dict(d=3, dist="uniform", ls=1.0, nodes=64),
+    "uniform3_ls0.1": dict(d=3, dist="uniform", ls=0.1, nodes=64),
+    "uniform3_ls10": dict(d=3, dist="uniform", ls=10.0, nodes=64),
+    "normal3_ls1": dict(d=3, dist="normal", ls=1.0, nodes=64),
+    "normal3_ls0.1": dict(d=3, dist="normal", ls=0.1, nodes=64),
+    "normal3_ls10": dict(d=3, dist="normal", ls=10.0, nodes=64),
+    "clustered3_xy_ls0.5": dict(d=3, dist="clustered", ls=0.5, nodes=64, m_ratio=10),
+    "uniform4_81nodes": dict(d=4, dist="uniform", ls=1.0, nodes=81),
+    "uniform5_243nodes": dict(d=5, dist="uniform", ls=1.0, nodes=243),
+}
+
+# rel-L2 error of the product against the fp64 exact product that the F3M algorithm itself has at these
+# node counts and lengthscales at N = 1e7 (measured with this engine, which matches the CPU restatement of
+# the reference algorithm to 1e-5 on clouds of the same kind at sizes that restatement can run); the
+# full-size tests allow 1.5x these.  Where the figure is above 1e-3 the algorithm at 64 nodes per box does
+# not reach the 1e-3 target at that lengthscale, whatever computes it.
+ALGORITHM_ERROR_N1E7 = {
+    "uniform3_ls1": 3.4e-6, "uniform3_ls0.1": 1.4e-3, "uniform3_ls10": 6e-7,
+    "normal3_ls1": 1.1e-3, "normal3_ls0.1": 1.4e-3, "normal3_ls10": 1.0e-6,
+    "clustered3_xy_ls0.5": 1.5e-3, "uniform4_81nodes": 1.0e-4, "uniform5_243nodes": 7.7e-4,
+}
+
+
+def make(name, n, seed=1, columns=1, device="cuda"):
+    """-> X, Y (None when X = Y), b, engine parameters; tensors on `device`."""
+    cfg = CONFIGS[name]
+    d = cfg["d"]
+    g = torch.Generator().manual_seed(seed)
+    Y = None
+    if cfg["dist"] == "clustered":
+        mu, sd = 10 * torch.rand(50, d, generator=g), 0.05 + 0.45 * torch.rand(50, d, generator=g)
+        comp = torch.arange(n) % 50
+        X = mu[comp] + sd[comp] * torch.randn(n, d, generator=g)
+        lo, hi = X.min(0).values, X.max(0).values
+        Y = (lo + (hi - lo) * torch.rand(n // cfg["m_ratio"], d, generator=g)).to(device)
+        X = X.to(device)
+    elif cfg["dist"] == "uniform":
+        X = torch.rand(n, d, generator=g).to(device)
+    else:
+        X = torch.randn(n, d, generator=g).to(device)
+    m = n if Y is None else Y.shape[0]
+    b = torch.randn(m, columns, generator=g).to(device)
+    prm = dict(ls=cfg["ls"], min_points=1000, nr_of_interpolation=cfg["nodes"], small_field_points=1000)
+    return X, Y, b, prm
+
+
+def describe(name, n):
+    cfg = CONFIGS[name]
+    d = cfg["d"]
+    if cfg["dist"] == "clustered":
+        return "X: %d points from 50 anisotropic Gaussians in %d-D, Y: %d uniform over X's bounding box" % (n, d, n // cfg["m_ratio"])
+    return "%d points %s, X = Y" % (n, "uniform [0,1]^%d" % d if cfg["dist"] == "uniform" else "N(0,I_%d)" % d)
