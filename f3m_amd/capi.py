@@ -18,7 +18,7 @@ class F3MError(RuntimeError):
 
 SYMBOLS = [
     "f3m_kmvm_f32", "f3m_exact_f32", "f3m_exact_grad_f32", "f3m_exact_f64", "f3m_plan_create", "f3m_plan_apply",
-    "f3m_plan_apply_noalloc", "f3m_plan_destroy", "f3m_plan_depth", "f3m_plan_symmetric", "f3m_plan_level_sizes", "f3m_plan_list_rows", "f3m_plan_level_copy",
+    "f3m_plan_apply_noalloc", "f3m_plan_apply_transpose", "f3m_plan_destroy", "f3m_plan_depth", "f3m_plan_symmetric", "f3m_plan_level_sizes", "f3m_plan_list_rows", "f3m_plan_level_copy",
     "f3m_plan_far_level", "f3m_plan_near_level", "f3m_plan_work", "f3m_plan_lookup_boxes", "f3m_hash_slot",
     "f3m_set_timing", "f3m_get_timing",
     "f3m_last_error", "f3m_release_cache", "f3m_version",
@@ -36,6 +36,7 @@ def bind(lib):
     lib.f3m_plan_create.argtypes = [i, vp, i64, vp, i64, pp, vp, C.POINTER(vp)]
     lib.f3m_plan_apply.argtypes = [vp, vp, i, vp, vp]
     lib.f3m_plan_apply_noalloc.argtypes = [vp, vp, i, vp, vp]
+    lib.f3m_plan_apply_transpose.argtypes = [vp, vp, i, vp, vp]
     lib.f3m_plan_destroy.argtypes = [vp]
     lib.f3m_plan_depth.argtypes = [vp]
     lib.f3m_plan_symmetric.argtypes = [vp]

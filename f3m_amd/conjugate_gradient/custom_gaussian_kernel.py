@@ -13,7 +13,8 @@ class custom_GaussianKernel:
     product with the (X1, X2) it is given -- min_points defaults to 4^d and the small-field cutoff to
     the node count (:21-25) -- and kept: ``mmv`` multiplies by K(X1,X2), ``dmmv`` computes
     K(X1,X2)^T (K(X1,X2) v + w).  Where the reference makes 48 chunked engine calls for the transposed
-    product (:85), one plan of (X2, X1) is built once and reused."""
+    product (:85), the one plan of (X1, X2) serves both products: the transposed one swaps the roles of
+    its two trees and reads every interaction list from its X2 boxes."""
 
     def __init__(self, sigma, opt=None, min_points=None, var_compression=True, interpolation_nr=64, eff_var_limit=0.3):
         self.sigma = float(sigma)
@@ -26,7 +27,6 @@ class custom_GaussianKernel:
         self.ffm_initialized = False
         self.device = "cuda:0"
         self._fwd = None
-        self._bwd = None
         self._plan_key = None
 
     # dense kernel matrix, used for the M x M preconditioner only
@@ -59,7 +59,6 @@ class custom_GaussianKernel:
             Yd = X2.to(self.device, torch.float32)
             prm = self._engine_params(Xd.shape[1])
             self._fwd = engine.Plan(Xd, Yd, **prm)
-            self._bwd = engine.Plan(Yd, Xd, **prm)
             self._plan_key = key
             self.ffm_initialized = True
 
@@ -86,4 +85,4 @@ class custom_GaussianKernel:
             res = self._fwd.apply(v.to(self.device, torch.float32))
             if w is not None:
                 res = res + w.to(self.device, torch.float32)
-        return self._bwd.apply(res).to(X1.device)
+        return self._fwd.apply_transpose(res).to(X1.device)

@@ -106,6 +106,10 @@ inline int m2l_table_omin(float origin_x, float origin_y, float edge)
 
 struct PlanLevel {
     PairList far, small_, keep;
+    // the same lists seen from the Y boxes, (by, bx) sorted by (by, bx) with row pointers over the Y boxes:
+    // what the transposed product K(X,Y)^T u walks (built on its first use; plans of two trees only)
+    PairList farT, smallT, keepT;
+    bool haveT = false;
     int num_nodes = 0;
 };
 
@@ -142,6 +146,9 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                   ListsPending &pend, long long *dtot, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
                   const ClassifyParams &cp, PlanLevel &out, long long *drow /* 8 zeroed words or null */, hipStream_t s);
+// out = `in` with the two boxes of every pair swapped, sorted by (by, bx) (a stable sort by `by` of a list that is
+// sorted by bx), its row pointers over the nby boxes of the Y level, and its row statistics for the near field
+void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipStream_t s);
 void exclusive_scan_i32(const int *in, long long n, int *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64(const long long *in, long long n, long long *out /* n+1 */, hipStream_t s);
 void exclusive_scan_i64_batched(const long long *in, long long n, long long pitch, int nch, long long *out, hipStream_t s);

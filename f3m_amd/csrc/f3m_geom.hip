@@ -849,6 +849,68 @@ void build_rowptr(PairList &l, int nbx, hipStream_t s)
     check_launch("rowptr");
 }
 
+// ------------------------------------------------------------------------------------------------
+// A list seen from its Y boxes.  The predicates of a pair depend on n_x + n_y and on |c_y - c_x| only
+// (F3M_src/1_d_conv.cu:927-952), so the lists of the problem (Y, X) are these lists with the boxes of every pair
+// swapped, in the order (by, bx): a stable sort by `by` of pairs that are already sorted by bx.
+
+__global__ void split_pairs_kernel(const int *__restrict__ pairs, long long n, uint32_t *__restrict__ key, int *__restrict__ val)
+{
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) { key[t] = (uint32_t)pairs[2 * t + 1]; val[t] = pairs[2 * t]; }
+}
+__global__ void join_pairs_kernel(const uint32_t *__restrict__ key, const int *__restrict__ val, long long n, int *__restrict__ pairs)
+{
+    long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) { pairs[2 * t] = (int)key[t]; pairs[2 * t + 1] = val[t]; }
+}
+// row statistics of one list (the first four words of list_rowstats_kernel's record)
+__global__ void __launch_bounds__(kRowStatBlock) one_list_rowstats_kernel(const int *__restrict__ rowptr, const int *__restrict__ off,
+                                                                           int nb, unsigned long long *__restrict__ out)
+{
+    __shared__ unsigned long long acc[4];
+    if (threadIdx.x < 4) acc[threadIdx.x] = 0;
+    __syncthreads();
+    const int b = blockIdx.x * kRowStatBlock + threadIdx.x;
+    if (b < nb && rowptr[b + 1] > rowptr[b]) {
+        const unsigned long long n = (unsigned long long)(off[b + 1] - off[b]);
+        atomicAdd(&acc[0], 1ull);
+        atomicAdd(&acc[1], n);
+        atomicAdd(&acc[2], (n + 127) / 128);
+        atomicAdd(&acc[3], (n + 159) / 160);
+    }
+    __syncthreads();
+    if (threadIdx.x < 4 && acc[threadIdx.x]) atomicAdd(&out[threadIdx.x], acc[threadIdx.x]);
+}
+
+void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipStream_t s)
+{
+    out.n = in.n;
+    out.outliers = -1;
+    out.beyond_tables = 0;
+    out.pairs.reset((size_t)std::max<long long>(1, in.n) * 2);
+    if (in.n > 0) {
+        DBuf<uint32_t> key((size_t)in.n);
+        DBuf<int> val((size_t)in.n);
+        F3M_LAUNCH(split_pairs_kernel, cdiv(in.n, 256), 256, 0, s, in.pairs.get(), in.n, key.get(), val.get());
+        check_launch("split_pairs");
+        int bits = 1;
+        while ((1ll << bits) < (long long)ly.nb) bits++;
+        radix_sort(key, val, in.n, 0, bits, s);
+        F3M_LAUNCH(join_pairs_kernel, cdiv(in.n, 256), 256, 0, s, key.get(), val.get(), in.n, out.pairs.get());
+        check_launch("join_pairs");
+    }
+    build_rowptr(out, ly.nb, s);
+    DBuf<unsigned long long> dstat(4);
+    dev_fill(dstat.get(), 0, 4 * sizeof(unsigned long long), s);
+    F3M_LAUNCH(one_list_rowstats_kernel, cdiv(ly.nb, kRowStatBlock), kRowStatBlock, 0, s, out.rowptr.get(), ly.off.get(), ly.nb,
+               dstat.get());
+    check_launch("one_list_rowstats");
+    unsigned long long h[4];
+    fetch_small(h, dstat.get(), 4, s);
+    out.rows = (long long)h[0], out.row_points = (long long)h[1], out.items128 = (long long)h[2], out.items160 = (long long)h[3];
+}
+
 void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
                   ListsPending &pend, long long *dtot, hipStream_t s)
 {

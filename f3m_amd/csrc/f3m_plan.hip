@@ -355,12 +355,15 @@ static void far_level(f3m_plan *P, int level, const float *bs, float *outs, floa
 // Where a level has more nodes per dimension than the next deeper one (var_compression lowers the node
 // count of small boxes, F3M_src/n_tree.cu:971-978) the hand-over would not be exact, and that level
 // is interpolated from / evaluated at the points directly, as the reference does for every level.
-static void far_tree(f3m_plan *P, const float *bs, float *outs, hipStream_t s)
+static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs, hipStream_t s)
 {
     const int depth = (int)P->levels.size();
+    // targets and sources of this product: the X and Y tree, or the other way round for K(X,Y)^T
+    const Tree &TX = transposed ? *P->ty : P->tx, &TY = transposed ? P->tx : *P->ty;
+    auto far_of = [&](int k) -> const PairList & { return transposed ? P->levels[k - 1].farT : P->levels[k - 1].far; };
     int ku = 0, kd = 0;
     for (int k = 1; k <= depth; k++)
-        if (P->levels[k - 1].far.n > 0) { if (!ku) ku = k; kd = k; }
+        if (far_of(k).n > 0) { if (!ku) ku = k; kd = k; }
     if (!ku) return;
     const int mode = m2l_mode_env();
     const int d = P->d;
@@ -369,13 +372,13 @@ static void far_tree(f3m_plan *P, const float *bs, float *outs, hipStream_t s)
     // upward
     for (int k = kd; k >= ku; k--) {
         NodeSet &ns = ns_of(k);
-        const TreeLevel &ly = P->ty->lev[k];
+        const TreeLevel &ly = TY.lev[k];
         mom[k].reset((size_t)ly.nb * ns.P);
         if (k < kd && nodes_nest(ns, ns_of(k + 1))) {
             const float *tab = P->shift_table(P->levels[k - 1].num_nodes, P->levels[k].num_nodes, s);
-            shift_level(false, ly, P->ty->lev[k + 1], ns, ns_of(k + 1), tab, mom[k + 1].get(), mom[k].get(), s);
+            shift_level(false, ly, TY.lev[k + 1], ns, ns_of(k + 1), tab, mom[k + 1].get(), mom[k].get(), s);
         } else {
-            p2m_level(d, *P->ty, ly, nullptr, ns, bs, mom[k].get(), s);
+            p2m_level(d, TY, ly, nullptr, ns, bs, mom[k].get(), s);
         }
     }
     // downward
@@ -383,23 +386,40 @@ static void far_tree(f3m_plan *P, const float *bs, float *outs, hipStream_t s)
     int pending = 0;        // level whose local expansions (in prev) still wait to be evaluated
     for (int k = ku; k <= kd; k++) {
         NodeSet &ns = ns_of(k);
-        const TreeLevel &lx = P->tx.lev[k];
+        const TreeLevel &lx = TX.lev[k];
         loc.reset((size_t)lx.nb * ns.P);
-        m2l_level(d, P->tx, lx, *P->ty, P->ty->lev[k], P->levels[k - 1].far, ns, P->lcs, mode, mom[k].get(), loc.get(), s);
+        m2l_level(d, TX, lx, TY, TY.lev[k], far_of(k), ns, P->lcs, mode, mom[k].get(), loc.get(), s);
         mom[k].free();
         if (pending) {
             NodeSet &nsp = ns_of(pending);
             if (nodes_nest(nsp, ns)) {
                 const float *tab = P->shift_table(P->levels[pending - 1].num_nodes, P->levels[k - 1].num_nodes, s);
-                shift_level(true, P->tx.lev[pending], lx, nsp, ns, tab, prev.get(), loc.get(), s);
+                shift_level(true, TX.lev[pending], lx, nsp, ns, tab, prev.get(), loc.get(), s);
             } else {
-                l2p_level(d, P->tx, P->tx.lev[pending], nullptr, nsp, prev.get(), outs, s);
+                l2p_level(d, TX, TX.lev[pending], nullptr, nsp, prev.get(), outs, s);
             }
         }
         std::swap(loc, prev);
         pending = k;
     }
-    l2p_level(d, P->tx, P->tx.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s);
+    l2p_level(d, TX, TX.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s);
+}
+
+// The lists seen from the Y boxes, for the transposed product (built once, on its first use).
+static void ensure_transposed_lists(f3m_plan *P, hipStream_t s)
+{
+    if (P->symmetric) return;          // one tree: K and every list are symmetric
+    for (size_t l = 0; l < P->levels.size(); l++) {
+        PlanLevel &L = P->levels[l];
+        if (L.haveT) continue;
+        require_tables_may_be_built("the transposed lists");
+        const TreeLevel &ly = P->ty->lev[l + 1];
+        transpose_list(L.far, ly, L.farT, s);
+        transpose_list(L.small_, ly, L.smallT, s);
+        // only the keep list of the last level is ever summed
+        if (l + 1 == P->levels.size()) transpose_list(L.keep, ly, L.keepT, s);
+        L.haveT = true;
+    }
 }
 
 // waits for the stream, except while it is being captured into a graph (where a wait is an error and
@@ -414,29 +434,38 @@ static void finish_stream(hipStream_t s)
     F3M_HIP(hipStreamSynchronize(s));
 }
 
-static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s)
+// out = K(X,Y) b, or with `transposed` out = K(X,Y)^T b (b then has N rows and out M): the same trees
+// with the roles of targets and sources swapped and every list seen from its Y boxes.
+static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s, bool transposed = false)
 {
     F3M_REQUIRE(P != nullptr, 1, "plan is NULL");
     F3M_REQUIRE(c >= 1, 12, "b has no columns");
     check_device_ptr(b, "b");
     check_device_ptr(out, "out");
+    if (P->symmetric) transposed = false;           // K(X,X) is symmetric
     if (P->levels.empty()) {
         const float *Yp = P->symmetric ? P->Xraw.get() : P->Yraw.get();
         Scope sc(kNear, s);
-        exact_f32(P->d, P->Xraw.get(), P->N, Yp, P->M, b, c, P->prm.ls, false, out, s);
+        if (transposed) exact_f32(P->d, Yp, P->M, P->Xraw.get(), P->N, b, c, P->prm.ls, false, out, s);
+        else exact_f32(P->d, P->Xraw.get(), P->N, Yp, P->M, b, c, P->prm.ls, false, out, s);
         finish_stream(s);
         return;
     }
+    if (transposed) ensure_transposed_lists(P, s);
+    const Tree &TX = transposed ? *P->ty : P->tx, &TY = transposed ? P->tx : *P->ty;     // targets, sources
+    const long long NT = TX.n, NS = TY.n;
+    auto small_of = [&](int k) -> const PairList & { return transposed ? P->levels[k - 1].smallT : P->levels[k - 1].small_; };
+    auto keep_of = [&](int k) -> const PairList & { return transposed ? P->levels[k - 1].keepT : P->levels[k - 1].keep; };
     // Columns are taken four at a time while at least three are left (the near field then computes every
     // exponential once for the four), two at a time when two are left, else one.  bs columns are padded by one tile:
     // near_g_kernel reads whole tiles.
-    const long long bstride = P->M + 32, ostride = P->N;
+    const long long bstride = NS + 32, ostride = NT;
     const int width = c >= 2 ? 4 : 1;
     DBuf<float> bs((size_t)bstride * width), outs((size_t)ostride * width);
     const int depth = (int)P->levels.size();
     // F3M_FAR=levels: interpolate every level from the points like the reference (cross-check)
     const char *fe = getenv("F3M_FAR");
-    const bool per_level = fe && !strcmp(fe, "levels");
+    const bool per_level = fe && !strcmp(fe, "levels") && !transposed;
     for (int col = 0; col < c;) {
         const int left = c - col;
         const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);   // columns of this pass (past `left`: zero weights)
@@ -444,26 +473,25 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         {
             Scope sc(kPerm, s);
             if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
-            for (int q = 0; q < ncol; q++) gather_column(b, P->ty->perm.get(), P->M, c, col + q, bs.get() + q * bstride, s);
+            for (int q = 0; q < ncol; q++) gather_column(b, TY.perm.get(), NS, c, col + q, bs.get() + q * bstride, s);
             dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
         }
         for (int k = 1; k <= depth; k++) {
-            PlanLevel &L = P->levels[k - 1];
             // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
-            near_field(P->d, P->tx, P->tx.lev[k], *P->ty, P->ty->lev[k], L.small_, bs.get(), outs.get(), P->lcs, s, nc,
-                       bstride, ostride, /*only_list=*/k < depth || P->levels[depth - 1].keep.n == 0);
+            near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
+                       bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0);
             if (per_level)
                 for (int q = 0; q < ncol; q++)
                     far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
         }
         if (!per_level)
-            for (int q = 0; q < ncol; q++) far_tree(P, bs.get() + q * bstride, outs.get() + q * ostride, s);
+            for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs.get() + q * ostride, s);
         // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
-        near_field(P->d, P->tx, P->tx.lev[depth], *P->ty, P->ty->lev[depth], P->levels[depth - 1].keep, bs.get(),
+        near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
                    outs.get(), P->lcs, s, nc, bstride, ostride);
         {
             Scope sc(kPerm, s);
-            for (int q = 0; q < ncol; q++) scatter_column(outs.get() + q * ostride, P->tx.perm.get(), P->N, c, col + q, out, s);
+            for (int q = 0; q < ncol; q++) scatter_column(outs.get() + q * ostride, TX.perm.get(), NT, c, col + q, out, s);
         }
         col += ncol;
     }
@@ -569,6 +597,15 @@ int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stre
     return guarded([&] {
         g_timer.reset();
         plan_apply(plan, b, c, out, (hipStream_t)stream);
+        g_timer.collect();
+    });
+}
+
+int f3m_plan_apply_transpose(f3m_plan *plan, const float *u, int c, float *out, void *stream)
+{
+    return guarded([&] {
+        g_timer.reset();
+        plan_apply(plan, u, c, out, (hipStream_t)stream, /*transposed=*/true);
         g_timer.collect();
     });
 }

@@ -136,6 +136,19 @@ class Plan:
 
     __matmul__ = apply
 
+    def apply_transpose(self, u):
+        """K(X,Y)^T u with this plan's trees and lists (u has N rows, the result M): what a second plan of
+        (Y, X) would give (reference: FFM.chunk_forward_transpose, experiments/FFM_classes.py:54-61)."""
+        _need_cuda(u)
+        u = _prep(u, torch.float32)
+        if u.dim() != 2 or u.shape[0] != self.N:
+            raise AssertionError("u must be (N, c)")
+        out = torch.empty((self.M, u.shape[1]), dtype=torch.float32, device=self.device)
+        with torch.cuda.device(self.device):
+            rc = self._lib.f3m_plan_apply_transpose(self._h, _ptr(u), u.shape[1], _ptr(out), _stream())
+        capi.check(self._lib, rc)
+        return out
+
     def apply_noalloc(self, b, out):
         """The same product written into `out` (N, c) without any device allocation by the library: its
         temporaries come from static device memory (128 MiB per GPU).  The plan must have been applied once

@@ -60,6 +60,13 @@ int f3m_exact_f64(int d, const double *X, int64_t N, const double *Y, int64_t M,
 int f3m_plan_create(int d, const float *X, int64_t N, const float *Y, int64_t M, const f3m_params *params,
                     void *stream, f3m_plan **plan);
 int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stream);
+/* out(M,c) = K(X,Y)^T u, u (N,c), with the plan of (X, Y): the two trees swap roles and every interaction
+ * list is read from its Y boxes (the lists of (Y, X) are the lists of (X, Y) with the boxes of each pair
+ * swapped: the classification of F3M_src/1_d_conv.cu:927-952 depends on n_x + n_y and |c_y - c_x| only).
+ * Replaces FFM.chunk_forward_transpose (experiments/FFM_classes.py:54-61: one FFM_XY call per chunk of the
+ * rows of X, 48 of them per product at conjugate_gradient/custom_gaussian_kernel.py:85) and a second plan of
+ * (Y, X), whose product it equals.  The transposed lists are built by the first call and kept. */
+int f3m_plan_apply_transpose(f3m_plan *plan, const float *u, int c, float *out, void *stream);
 int f3m_plan_destroy(f3m_plan *plan);
 /* f3m_plan_apply without any device allocation.  No counterpart in the reference: it is for callers that
  * cannot allocate (a stream under HIP graph capture, a serving loop that must not touch the allocator, a

@@ -111,6 +111,12 @@ class Plan:
         capi.check(lib(), lib().f3m_plan_apply(self._h, _p(b), b.shape[1], _p(out), None))
         return out
 
+    def apply_transpose(self, u):
+        u = _f32(u)
+        out = np.empty((self.M, u.shape[1]), np.float32)
+        capi.check(lib(), lib().f3m_plan_apply_transpose(self._h, _p(u), u.shape[1], _p(out), None))
+        return out
+
     def far_level(self, level, b, P):
         b = _f32(b)
         sz = self.level_sizes(level)

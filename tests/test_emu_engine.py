@@ -137,6 +137,30 @@ def test_stages_and_product(oracle, name, P):
     assert rel_l2(ee.kmvm(X, Y, b, **prm), got) == 0.0
 
 
+@pytest.mark.parametrize("name,P", [("asym3", 64), ("asym3", 27)])
+def test_transposed_product_on_the_same_plan(oracle, name, P):
+    """K(X,Y)^T u from the plan of (X, Y) -- trees swapped, lists read from their Y boxes -- is what the plan
+    of (Y, X) gives, bit for bit (same lists, same kernels, same order), and the oracle's product of (Y, X)."""
+    rng = np.random.default_rng(23)
+    X, Y = _cloud(name, rng)
+    u = rng.standard_normal((X.shape[0], 2)).astype(f32)
+    prm = dict(PRM, nr_of_interpolation=P)
+    fwd, bwd = ee.Plan(X, Y, **prm), ee.Plan(Y, X, **prm)
+    assert fwd.depth == bwd.depth and sum(fwd.level_sizes(k)["nfar"] for k in range(1, fwd.depth + 1)) > 0
+    for k in range(1, fwd.depth + 1):                       # the lists of (Y, X) are the transposed lists of (X, Y)
+        A, B = fwd.level(k), bwd.level(k)
+        for lst in ("far", "small", "keep"):
+            t = A[lst][:, ::-1]
+            assert np.array_equal(t[np.lexsort((t[:, 1], t[:, 0]))], B[lst]), (k, lst)
+    got = fwd.apply_transpose(u)
+    assert np.array_equal(got, bwd.apply(u))
+    assert rel_l2(got, oracle.kmvm(Y, X, u, **prm)) < 1e-5
+    assert np.array_equal(fwd.apply_transpose(u[:, :1]), got[:, :1])       # the kept transposed lists, one column
+    # one tree: K(X,X) is symmetric, the transposed product is the product
+    sym = ee.Plan(X, None, **prm)
+    assert np.array_equal(sym.apply_transpose(u), sym.apply(u))
+
+
 def test_far_sweeps_match_per_level_interpolation(oracle, monkeypatch):
     """The engine interpolates the points once and moves moments / local expansions between levels;
     F3M_FAR=levels interpolates every level from the points as the reference does

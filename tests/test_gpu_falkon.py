@@ -37,6 +37,15 @@ def test_falkon_matches_closed_form_and_fits():
     mse, mse_ref = float(((pred - Y.double()) ** 2).mean()), float(((pred_ref - Y.double()) ** 2).mean())
     print("prediction vs closed form rel-L2: %.3e, mse %.5f (closed form %.5f), CG iterations %d, CG time %.3fs"
           % (rel, mse, mse_ref, model.cg_iterations_, model.conjugate_gradient_time), flush=True)
+    # the operator of the normal equations, K_nm^T (K_nm v + w), against the dense fp64 one: both engine products
+    # (the second is the transposed product on the same plan) with their 1e-3 bound
+    g = torch.Generator().manual_seed(5)
+    v, w = torch.randn(M, 1, generator=g).cuda(), torch.randn(n, 1, generator=g).cuda()
+    dm = kernel.dmmv(X, C, v, w).double()
+    dm_ref = Knm.T @ (Knm @ v.double() + w.double())
+    rel_dmmv = float((dm - dm_ref).norm() / dm_ref.norm())
+    print("dmmv vs dense fp64: %.3e" % rel_dmmv, flush=True)
+    assert rel_dmmv < 1e-3
     # With lambda = 1e-6 the Nystrom system is ill conditioned: the ~1e-4 relative error of the engine's
     # products moves the coefficients along weakly determined directions, so predictions are compared
     # loosely and the fit itself tightly (the CG + preconditioner arithmetic is pinned against the closed

@@ -442,6 +442,38 @@ def test_far_sweeps_match_per_level_interpolation(eng, monkeypatch, name):
     assert rel_l2(sweeps, per_level) < 5e-6
 
 
+@pytest.mark.parametrize("name", ["clustered_xy", "falkon_shape"])
+def test_transposed_product_on_the_same_plan(eng, oracle, name):
+    """K(X,Y)^T u from the plan of (X, Y) -- trees swapped, every list read from its Y boxes -- against a second
+    plan of (Y, X) (the same lists, kernels and order: the same bits) and against the oracle's product of
+    (Y, X).  Reference: FFM.chunk_forward_transpose, experiments/FFM_classes.py:54-61."""
+    print("case transposed", name, flush=True)
+    rng = np.random.default_rng(24)
+    if name == "falkon_shape":           # many targets against few centres, the kernel wrapper's tree parameters
+        X = (rng.random((30000, 3)) * 2 - 1).astype(f32)
+        Y = X[rng.choice(30000, 400, replace=False)].copy()
+        prm = dict(ls=0.5, min_points=64, nr_of_interpolation=64, small_field_points=64, var_compression=True,
+                   eff_var_limit=0.3)
+    else:
+        X, Y, prm = clouds(name, rng)
+    u = rng.standard_normal((X.shape[0], 3)).astype(f32)
+    fwd, bwd = eng.Plan(dev(X), dev(Y), **prm), eng.Plan(dev(Y), dev(X), **prm)
+    assert fwd.depth == bwd.depth >= 1
+    got = fwd.apply_transpose(dev(u)).cpu().numpy()
+    assert got.shape == (Y.shape[0], 3)
+    assert np.array_equal(got, bwd.apply(dev(u)).cpu().numpy())
+    assert rel_l2(got, oracle.kmvm(Y, X, u, **prm)) < 1e-5
+    exact = oracle.exact_f64(Y, X, u, prm["ls"])
+    assert rel_l2(got, exact) <= 1.5 * rel_l2(oracle.kmvm(Y, X, u, **prm), exact) + 1e-6
+    # the forward product of the same plan is untouched by the transposed lists
+    b = rng.standard_normal((Y.shape[0], 1)).astype(f32)
+    assert np.array_equal(fwd.apply(dev(b)).cpu().numpy(), eng.kmvm(dev(X), dev(Y), dev(b), **prm).cpu().numpy())
+    # no division at all: the exact product, transposed
+    small = eng.Plan(dev(X[:500]), dev(Y[:300]), ls=0.5)
+    assert small.depth == 0
+    assert rel_l2(small.apply_transpose(dev(u[:500])).cpu().numpy(), oracle.exact_f64(Y[:300], X[:500], u[:500], 0.5)) < 1e-5
+
+
 def test_inputs_at_any_four_byte_alignment(eng):
     """Views that start in the middle of an allocation (12-byte rows) are not 16-byte aligned."""
     rng = np.random.default_rng(17)
