@@ -25,6 +25,11 @@ class FalkonOptions(ConjugateGradientOptions):
     # keep T^-1 and A^-1 as dense matrices (two more M x M matrices) so that every triangular solve of
     # the conjugate-gradient loop becomes one matrix-vector product; off: back-substitution each time
     pc_explicit_inverse: bool = True
+    # Preconditioner factorised, multiplied and solved tile by tile in fp32 storage (diagonal tiles in fp64), so
+    # that no library call sees more than pc_block_size^2 entries: None = whenever a matrix in pc_dtype would
+    # exceed the limit for whole-matrix calls (the benchmark's M = 1e5), True = always, False = never
+    pc_blocked: object = None
+    pc_block_size: int = 8192
     use_cpu: bool = False                # kept for signature compatibility; the engine is GPU only
     debug: bool = False
 

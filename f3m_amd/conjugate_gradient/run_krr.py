@@ -25,6 +25,10 @@ def main():
     ap.add_argument("--nodes", type=int, default=64)
     ap.add_argument("--var-compression", action="store_true")
     ap.add_argument("--pc-dtype", default="float64", choices=["float32", "float64"])
+    ap.add_argument("--pc-blocked", default="auto", choices=["auto", "yes", "no"],
+                    help="tile-by-tile fp32 preconditioner (auto: when a whole matrix would exceed the limit for single "
+                         "library calls, as with M = 1e5)")
+    ap.add_argument("--pc-block-size", type=int, default=8192)
     ap.add_argument("--products-only", action="store_true",
                     help="time only the two engine products of one CG iteration (no preconditioner, no solve)")
     args = ap.parse_args()
@@ -33,14 +37,15 @@ def main():
     X = 2 * torch.rand(n, 3, generator=g) - 1
     y = torch.sin(3 * X[:, 0]) * torch.cos(2 * X[:, 1]) + X[:, 2] ** 2 + 0.1 * torch.randn(n, generator=g)
     X, Y = X.cuda(), y[:, None].cuda()
-    opt = FalkonOptions(pc_dtype=getattr(torch, args.pc_dtype))
+    opt = FalkonOptions(pc_dtype=getattr(torch, args.pc_dtype), pc_block_size=args.pc_block_size,
+                        pc_blocked={"auto": None, "yes": True, "no": False}[args.pc_blocked])
     kernel = custom_GaussianKernel(args.ls, opt=opt, var_compression=args.var_compression, interpolation_nr=args.nodes)
     if args.products_only:
         C = X[torch.randperm(n, generator=g)[:m].cuda()].contiguous()
         v = torch.randn(m, 1, generator=g).cuda()
         torch.cuda.synchronize()
         t0 = time.time()
-        kernel.dmmv(X, C, v, None)             # builds both plans, then K_nm v and K_nm^T (.)
+        kernel.dmmv(X, C, v, None)             # builds the plan, then K_nm v and K_nm^T (.)
         torch.cuda.synchronize()
         t_first = time.time() - t0
         times = []
@@ -68,6 +73,7 @@ def main():
                       "preconditioner_s": model.fit_times_[0], "cg_s": model.conjugate_gradient_time,
                       "cg_s_per_iteration": model.conjugate_gradient_time / max(1, model.cg_iterations_),
                       "fit_s": t_fit, "predict_s": t_pred, "mse": mse, "r2": r2,
+                      "gpu_peak_allocated_gib": torch.cuda.max_memory_allocated() / 2 ** 30,
                       "mmv_s": [round(t, 4) for t in model_optimizer_times(model)]}))
 
 

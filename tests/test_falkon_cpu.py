@@ -46,6 +46,66 @@ def test_preconditioned_cg_converges_to_closed_form():
     assert errs[0] > errs[1] > errs[2] and errs[1] < 5e-3 and errs[2] < 1e-7, errs
 
 
+def test_blocked_preconditioner_matches_the_whole_matrix_form():
+    """The tile-by-tile form (fp32 storage, diagonal tiles in fp64; what M = 1e5 centres go through) against the
+    whole-matrix fp64 form on the same centres: factor identities, both factors, every solve."""
+    from f3m_amd.conjugate_gradient.options import FalkonOptions
+    from f3m_amd.conjugate_gradient.preconditioner import BlockedUpperFactor, FalkonPreconditioner
+    torch.manual_seed(1)
+    M, lam, sigma, eps = 1100, 1e-6, 0.5, 1e-5          # 1100 = 4 tiles of 300 with a ragged last one
+    C = 2 * torch.rand(M, 3) - 1
+    k = DenseGaussian(sigma)
+    k.device = "cpu"
+    whole = FalkonPreconditioner(lam, k, FalkonOptions(pc_epsilon_32=eps, pc_blocked=False, pc_explicit_inverse=False)).init(C)
+    blocked = FalkonPreconditioner(lam, k, FalkonOptions(pc_epsilon_32=eps, pc_blocked=True, pc_block_size=300)).init(C)
+    assert blocked.blocked and isinstance(blocked.T, BlockedUpperFactor) and len(blocked.T.tiles) == 4
+    Tb, Ab = blocked.T.dense_upper().double(), blocked.A.dense_upper().double()
+    Kj = k(C, C) + eps * M * torch.eye(M, dtype=torch.float64)
+    # fp32 storage: identities to fp32 accuracy of entries of size <= M eps + 1
+    assert (Tb.T @ Tb - Kj).abs().max() < 2e-5
+    assert (Ab.T @ Ab - (Tb @ Tb.T / M + lam * torch.eye(M, dtype=torch.float64))).abs().max() < 2e-6
+    assert (Tb - whole.T).abs().max() < 1e-4 * whole.T.abs().max()
+    v = torch.randn(M, 2, dtype=torch.float64)
+    for name in ("invT", "invTt", "invA", "invAt", "apply", "apply_t"):
+        got, want = getattr(blocked, name)(v), getattr(whole, name)(v)
+        rel = float((got - want).norm() / want.norm())
+        # the solves amplify the fp32 rounding of the factors by their condition (K_MM + eps M I: up to ~1e4 here)
+        assert rel < 2e-2, (name, rel)
+    # exactness of the solves against the blocked factors themselves (what the CG relies on)
+    for fac, dense in ((blocked.T, Tb), (blocked.A, Ab)):
+        x = fac.solve(v)
+        assert float((dense @ x - v).norm() / v.norm()) < 1e-4
+        xt = fac.solve(v[:, 0], transpose=True)
+        assert xt.shape == (M,) and float((dense.T @ xt - v[:, 0]).norm() / v[:, 0].norm()) < 1e-4
+
+
+def test_blocked_preconditioner_in_the_cg_loop():
+    """FALKON with the tile-by-tile preconditioner against the closed form of the system.  Its triangular solves run
+    in fp32 (as the reference's preconditioner does on fp32 data), and that rounding, amplified by the condition of
+    the factors (~1e5 at lambda = 1e-6), is what limits the agreement; the fp64 whole-matrix form reaches 1e-7."""
+    from f3m_amd.conjugate_gradient.custom_conjugate_gradient_falkon import FalkonConjugateGradient_custom
+    from f3m_amd.conjugate_gradient.options import FalkonOptions
+    from f3m_amd.conjugate_gradient.preconditioner import FalkonPreconditioner
+    torch.manual_seed(0)
+    n, M, lam, sigma, eps = 3000, 150, 1e-6, 0.5, 1e-5
+    X = 2 * torch.rand(n, 3) - 1
+    y = (torch.sin(3 * X[:, 0]) * torch.cos(2 * X[:, 1]) + X[:, 2] ** 2 + 0.1 * torch.randn(n))[:, None].double()
+    k = DenseGaussian(sigma)
+    k.device = "cpu"
+    C = X[torch.randperm(n)[:M]]
+    opt = FalkonOptions(cg_tolerance=1e-13, pc_epsilon_32=eps, pc_blocked=True, pc_block_size=64)
+    pc = FalkonPreconditioner(lam, k, opt).init(C)
+    Knm = k(X, C)
+    H = Knm.T @ Knm + lam * n * (k(C, C) + eps * M * torch.eye(M, dtype=torch.float64))
+    pred_ref = Knm @ torch.linalg.solve(H, Knm.T @ y)
+    cg = FalkonConjugateGradient_custom(k, pc, opt)
+    beta = cg.solve(Knm, None, y, lam, None, 100)
+    pred = Knm @ pc.apply(beta)
+    assert float((pred - pred_ref).norm() / pred_ref.norm()) < 2e-2
+    mse, mse_ref = float(((pred - y) ** 2).mean()), float(((pred_ref - y) ** 2).mean())
+    assert mse < 1.02 * mse_ref
+
+
 def test_options_defaults_are_documented_values():
     from f3m_amd.conjugate_gradient import ConjugateGradientOptions, FalkonOptions
     o = FalkonOptions()

@@ -58,3 +58,45 @@ def test_falkon_matches_closed_form_and_fits():
     Xt, Yt = _problem(5000, seed=9)
     pt = model.predict(Xt).double()
     assert float(((pt - Yt.double()) ** 2).mean()) < 0.03
+
+
+def test_blocked_preconditioner_matches_whole_matrix_form_on_the_gpu():
+    """M = 12000 centres through the tile-by-tile preconditioner (fp32 storage, tiles of 4096, no library call on
+    more than one tile: the form M = 1e5 needs) and through the whole-matrix fp64 form: same solves up to the
+    fp32 rounding amplified by the factors' condition, same quality of the fit."""
+    import torch
+    from f3m_amd.conjugate_gradient import FalkonOptions, custom_Falkon, custom_GaussianKernel
+    from f3m_amd.conjugate_gradient.preconditioner import FalkonPreconditioner
+    print("case falkon blocked preconditioner n=300000 M=12000", flush=True)
+    n, M, lam, sigma = 300000, 12000, 1e-6, 0.5
+    X, Y = _problem(n, seed=2)
+    fits = {}
+    for blocked in (False, True):
+        kernel = custom_GaussianKernel(sigma, var_compression=False, interpolation_nr=64)
+        opt = FalkonOptions(pc_blocked=blocked, pc_block_size=4096)
+        model = custom_Falkon(kernel, lam, M, maxiter=20, seed=3, options=opt)
+        model.fit(X, Y)
+        pred = model.predict(X).double()
+        mse = float(((pred - Y.double()) ** 2).mean())
+        fits[blocked] = (mse, pred, model.ny_points_)
+        print("blocked=%s: mse %.5f, preconditioner %.2fs, CG %.2fs" % (blocked, mse, model.fit_times_[0], model.conjugate_gradient_time), flush=True)
+    assert torch.equal(fits[False][2], fits[True][2])                   # same centres
+    assert fits[True][0] < 1.02 * fits[False][0] + 1e-5
+    rel = float((fits[True][1] - fits[False][1]).norm() / fits[False][1].norm())
+    print("predictions blocked vs whole-matrix: %.3e" % rel, flush=True)
+    assert rel < 2e-2
+    # the factors themselves, on the same centres
+    C = fits[True][2]
+    kernel = custom_GaussianKernel(sigma)
+    whole = FalkonPreconditioner(lam, kernel, FalkonOptions(pc_blocked=False, pc_explicit_inverse=False)).init(C)
+    blk = FalkonPreconditioner(lam, kernel, FalkonOptions(pc_blocked=True, pc_block_size=4096)).init(C)
+    assert blk.blocked and len(blk.T.tiles) == 3
+    Tb = blk.T.dense_upper().double()
+    assert float((Tb - whole.T).abs().max() / whole.T.abs().max()) < 1e-4
+    g = torch.Generator().manual_seed(7)
+    v = torch.randn(M, 1, generator=g, dtype=torch.float64).cuda()
+    for fac, dense in ((blk.T, Tb), (blk.A, blk.A.dense_upper().double())):
+        x = fac.solve(v)
+        assert float((dense @ x - v).norm() / v.norm()) < 1e-3          # each solve inverts its own factor
+        xt = fac.solve(v, transpose=True)
+        assert float((dense.T @ xt - v).norm() / v.norm()) < 1e-3
