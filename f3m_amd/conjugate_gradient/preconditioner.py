@@ -45,7 +45,7 @@ class BlockedUpperFactor:
             D = S[k0:k1, k0:k1].double()
             D = torch.triu(D) + torch.triu(D, 1).T                     # the lower part of S is never read as data
             U = torch.linalg.cholesky(D, upper=True)
-            Ui = torch.linalg.solve_triangular(U, torch.eye(k1 - k0, dtype=torch.float64, device=S.device), upper=True)
+            Ui = FalkonPreconditioner._inverse_upper(U)               # 1024 identity columns per library call
             S[k0:k1, k0:k1] = U.float()
             Ui = Ui.float()
             self.dinv.append(Ui)
