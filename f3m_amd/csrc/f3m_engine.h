@@ -172,7 +172,15 @@ void set_node_offsets(NodeSet &ns, float edge, hipStream_t s);
 void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s);
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
+// ncol (1..4) neighbouring columns at once, one access per row; the scatter adds outs2 (same layout) if it is given
+void gather_columns(const float *b, const int *perm, long long n, int c, int col, int ncol, float *bs, long long bstride,
+                    hipStream_t s);
+void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
+                     int ncol, float *out, hipStream_t s);
 
+// builds the table "box of every 32nd point" of a level now, on stream s, if it does not exist yet (kernels of
+// the near field and of L2P start from it; when those run on different streams the table must exist before)
+void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s);
 // nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride;
 // only_list: no other near list of this level will be applied with this plan
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,

@@ -43,28 +43,64 @@ void gather_points(const float *X, const int *perm, long long n, int d, float *p
     check_launch("gather_points");
 }
 
-__global__ void gather_column_kernel(const float *__restrict__ b, const int *__restrict__ perm, long long n, int c, int col,
-                                     float *__restrict__ bs)
+// Columns col .. col+NC-1 of row perm[i] of b (row-major, c columns) to NC arrays bstride apart: a row sits at a
+// random place, so its NC values are fetched with one load.  VEC: the row slice is read as one vector of NC
+// floats (any 4-byte alignment), else value by value.
+template <int NC>
+__global__ void gather_columns_kernel(const float *__restrict__ b, const int *__restrict__ perm, long long n, int c, int col,
+                                      float *__restrict__ bs, long long bstride)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) bs[i] = b[(long long)perm[i] * c + col];
+    if (i >= n) return;
+    const fvec<NC> row = *reinterpret_cast<const fvec<NC> *>(b + (long long)perm[i] * c + col);
+#pragma unroll
+    for (int q = 0; q < NC; q++) bs[q * bstride + i] = row.v[q];
+}
+void gather_columns(const float *b, const int *perm, long long n, int c, int col, int ncol, float *bs, long long bstride,
+                    hipStream_t s)
+{
+    switch (ncol) {
+    case 1: F3M_LAUNCH((gather_columns_kernel<1>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 2: F3M_LAUNCH((gather_columns_kernel<2>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 3: F3M_LAUNCH((gather_columns_kernel<3>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 4: F3M_LAUNCH((gather_columns_kernel<4>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    default: throw Error(34, "1 to 4 columns at a time");
+    }
+    check_launch("gather_columns");
 }
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s)
 {
-    F3M_LAUNCH(gather_column_kernel, cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs);
-    check_launch("gather_column");
+    gather_columns(b, perm, n, c, col, 1, bs, 0, s);
 }
 
-__global__ void scatter_column_kernel(const float *__restrict__ outs, const int *__restrict__ perm, long long n, int c,
-                                      int col, float *__restrict__ out)
+// out[perm[i]][col + q] = outs[q][i] (+ outs2[q][i] if outs2 is given: the far field's share when it was computed
+// beside the near field), q < NC, one store of NC floats per row
+template <int NC>
+__global__ void scatter_columns_kernel(const float *__restrict__ outs, const float *__restrict__ outs2, long long ostride,
+                                       const int *__restrict__ perm, long long n, int c, int col, float *__restrict__ out)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) out[(long long)perm[i] * c + col] = outs[i];
+    if (i >= n) return;
+    fvec<NC> row;
+#pragma unroll
+    for (int q = 0; q < NC; q++) row.v[q] = outs[q * ostride + i] + (outs2 ? outs2[q * ostride + i] : 0.f);
+    *reinterpret_cast<fvec<NC> *>(out + (long long)perm[i] * c + col) = row;
+}
+void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
+                     int ncol, float *out, hipStream_t s)
+{
+    switch (ncol) {
+    case 1: F3M_LAUNCH((scatter_columns_kernel<1>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
+    case 2: F3M_LAUNCH((scatter_columns_kernel<2>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
+    case 3: F3M_LAUNCH((scatter_columns_kernel<3>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
+    case 4: F3M_LAUNCH((scatter_columns_kernel<4>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
+    default: throw Error(34, "1 to 4 columns at a time");
+    }
+    check_launch("scatter_columns");
 }
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s)
 {
-    F3M_LAUNCH(scatter_column_kernel, cdiv(n, 256), 256, 0, s, outs, perm, n, c, col, out);
-    check_launch("scatter_column");
+    scatter_columns(outs, nullptr, 0, perm, n, c, col, 1, out, s);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -243,6 +279,8 @@ static const int *box_table(const TreeLevel &lev, long long npoints, hipStream_t
     }
     return lev.box32.get();
 }
+
+void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s) { (void)box_table(lev, npoints, s); }
 
 // ------------------------------------------------------------------------------------------------
 // near field (F3M_src/1_d_conv.cu:255-335): out_i += sum over the y boxes listed for the box of i of

@@ -434,6 +434,31 @@ static void finish_stream(hipStream_t s)
     F3M_HIP(hipStreamSynchronize(s));
 }
 
+// A second stream per device, on which the far field of a product runs beside the near field (which is bound
+// by vector-ALU issue and leaves the memory system and the latency-bound far-field kernels room), with the two
+// events that fork it from and join it to the caller's stream.  Default priority, kept for the life of the process.
+#ifndef F3M_CPU_EMU
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+};
+static SideStream &side_stream()
+{
+    static std::mutex mu;
+    static std::map<int, SideStream> per_device;
+    int dev = 0;
+    F3M_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(mu);
+    SideStream &ss = per_device[dev];
+    if (ss.stream == nullptr) {
+        F3M_HIP(hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking));
+        F3M_HIP(hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming));
+        F3M_HIP(hipEventCreateWithFlags(&ss.join, hipEventDisableTiming));
+    }
+    return ss;
+}
+#endif
+
 // out = K(X,Y) b, or with `transposed` out = K(X,Y)^T b (b then has N rows and out M): the same trees
 // with the roles of targets and sources swapped and every list seen from its Y boxes.
 static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s, bool transposed = false)
@@ -466,6 +491,34 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     // F3M_FAR=levels: interpolate every level from the points like the reference (cross-check)
     const char *fe = getenv("F3M_FAR");
     const bool per_level = fe && !strcmp(fe, "levels") && !transposed;
+    // The far field runs on a second stream beside the near field and adds its share when the result is
+    // scattered (F3M_OVERLAP=0: one stream).  Not for a call whose temporaries come from an arena (it would need
+    // one more array of N floats per column) and not for the per-level cross-check.
+    bool overlap = false;
+#ifndef F3M_CPU_EMU
+    {
+        bool any_far = false;
+        for (int k = 1; k <= depth; k++) any_far = any_far || (transposed ? P->levels[k - 1].farT.n : P->levels[k - 1].far.n) > 0;
+        const char *oe = getenv("F3M_OVERLAP");
+        overlap = any_far && !per_level && g_arena == nullptr && !(oe && atoi(oe) == 0);
+    }
+#endif
+    DBuf<float> outs_far;
+    if (overlap) {
+        outs_far.reset((size_t)ostride * width);
+        // The one table that kernels of both streams read has to exist before the streams part: L2P starts from the
+        // box table of the deepest level with far pairs (and of every level with far pairs where the node counts
+        // change between levels, since such levels are evaluated at the points themselves).
+        int ku = 0, kd = 0;
+        bool same_nodes = true;
+        for (int k = 1; k <= depth; k++)
+            if ((transposed ? P->levels[k - 1].farT.n : P->levels[k - 1].far.n) > 0) {
+                if (!ku) ku = k;
+                if (kd && P->levels[k - 1].num_nodes != P->levels[kd - 1].num_nodes) same_nodes = false;
+                kd = k;
+            }
+        for (int k = same_nodes ? kd : ku; k <= kd; k++) ensure_box_table(TX.lev[k], NT, s);
+    }
     for (int col = 0; col < c;) {
         const int left = c - col;
         const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);   // columns of this pass (past `left`: zero weights)
@@ -473,9 +526,23 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         {
             Scope sc(kPerm, s);
             if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
-            for (int q = 0; q < ncol; q++) gather_column(b, TY.perm.get(), NS, c, col + q, bs.get() + q * bstride, s);
+            gather_columns(b, TY.perm.get(), NS, c, col, ncol, bs.get(), bstride, s);
             dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
+            if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
         }
+        std::vector<void *> parked;      // temporaries of the far field, given back once the main stream waits for it
+#ifndef F3M_CPU_EMU
+        if (overlap) {
+            SideStream &ss = side_stream();
+            F3M_HIP(hipEventRecord(ss.fork, s));
+            F3M_HIP(hipStreamWaitEvent(ss.stream, ss.fork, 0));
+            {
+                DeferScope hold(&parked);
+                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs_far.get() + q * ostride, ss.stream);
+            }
+            F3M_HIP(hipEventRecord(ss.join, ss.stream));
+        }
+#endif
         for (int k = 1; k <= depth; k++) {
             // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
             near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
@@ -484,14 +551,21 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 for (int q = 0; q < ncol; q++)
                     far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
         }
-        if (!per_level)
-            for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs.get() + q * ostride, s);
         // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
         near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
                    outs.get(), P->lcs, s, nc, bstride, ostride);
+        // one stream: the far field after the near field, so that either way a result is (near sums) + (far sum)
+        if (!per_level && !overlap)
+            for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs.get() + q * ostride, s);
+#ifndef F3M_CPU_EMU
+        if (overlap) {
+            F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
+            for (void *p : parked) Pool::get().release(p);
+        }
+#endif
         {
             Scope sc(kPerm, s);
-            for (int q = 0; q < ncol; q++) scatter_column(outs.get() + q * ostride, TX.perm.get(), NT, c, col + q, out, s);
+            scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
         }
         col += ncol;
     }

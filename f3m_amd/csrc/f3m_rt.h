@@ -76,6 +76,10 @@ struct Arena {
     const char *owner = "";
 };
 inline thread_local Arena *g_arena = nullptr;
+// While set, blocks given back to the pool are parked in this list instead (DeferScope): work queued on a
+// second stream may still use them, so they return to the pool only once the main stream has been made to wait
+// for that work.
+inline thread_local std::vector<void *> *g_deferred = nullptr;
 struct ArenaScope {
     Arena *prev;
     explicit ArenaScope(Arena *a) : prev(g_arena) { g_arena = a; }
@@ -130,6 +134,7 @@ public:
     void release(void *p)
     {
         if (!p) return;
+        if (g_deferred != nullptr) { g_deferred->push_back(p); return; }
         std::lock_guard<std::mutex> g(mu_);
         auto it = live_.find(p);
         if (it == live_.end()) return;
@@ -155,6 +160,14 @@ private:
     std::map<int, std::multimap<size_t, void *>> free_;
     std::map<void *, Block> live_;
     size_t reserved_ = 0;
+};
+
+struct DeferScope {
+    std::vector<void *> *prev;
+    explicit DeferScope(std::vector<void *> *list) : prev(g_deferred) { g_deferred = list; }
+    ~DeferScope() { g_deferred = prev; }
+    DeferScope(const DeferScope &) = delete;
+    DeferScope &operator=(const DeferScope &) = delete;
 };
 
 template <typename T>
