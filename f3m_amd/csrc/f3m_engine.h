@@ -129,6 +129,8 @@ void gather_tree_points(Tree &t, const float *X, hipStream_t s);
 // the two numbers the kernels left in dstats (boxes, largest count) once the host has fetched them;
 // divide_discard drops a level that turned out not to be needed.
 void divide_launch(Tree &t, int *dstats, hipStream_t s);
+// whether the next divide_launch will first sort more key bits (and thereby replace the key and order arrays)
+bool divide_will_sort(const Tree &t);
 void divide_finish(Tree &t, const int *hstats);
 void divide_discard(Tree &t);
 // The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts and scans (the
@@ -182,10 +184,11 @@ void scatter_columns(const float *outs, const float *outs2, long long ostride, c
 // the near field and of L2P start from it; when those run on different streams the table must exist before)
 void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s);
 // nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride;
-// only_list: no other near list of this level will be applied with this plan
+// only_list: no other near list of this level will be applied with this plan;
+// prepare_only: build the tables of the list that are kept with the plan (tile table, source operands), launch nothing else
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc = 1, long long bstride = 0,
-                long long ostride = 0, bool only_list = false);
+                long long ostride = 0, bool only_list = false, bool prepare_only = false);
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);

@@ -720,7 +720,7 @@ __global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, i
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride,
-                bool only_list)
+                bool only_list, bool prepare_only)
 {
     if (list.n == 0) return;
     F3M_REQUIRE(nc == 1 || nc == 2 || nc == 4, 34, "near field takes 1, 2 or 4 columns at a time");
@@ -819,6 +819,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #undef F3M_CASE
             check_launch("near_operands");
         }
+        if (prepare_only) return;
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
         // Few targets against long lists (the transposed product of a tall kernel matrix): too few work
@@ -870,6 +871,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                        tpw * 32, tileoff.get(), lx.nb, lx.off.get(), outs, ostride);
         }
     } else {
+        if (prepare_only) return;
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
@@ -1978,7 +1980,7 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
         check_launch("p2m");
     }
 #undef F3M_CASE
-    F3M_LAUNCH(p2m_reduce_kernel, cdiv((long long)ly.nb * P, 256), 256, 0, s, partial.get(), tiley.get(), ly.nb, P, mom);
+    F3M_LAUNCH(p2m_reduce_kernel, cdiv((long long)ly.nb * P, 64), 64, 0, s, partial.get(), tiley.get(), ly.nb, P, mom);
     timer_end(s);
     check_launch("p2m_reduce");
 }
@@ -2014,7 +2016,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         if (dtab.size() != (size_t)ntab) {
             require_tables_may_be_built("the M2L tables of a level");
             dtab.reset((size_t)ntab);
-            F3M_LAUNCH(sep_tables_kernel, cdiv(ntab, 256), 256, 0, s, nm, d, NT, kM2LOffsets, ns.dt.get(), edge, (double)lcs, sg,
+            F3M_LAUNCH(sep_tables_kernel, cdiv(ntab, 64), 64, 0, s, nm, d, NT, kM2LOffsets, ns.dt.get(), edge, (double)lcs, sg,
                        dtab.get());
             check_launch("sep_tables");
         }
@@ -2432,7 +2434,9 @@ __global__ void __launch_bounds__(1024) shift_kernel(const float *__restrict__ t
 // The same transfer for the 4 x 4 x 4 grid on both levels: one wavefront per parent box, lane = node
 // (a0 + 4 a1 + 16 a2); the three 4 x 4 factors are applied with exchanges inside the wavefront (groups of
 // four lanes, lanes 4 apart, lanes 16 apart), no LDS traffic besides the 96-entry table, no barriers.
-constexpr int kShiftQWaves = 4;
+// (workgroups of one wavefront: the far field runs beside the near field, whose wavefronts keep the compute
+// units full, and only small workgroups find room there)
+constexpr int kShiftQWaves = 1;
 
 template <bool DOWN>
 __global__ void __launch_bounds__(kShiftQWaves * 64) shift_q64_kernel(const float *__restrict__ tables, int nbp,
@@ -2504,7 +2508,7 @@ void make_shift_tables(const NodeSet &nsp, const NodeSet &nsc, DBuf<float> &tab,
     ShiftMeta sm = shift_meta(nsp, nsc);
     const int ntab = nsp.d * 2 * sm.NTp * sm.NTc;
     tab.reset((size_t)ntab);
-    F3M_LAUNCH(shift_tables_kernel, cdiv(ntab, 256), 256, 0, s, sm, nsp.d, meta_of(nsp), meta_of(nsc), nsp.dt.get(),
+    F3M_LAUNCH(shift_tables_kernel, cdiv(ntab, 64), 64, 0, s, sm, nsp.d, meta_of(nsp), meta_of(nsc), nsp.dt.get(),
                nsp.dw.get(), nsc.dt.get(), tab.get());
     check_launch("shift_tables");
 }

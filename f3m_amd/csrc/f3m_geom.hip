@@ -540,6 +540,12 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
     }
 }
 
+bool divide_will_sort(const Tree &t)
+{
+    const int k = (int)t.lev.size();
+    return t.geo.d * (t.geo.L - k) < t.sorted_from;
+}
+
 void divide_launch(Tree &t, int *dstats, hipStream_t s)
 {
     const int d = t.geo.d;

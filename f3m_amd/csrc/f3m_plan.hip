@@ -92,6 +92,10 @@ struct f3m_plan {
     std::vector<PlanLevel> levels;         // levels[k-1] = depth k
     std::map<int, std::unique_ptr<NodeSet>> nodes;
     DBuf<float> Xraw, Yraw;                // row-major copies, only when no division happened
+    // one-shot products: the first column group of b, already in sorted order (gathered while the lists were built)
+    DBuf<float> early_bs;
+    const float *early_b = nullptr;
+    int early_c = 0, early_ncol = 0;
     std::map<std::pair<int, int>, std::unique_ptr<DBuf<float>>> shift_tabs;   // (parent nodes, child nodes)
     const float *shift_table(int nodes_parent, int nodes_child, hipStream_t s)
     {
@@ -171,8 +175,35 @@ static ClassifyParams classify_params(const f3m_plan &P, float edge)
     return cp;
 }
 
+// A second stream per device, on which the far field of a product runs beside the near field (which is bound
+// by vector-ALU issue and leaves the memory system and the latency-bound far-field kernels room), with the two
+// events that fork it from and join it to the caller's stream.  Default priority, kept for the life of the process.
+#ifndef F3M_CPU_EMU
+struct SideStream {
+    hipStream_t stream = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr;
+};
+static SideStream &side_stream()
+{
+    static std::mutex mu;
+    static std::map<int, SideStream> per_device;
+    int dev = 0;
+    F3M_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(mu);
+    SideStream &ss = per_device[dev];
+    if (ss.stream == nullptr) {
+        F3M_HIP(hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking));
+        F3M_HIP(hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming));
+        F3M_HIP(hipEventCreateWithFlags(&ss.join, hipEventDisableTiming));
+    }
+    return ss;
+}
+#endif
+
+// b_early (nullable, with c_early columns): the weights of the product that will follow at once (f3m_kmvm_f32);
+// their first column group is put into sorted order while the lists are built.
 static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y, long long M, const f3m_params *prm,
-                             hipStream_t s)
+                             hipStream_t s, const float *b_early = nullptr, int c_early = 0)
 {
     bool sym = (Y == nullptr || Y == X);
     check_params(d, N, M, sym, prm);
@@ -264,7 +295,48 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         divide_finish(P->tx, hres + 8);
         if (!sym) divide_finish(P->ty_, hres + 10);
     };
+    // The points (and the weights of a one-shot product) are moved into sorted order on the second stream while the
+    // levels and lists are built here: those are many small kernels that leave the memory system idle, the moves are
+    // bound by it.  The order of the first sort is final unless a deep level asks for more key bits to be sorted
+    // (divide_launch); then the moves wait for that and are done again at the end.
+    bool early = false;
+    int early_from_x = 0, early_from_y = 0;
+#ifndef F3M_CPU_EMU
+    if (need_tree && wants_division() && g_arena == nullptr && !(getenv("F3M_OVERLAP") && atoi(getenv("F3M_OVERLAP")) == 0)) {
+        SideStream &ss = side_stream();
+        F3M_HIP(hipEventRecord(ss.fork, s));
+        F3M_HIP(hipStreamWaitEvent(ss.stream, ss.fork, 0));
+        gather_tree_points(P->tx, X, ss.stream);
+        if (!sym) gather_tree_points(P->ty_, Y, ss.stream);
+        if (b_early != nullptr && c_early >= 1) {
+            const long long bstride = P->M + 32;
+            P->early_ncol = c_early >= 3 ? std::min(c_early, 4) : c_early;
+            const int nc = c_early >= 3 ? 4 : c_early;
+            P->early_bs.reset((size_t)bstride * (c_early >= 2 ? 4 : 1));
+            if (nc > P->early_ncol) dev_fill(P->early_bs.get(), 0, sizeof(float) * (size_t)bstride * nc, ss.stream);
+            gather_columns(b_early, P->ty->perm.get(), P->M, c_early, 0, P->early_ncol, P->early_bs.get(), bstride, ss.stream);
+            P->early_b = b_early;
+            P->early_c = c_early;
+        }
+        F3M_HIP(hipEventRecord(ss.join, ss.stream));
+        early = true;
+        early_from_x = P->tx.sorted_from;
+        early_from_y = P->ty->sorted_from;
+    }
+    // before a division sorts more key bits (which replaces the order arrays the moves read), the moves must be done
+    auto settle_early = [&]() {
+        if (early && (divide_will_sort(P->tx) || (!sym && divide_will_sort(P->ty_)))) {
+            F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
+            early = false;
+            P->early_b = nullptr;
+            P->early_bs.free();
+        }
+    };
+#else
+    auto settle_early = [&]() {};
+#endif
     if (need_tree && wants_division()) {
+        settle_early();
         start_division();
         fetch_level(nullptr, true);
         finish_division();
@@ -277,7 +349,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             ListsPending pend;
             lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
             const bool ahead = wants_division();
-            if (ahead) start_division();
+            if (ahead) { settle_early(); start_division(); }
             fetch_level(&pend, ahead);
             F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
@@ -298,7 +370,13 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             break;
         }
     }
-    if (need_tree) {
+#ifndef F3M_CPU_EMU
+    if (early) {
+        F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));       // the moves of the second stream are part of the plan
+        (void)early_from_x; (void)early_from_y;
+    }
+#endif
+    if (need_tree && !early) {
         gather_tree_points(P->tx, X, s);
         if (!sym) gather_tree_points(P->ty_, Y, s);
     }
@@ -434,31 +512,6 @@ static void finish_stream(hipStream_t s)
     F3M_HIP(hipStreamSynchronize(s));
 }
 
-// A second stream per device, on which the far field of a product runs beside the near field (which is bound
-// by vector-ALU issue and leaves the memory system and the latency-bound far-field kernels room), with the two
-// events that fork it from and join it to the caller's stream.  Default priority, kept for the life of the process.
-#ifndef F3M_CPU_EMU
-struct SideStream {
-    hipStream_t stream = nullptr;
-    hipEvent_t fork = nullptr, join = nullptr;
-};
-static SideStream &side_stream()
-{
-    static std::mutex mu;
-    static std::map<int, SideStream> per_device;
-    int dev = 0;
-    F3M_HIP(hipGetDevice(&dev));
-    std::lock_guard<std::mutex> g(mu);
-    SideStream &ss = per_device[dev];
-    if (ss.stream == nullptr) {
-        F3M_HIP(hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking));
-        F3M_HIP(hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming));
-        F3M_HIP(hipEventCreateWithFlags(&ss.join, hipEventDisableTiming));
-    }
-    return ss;
-}
-#endif
-
 // out = K(X,Y) b, or with `transposed` out = K(X,Y)^T b (b then has N rows and out M): the same trees
 // with the roles of targets and sources swapped and every list seen from its Y boxes.
 static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream_t s, bool transposed = false)
@@ -525,48 +578,68 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
-            if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
-            gather_columns(b, TY.perm.get(), NS, c, col, ncol, bs.get(), bstride, s);
+            if (col == 0 && !transposed && P->early_b == b && P->early_c == c && P->early_ncol == ncol && P->early_bs.size() > 0) {
+                std::swap(bs, P->early_bs);                 // this group's weights were put in order while the plan was built
+                P->early_b = nullptr;
+                P->early_bs.free();
+            } else {
+                if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
+                gather_columns(b, TY.perm.get(), NS, c, col, ncol, bs.get(), bstride, s);
+            }
             dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
             if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
         }
-        std::vector<void *> parked;      // temporaries of the far field, given back once the main stream waits for it
-#ifndef F3M_CPU_EMU
-        if (overlap) {
-            SideStream &ss = side_stream();
-            F3M_HIP(hipEventRecord(ss.fork, s));
-            F3M_HIP(hipStreamWaitEvent(ss.stream, ss.fork, 0));
-            {
-                DeferScope hold(&parked);
-                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs_far.get() + q * ostride, ss.stream);
-            }
-            F3M_HIP(hipEventRecord(ss.join, ss.stream));
-        }
-#endif
-        for (int k = 1; k <= depth; k++) {
-            // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
-            near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
-                       bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0);
-            if (per_level)
-                for (int q = 0; q < ncol; q++)
-                    far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
-        }
-        // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
-        near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
-                   outs.get(), P->lcs, s, nc, bstride, ostride);
-        // one stream: the far field after the near field, so that either way a result is (near sums) + (far sum)
-        if (!per_level && !overlap)
-            for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, outs.get() + q * ostride, s);
-#ifndef F3M_CPU_EMU
-        if (overlap) {
-            F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
-            for (void *p : parked) Pool::get().release(p);
-        }
-#endif
+        // Every temporary that is given back while this column group is being queued is parked until the streams
+        // have joined: work queued on one stream may still use a block when host code of the other asks for memory.
+        std::vector<void *> parked;
         {
+            DeferScope hold(&parked);
+#ifndef F3M_CPU_EMU
+            if (overlap) {
+                // The near field's own tables first (kept with the plan from then on), so that its long launches
+                // follow without delay; the streams part after that: the far field then runs beside those launches.
+                for (int k = 1; k <= depth; k++)
+                    near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc, bstride,
+                               ostride, /*only_list=*/k < depth || keep_of(depth).n == 0, /*prepare_only=*/true);
+                near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(), outs.get(), P->lcs, s, nc,
+                           bstride, ostride, false, /*prepare_only=*/true);
+                F3M_HIP(hipEventRecord(side_stream().fork, s));
+                F3M_HIP(hipStreamWaitEvent(side_stream().stream, side_stream().fork, 0));
+            }
+#endif
+            // the near field first: it is the long pole, and the host needs a while to queue the far field's many
+            // small kernels
+            for (int k = 1; k <= depth; k++) {
+                // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
+                near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
+                           bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0);
+                if (per_level)
+                    for (int q = 0; q < ncol; q++)
+                        far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
+            }
+            // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
+            near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
+                       outs.get(), P->lcs, s, nc, bstride, ostride);
+            // the far field: beside the near field on the second stream into its own array, or after it on the one
+            // stream; either way a result is (near sums) + (far sum)
+            if (!per_level) {
+                hipStream_t fs = s;
+                float *fo = outs.get();
+#ifndef F3M_CPU_EMU
+                if (overlap) { fs = side_stream().stream; fo = outs_far.get(); }
+#endif
+                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs);
+            }
+#ifndef F3M_CPU_EMU
+            if (overlap) {
+                F3M_HIP(hipEventRecord(side_stream().join, side_stream().stream));
+                F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
+            }
+#endif
             Scope sc(kPerm, s);
             scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
         }
+        for (void *p : parked) Pool::get().release(p);
         col += ncol;
     }
     finish_stream(s);
@@ -603,7 +676,7 @@ int f3m_kmvm_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, co
     return guarded([&] {
         hipStream_t s = (hipStream_t)stream;
         g_timer.reset();
-        std::unique_ptr<f3m_plan> P(plan_create(d, X, N, Y, M, params, s));
+        std::unique_ptr<f3m_plan> P(plan_create(d, X, N, Y, M, params, s, b, c));
         plan_apply(P.get(), b, c, out, s);
         g_timer.collect();
     });

@@ -358,8 +358,9 @@ inline void dev_fill(void *p, int byte, size_t bytes, hipStream_t s)
     if ((reinterpret_cast<uintptr_t>(p) | bytes) & 3) throw Error(104, "fill of a range that is not a multiple of 4 bytes");
     const unsigned b = (unsigned)byte & 255u, word = b * 0x01010101u;
     const size_t n32 = bytes / 4;
-    const unsigned grid = (unsigned)std::min<size_t>((n32 + 255) / 256, 8192);
-    F3M_LAUNCH((fill_words_kernel<256>), grid, 256, 0, s, static_cast<unsigned *>(p), n32, word);
+    // workgroups of one wavefront: they find room beside a kernel that keeps the compute units full
+    const unsigned grid = (unsigned)std::min<size_t>((n32 + 63) / 64, 32768);
+    F3M_LAUNCH((fill_words_kernel<64>), grid, 64, 0, s, static_cast<unsigned *>(p), n32, word);
     check_launch("fill");
 }
 
