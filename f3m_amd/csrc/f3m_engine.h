@@ -183,6 +183,8 @@ void scatter_columns(const float *outs, const float *outs2, long long ostride, c
 // builds the table "box of every 32nd point" of a level now, on stream s, if it does not exist yet (kernels of
 // the near field and of L2P start from it; when those run on different streams the table must exist before)
 void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s);
+// the near field's source operands of every box of a level, ahead of its use (kept with the level)
+void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs, hipStream_t s);
 // nc = 1 or 4 right-hand sides at a time: columns of bs are bstride floats apart, those of outs ostride;
 // only_list: no other near list of this level will be applied with this plan;
 // prepare_only: build the tables of the list that are kept with the plan (tile table, source operands), launch nothing else

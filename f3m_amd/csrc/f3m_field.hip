@@ -718,6 +718,61 @@ __global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, i
     }
 }
 
+// whether the near field of a level goes to the matrix-pipe kernel (see near_field)
+static bool near_on_matrix_pipe(int d, float lcs, float edge)
+{
+    const float sc_edge = sqrtf(lcs * kLog2e) * edge;
+    bool use_mfma = 30.f * (float)d * sc_edge * sc_edge <= 1200.f;
+    if (const char *env = getenv("F3M_NEAR")) use_mfma = !strcmp(env, "mfma") ? true : (!strcmp(env, "valu") ? false : use_mfma);
+    return use_mfma;
+}
+
+// The split-f16 source operands of a level, kept with it.  only (nullable): operands are needed for the source boxes
+// of this list alone (at most levels a small part of the boxes); otherwise for every box.
+static void build_near_operands(int d, const Tree &ty, const TreeLevel &ly, float sc, const PairList *only, hipStream_t s)
+{
+    const bool only_list = only != nullptr;
+    if (ly.nearops.size() != 0 && ly.nearops_sc == sc && !(ly.nearops_partial && !only_list)) return;
+    const int NS = near_insts(d);
+    const long long stride = ty.n + 32;
+    require_tables_may_be_built("the near-field source operands of a level");
+    ly.nearops.reset((size_t)NS * 2 * stride * 16);
+    ly.nearops_sc = sc;
+    ly.nearops_partial = only_list;
+    DBuf<int> need;
+    if (only_list) {
+        DBuf<int> fy((size_t)ly.nb);
+        dev_fill(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s);
+        F3M_LAUNCH(mark_cols_kernel, cdiv(only->n, 256), 256, 0, s, only->pairs.get(), only->n, fy.get());
+        check_launch("mark_cols");
+        need.reset((size_t)ly.nb + 1);
+        exclusive_scan_i32(fy.get(), ly.nb, need.get(), s);
+    }
+    const int *box32 = box_table(ly, ty.n, s);
+#define F3M_CASE(DD)                                                                                                  \
+    case DD:                                                                                                          \
+        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
+                   ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
+                   only_list ? need.get() : (const int *)nullptr, box32,                                              \
+                   reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
+    check_launch("near_operands");
+}
+
+// The operands of every box of a level, ahead of the near field (the plan calls this for its deepest level, beside
+// the kernels that build that level's lists); nothing happens where the near field would take the all-vector kernel.
+void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs, hipStream_t s)
+{
+    if (!near_on_matrix_pipe(d, lcs, ly.edge)) return;
+    build_near_operands(d, ty, ly, sqrtf(lcs * kLog2e), nullptr, s);
+}
+
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride,
                 bool only_list, bool prepare_only)
@@ -733,9 +788,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // i.e. a relative error of a term below 3e-5 (box edge up to ~3.6 lengthscales in 3-D; the N(0,I) cloud
     // with ls = 0.1 has the same error against the fp64 product, 1.3968e-3, with either kernel at every
     // level), otherwise the all-vector kernel.  F3M_NEAR=valu|mfma overrides the choice.
-    const float sc_edge = sqrtf(lcs * kLog2e) * lx.edge;
-    bool use_mfma = 30.f * (float)d * sc_edge * sc_edge <= 1200.f;
-    if (const char *env = getenv("F3M_NEAR")) use_mfma = !strcmp(env, "mfma") ? true : (!strcmp(env, "valu") ? false : use_mfma);
+    const bool use_mfma = near_on_matrix_pipe(d, lcs, lx.edge);
     constexpr int T = 1;
     // all-vector kernel: whole boxes per workgroup where possible (multiple of the wave size, <= 512 lanes)
     int bd = ((lx.maxcount + kWave - 1) / kWave) * kWave;
@@ -785,40 +838,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     if (use_mfma && items_exact >= 0) ntiles = (int)std::max<long long>(1, items_exact);
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
-        const int NS = near_insts(d);
         const long long stride = ty.n + 32;
-        // The operands of a level are kept in the plan.  only_list: this list is the only near list of
-        // its level, so operands are needed for its source boxes only (at most levels a small part).
-        if (ly.nearops.size() == 0 || ly.nearops_sc != sc || (ly.nearops_partial && !only_list)) {
-            require_tables_may_be_built("the near-field source operands of a level");
-            ly.nearops.reset((size_t)NS * 2 * stride * 16);
-            ly.nearops_sc = sc;
-            ly.nearops_partial = only_list;
-            DBuf<int> need;
-            if (only_list) {
-                DBuf<int> fy((size_t)ly.nb);
-                dev_fill(fy.get(), 0, sizeof(int) * (size_t)ly.nb, s);
-                F3M_LAUNCH(mark_cols_kernel, cdiv(list.n, 256), 256, 0, s, list.pairs.get(), list.n, fy.get());
-                check_launch("mark_cols");
-                need.reset((size_t)ly.nb + 1);
-                exclusive_scan_i32(fy.get(), ly.nb, need.get(), s);
-            }
-            const int *box32 = box_table(ly, ty.n, s);
-#define F3M_CASE(DD)                                                                                                  \
-    case DD:                                                                                                          \
-        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
-                   ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
-                   only_list ? need.get() : (const int *)nullptr, box32,                                              \
-                   reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
-        break;
-            switch (d) {
-                F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
-                F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
-            default: throw Error(2, "dimension must be 1..10");
-            }
-#undef F3M_CASE
-            check_launch("near_operands");
-        }
+        build_near_operands(d, ty, ly, sc, only_list ? &list : nullptr, s);
         if (prepare_only) return;
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid

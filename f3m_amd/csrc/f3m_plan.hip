@@ -300,7 +300,9 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // bound by it.  The order of the first sort is final unless a deep level asks for more key bits to be sorted
     // (divide_launch); then the moves wait for that and are done again at the end.
     bool early = false;
-    int early_from_x = 0, early_from_y = 0;
+    // While work is queued on both streams, blocks that host code gives back are parked (a kernel of the other stream
+    // may still use them, and the pool would hand them to the next request); they return to the pool at the end.
+    ParkingLot lot;
 #ifndef F3M_CPU_EMU
     if (need_tree && wants_division() && g_arena == nullptr && !(getenv("F3M_OVERLAP") && atoi(getenv("F3M_OVERLAP")) == 0)) {
         SideStream &ss = side_stream();
@@ -318,14 +320,13 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             P->early_b = b_early;
             P->early_c = c_early;
         }
-        F3M_HIP(hipEventRecord(ss.join, ss.stream));
         early = true;
-        early_from_x = P->tx.sorted_from;
-        early_from_y = P->ty->sorted_from;
+        lot.start();
     }
     // before a division sorts more key bits (which replaces the order arrays the moves read), the moves must be done
     auto settle_early = [&]() {
         if (early && (divide_will_sort(P->tx) || (!sym && divide_will_sort(P->ty_)))) {
+            F3M_HIP(hipEventRecord(side_stream().join, side_stream().stream));
             F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
             early = false;
             P->early_b = nullptr;
@@ -350,6 +351,12 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
             const bool ahead = wants_division();
             if (ahead) { settle_early(); start_division(); }
+#ifndef F3M_CPU_EMU
+            // No further division: this is the deepest level, whose near lists will be summed.  Its source operands
+            // are prepared on the second stream (behind the moves of the points) while its lists are built here.
+            // (The host has seen the counts of this level's division, so the level's arrays are complete.)
+            if (!ahead && early) prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
+#endif
             fetch_level(&pend, ahead);
             F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
@@ -372,8 +379,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     }
 #ifndef F3M_CPU_EMU
     if (early) {
-        F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));       // the moves of the second stream are part of the plan
-        (void)early_from_x; (void)early_from_y;
+        F3M_HIP(hipEventRecord(side_stream().join, side_stream().stream));
+        F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));       // the work of the second stream is part of the plan
     }
 #endif
     if (need_tree && !early) {
@@ -591,9 +598,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         }
         // Every temporary that is given back while this column group is being queued is parked until the streams
         // have joined: work queued on one stream may still use a block when host code of the other asks for memory.
-        std::vector<void *> parked;
         {
-            DeferScope hold(&parked);
+            ParkingLot lot;
+            lot.start();
 #ifndef F3M_CPU_EMU
             if (overlap) {
                 // The near field's own tables first (kept with the plan from then on), so that its long launches
@@ -639,7 +646,6 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             Scope sc(kPerm, s);
             scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
         }
-        for (void *p : parked) Pool::get().release(p);
         col += ncol;
     }
     finish_stream(s);

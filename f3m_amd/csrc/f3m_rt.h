@@ -76,7 +76,7 @@ struct Arena {
     const char *owner = "";
 };
 inline thread_local Arena *g_arena = nullptr;
-// While set, blocks given back to the pool are parked in this list instead (DeferScope): work queued on a
+// While set, blocks given back to the pool are parked in this list instead (ParkingLot): work queued on a
 // second stream may still use them, so they return to the pool only once the main stream has been made to wait
 // for that work.
 inline thread_local std::vector<void *> *g_deferred = nullptr;
@@ -162,13 +162,33 @@ private:
     size_t reserved_ = 0;
 };
 
-struct DeferScope {
-    std::vector<void *> *prev;
-    explicit DeferScope(std::vector<void *> *list) : prev(g_deferred) { g_deferred = list; }
-    ~DeferScope() { g_deferred = prev; }
-    DeferScope(const DeferScope &) = delete;
-    DeferScope &operator=(const DeferScope &) = delete;
+// Parks the blocks that the calling thread gives back between start() and the end of the object's life, and
+// returns them to the pool then (also when an exception ends the scope).
+class ParkingLot {
+public:
+    ParkingLot() = default;
+    ParkingLot(const ParkingLot &) = delete;
+    ParkingLot &operator=(const ParkingLot &) = delete;
+    void start()
+    {
+        if (active_) return;
+        prev_ = g_deferred;
+        g_deferred = &held_;
+        active_ = true;
+    }
+    ~ParkingLot();
+
+private:
+    std::vector<void *> held_, *prev_ = nullptr;
+    bool active_ = false;
 };
+
+inline ParkingLot::~ParkingLot()
+{
+    if (!active_) return;
+    g_deferred = prev_;
+    for (void *p : held_) Pool::get().release(p);
+}
 
 template <typename T>
 class DBuf {
