@@ -129,6 +129,12 @@ void gather_tree_points(Tree &t, const float *X, hipStream_t s);
 // the two numbers the kernels left in dstats (boxes, largest count) once the host has fetched them;
 // divide_discard drops a level that turned out not to be needed.
 void divide_launch(Tree &t, int *dstats, hipStream_t s);
+// Levels whose boxes the sorted key bits resolve; the count of the fullest cell at that depth (added to *dout by
+// atomicMax, *dout zero before): if it exceeds the division threshold the tree will go deeper than the sorted bits
+// reach, and sort_more_bits (eight more key bits; the levels built so far stay valid) is due sooner or later.
+int sorted_levels(const Tree &t);
+void max_run_launch(const Tree &t, int *dout, hipStream_t s);
+void sort_more_bits(Tree &t, hipStream_t s);
 // whether the next divide_launch will first sort more key bits (and thereby replace the key and order arrays)
 bool divide_will_sort(const Tree &t);
 void divide_finish(Tree &t, const int *hstats);

@@ -540,6 +540,41 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
     }
 }
 
+// Count of the fullest cell of the grid that the leading `bits` key bits resolve, added to *out by atomicMax (the
+// caller keeps *out zero).  One thread per cell: the range of its keys by two binary searches in the sorted keys.
+__global__ void max_run_kernel(const uint32_t *__restrict__ keys, long long n, int shift, unsigned ncell, int *__restrict__ out)
+{
+    const unsigned p = blockIdx.x * blockDim.x + threadIdx.x;
+    if (p >= ncell) return;
+    auto lower = [&](unsigned q) {                   // first index whose prefix is >= q
+        long long lo = 0, hi = n;
+        while (lo < hi) {
+            const long long mid = lo + ((hi - lo) >> 1);
+            if ((keys[mid] >> shift) < q) lo = mid + 1; else hi = mid;
+        }
+        return lo;
+    };
+    const long long cnt = lower(p + 1) - lower(p);
+    if (cnt > 0) atomicMax(out, (int)cnt);
+}
+
+int sorted_levels(const Tree &t) { return (t.geo.d * t.geo.L - t.sorted_from) / t.geo.d; }
+
+void max_run_launch(const Tree &t, int *dout, hipStream_t s)
+{
+    const int bits = t.geo.d * sorted_levels(t), shift = t.geo.d * t.geo.L - bits;     // bits <= 16
+    const unsigned ncell = 1u << bits;
+    F3M_LAUNCH(max_run_kernel, cdiv(ncell, 256), 256, 0, s, t.keys.get(), t.n, shift, ncell, dout);
+    check_launch("max_run");
+}
+
+void sort_more_bits(Tree &t, hipStream_t s)
+{
+    if (t.sorted_from == 0) return;
+    t.sorted_from = std::max(0, t.sorted_from - 8);
+    radix_sort(t.keys, t.perm, t.n, t.sorted_from, t.geo.d * t.geo.L, s);
+}
+
 bool divide_will_sort(const Tree &t)
 {
     const int k = (int)t.lev.size();

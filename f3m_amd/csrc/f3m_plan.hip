@@ -276,6 +276,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             L.add(dres.get() + 12, 2, 12, true);
         }
         if (division) L.add(dres.get() + 8, sym ? 2 : 4, 8, true);
+        if (division && pend == nullptr) L.add(dres.get() + 14, 2, 14, true);      // first division: fullest sorted cells
         if (L.nseg > 0) fetch_segments(L, hres, s);
     };
     // row statistics of the small and keep lists, 8 words per level; nothing at plan time depends on
@@ -304,7 +305,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // may still use them, and the pool would hand them to the next request); they return to the pool at the end.
     ParkingLot lot;
 #ifndef F3M_CPU_EMU
-    if (need_tree && wants_division() && g_arena == nullptr && !(getenv("F3M_OVERLAP") && atoi(getenv("F3M_OVERLAP")) == 0)) {
+    const bool two_streams = g_arena == nullptr && !(getenv("F3M_OVERLAP") && atoi(getenv("F3M_OVERLAP")) == 0);
+    auto start_early_moves = [&]() {
         SideStream &ss = side_stream();
         F3M_HIP(hipEventRecord(ss.fork, s));
         F3M_HIP(hipStreamWaitEvent(ss.stream, ss.fork, 0));
@@ -322,7 +324,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         }
         early = true;
         lot.start();
-    }
+    };
     // before a division sorts more key bits (which replaces the order arrays the moves read), the moves must be done
     auto settle_early = [&]() {
         if (early && (divide_will_sort(P->tx) || (!sym && divide_will_sort(P->ty_)))) {
@@ -339,8 +341,26 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     if (need_tree && wants_division()) {
         settle_early();
         start_division();
+#ifndef F3M_CPU_EMU
+        // with the first division's counts, the fullest cell at the depth that the sorted key bits resolve
+        // (words [14], [15] of the record)
+        if (two_streams) {
+            max_run_launch(P->tx, dres.get() + 14, s);
+            if (!sym) max_run_launch(P->ty_, dres.get() + 15, s);
+        }
+#endif
         fetch_level(nullptr, true);
         finish_division();
+#ifndef F3M_CPU_EMU
+        if (two_streams) {
+            // A tree whose fullest cell at that depth still calls for division will need more key bits sorted: now,
+            // rather than in the middle of the level loop, so that the order of the points is final from here on
+            // (deeper trees than that sort again later, and the moves below are then repeated).
+            if ((float)hres[14] > prm->min_points) sort_more_bits(P->tx, s);
+            if (!sym && (float)hres[15] > prm->min_points) sort_more_bits(P->ty_, s);
+            start_early_moves();
+        }
+#endif
         for (;;) {
             const int k = (int)P->tx.lev.size() - 1;
             const float e = P->tx.lev[k].edge;

@@ -474,6 +474,31 @@ def test_transposed_product_on_the_same_plan(eng, oracle, name):
     assert rel_l2(small.apply_transpose(dev(u[:500])).cpu().numpy(), oracle.exact_f64(Y[:300], X[:500], u[:500], 0.5)) < 1e-5
 
 
+def test_repeated_products_have_the_same_bits(eng):
+    """One-shot products and plan products of clouds of very different sizes, interleaved and repeated: every
+    repetition must give the bits of the first.  The library queues work on two streams and recycles its device
+    buffers between them; a buffer handed out while a kernel of the other stream still uses it would show up here
+    (on small clouds every cached buffer fits every request)."""
+    import golden_fixtures as gf
+    print("case repeated products", flush=True)
+    fx = gf.load()
+    rng = np.random.default_rng(41)
+    cases = []
+    for name in ("d2_normal", "d3_two_trees", "d5_slab_243nodes_far"):
+        X, Y, b, prm = gf.case(fx, name)
+        cases.append((dev(X), None if Y is None else dev(Y), dev(b), prm))
+    Xm = rng.random((200000, 3), dtype=f32)
+    cases.append((dev(Xm), None, dev(rng.standard_normal((200000, 3)).astype(f32)), dict(ls=0.3)))
+    Xa, Ya = rng.standard_normal((50000, 3)).astype(f32), rng.random((3000, 3), dtype=f32)
+    cases.append((dev(Xa), dev(Ya), dev(rng.standard_normal((3000, 1)).astype(f32)), dict(ls=0.5, min_points=200)))
+    first = [eng.kmvm(X, Y, b, **prm).cpu().numpy() for X, Y, b, prm in cases]
+    plans = [eng.Plan(X, Y, **prm) for X, Y, b, prm in cases]
+    for rep in range(6):
+        for i, (X, Y, b, prm) in enumerate(cases):
+            assert np.array_equal(eng.kmvm(X, Y, b, **prm).cpu().numpy(), first[i]), (rep, i, "one-shot")
+            assert np.array_equal(plans[i].apply(b).cpu().numpy(), first[i]), (rep, i, "plan")
+
+
 def test_inputs_at_any_four_byte_alignment(eng):
     """Views that start in the middle of an allocation (12-byte rows) are not 16-byte aligned."""
     rng = np.random.default_rng(17)
