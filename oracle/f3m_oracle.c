@@ -24,6 +24,7 @@
  *                                                    pair is far; rel-L2 vs fp64 exact; linearity)
  *   var_compression classification ................. pinned (independent numpy restatement of the
  *                                                    predicates, brute force over all box pairs)
+ *   sums for selected target rows (rowsel) ......... pinned (bit-equal to the unrestricted sums on those rows)
  */
 #include <math.h>
 #include <stdint.h>

@@ -114,3 +114,37 @@ def test_error_decreases_with_node_count_and_linearity(oracle):
     assert np.allclose(o[:, :1], o0, rtol=0, atol=0)     # columns are independent
     o2 = plan.apply(2.0 * b[:, :1] + b[:, 1:])
     assert oracle.rel_l2(o2, 2.0 * o[:, :1].astype(np.float64) + o[:, 1:]) < 1e-5
+
+
+def test_sums_restricted_to_selected_rows_are_the_unrestricted_sums(oracle):
+    """`rows=`: the same sums for some target rows only (M2L only for the boxes that hold one of them).  Used by
+    the GPU tests on clouds whose complete M2L would keep a CPU busy for minutes; on a cloud small enough for both,
+    the restricted results must have the bits of the unrestricted ones on those rows and be zero elsewhere."""
+    rng = np.random.default_rng(6)
+    X = rng.random((5000, 3)).astype(f32)
+    Y = rng.random((3000, 3)).astype(f32)
+    b = rng.standard_normal((3000, 2)).astype(f32)
+    plan = oracle.Plan(X, Y, ls=0.5, min_points=100, nr_of_interpolation=27, small_field_points=60)
+    assert plan.nlevels >= 2
+    rows = np.unique(rng.integers(0, 5000, 300))
+    others = np.setdiff1d(np.arange(5000), rows)
+    full, part = plan.apply(b), plan.apply(b, rows=rows)
+    assert np.array_equal(part[rows], full[rows]) and not part[others].any()
+    did_far = False
+    for k in range(plan.nlevels):
+        L = plan.level(k)
+        for which in ("small", "keep"):
+            f, p = plan.near_level(k, which, b), plan.near_level(k, which, b, rows=rows)
+            assert np.array_equal(p[rows], f[rows]) and not p[others].any()
+        if len(L["far"]):
+            did_far = True
+            (fo, fm, fl), (po, pm, pl) = plan.far_level(k, b), plan.far_level(k, b, rows=rows)
+            assert np.array_equal(pm, fm)                                  # moments of every Y box either way
+            assert np.array_equal(po[rows], fo[rows]) and not po[others].any()
+            box = np.empty(5000, np.int64)
+            box[L["permx"]] = np.repeat(np.arange(len(L["offx"]) - 1), np.diff(L["offx"]))
+            mine = np.unique(box[rows])
+            assert np.array_equal(pl[mine], fl[mine])                      # local expansions of the boxes that hold a row
+            rest = np.setdiff1d(np.arange(len(L["offx"]) - 1), mine)
+            assert not pl[rest].any()
+    assert did_far
