@@ -26,6 +26,7 @@ struct TreeLevel {
     DBuf<uint32_t> prefix;  // nb Morton prefixes (depth*d bits)
     DBuf<float> ctr;     // nb*d box centres, row-major
     DBuf<int> cell;      // nb*d integer cell coordinates of the box at its depth
+    DBuf<uint32_t> cellpack;   // nb: the same coordinates in one word, coordinate j in bits [j*depth, (j+1)*depth)
     DBuf<int> childstart;   // nb+1: compact id at depth+1 of each box's first child (set by the next level)
     // near-field source operands of this level (built on first use by near_field): per point, the
     // split-f16 matrix operand of its coordinates relative to its own box centre, scaled by nearops_sc

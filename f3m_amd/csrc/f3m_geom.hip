@@ -441,10 +441,10 @@ static void radix_sort(DBuf<uint32_t> &keys, DBuf<int> &idx, long long n, int fr
 
 // depth 0: one box with every point, centred at origin + edge0/2 (F3M_src/n_tree.cu:86-95)
 __global__ void root_level_kernel(Geo g, int n, int *__restrict__ off, uint32_t *__restrict__ prefix, float *__restrict__ ctr,
-                                  int *__restrict__ cell)
+                                  int *__restrict__ cell, uint32_t *__restrict__ cellpack)
 {
     int j = threadIdx.x;
-    if (j == 0) { off[0] = 0; off[1] = n; prefix[0] = 0u; }
+    if (j == 0) { off[0] = 0; off[1] = n; prefix[0] = 0u; cellpack[0] = 0u; }
     if (j < g.d) {
         float half = 0.5f * g.edge0;
         ctr[j] = g.origin[j] + half;
@@ -477,7 +477,9 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     r.prefix.reset(1);
     r.ctr.reset(geo.d);
     r.cell.reset(geo.d);
-    F3M_LAUNCH(root_level_kernel, 1, 64, 0, s, geo, (int)n, r.off.get(), r.prefix.get(), r.ctr.get(), r.cell.get());
+    r.cellpack.reset(1);
+    F3M_LAUNCH(root_level_kernel, 1, 64, 0, s, geo, (int)n, r.off.get(), r.prefix.get(), r.ctr.get(), r.cell.get(),
+               r.cellpack.get());
     check_launch("root_level");
 }
 
@@ -513,6 +515,7 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
                                    const uint32_t *__restrict__ prefix_prev, const float *__restrict__ ctr_prev,
                                    const int *__restrict__ cell_prev, float quarter, int *__restrict__ off,
                                    uint32_t *__restrict__ prefix, float *__restrict__ ctr, int *__restrict__ cell,
+                                   uint32_t *__restrict__ cellpack, int depth,
                                    int *__restrict__ childstart_prev, int *__restrict__ stats)
 {
     long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -531,11 +534,15 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
     if (cnt > 0) {
         off[id] = natpos[nat];
         prefix[id] = (prefix_prev[q] << d) | (uint32_t)child;
+        uint32_t pack = 0u;
         for (int j = 0; j < d; j++) {
             float step = ((child >> j) & 1) ? quarter : -quarter;      // 0.25*edge*sign, exact
             ctr[(long long)id * d + j] = ctr_prev[(long long)q * d + j] + step;
-            cell[(long long)id * d + j] = 2 * cell_prev[(long long)q * d + j] + ((child >> j) & 1);
+            const int cj = 2 * cell_prev[(long long)q * d + j] + ((child >> j) & 1);
+            cell[(long long)id * d + j] = cj;
+            pack |= (uint32_t)cj << (j * depth);                       // d * depth <= 31
         }
+        cellpack[id] = pack;
         atomicMax(&stats[1], cnt);
     }
 }
@@ -608,11 +615,12 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     cur.prefix.reset(bound);
     cur.ctr.reset(bound * d);
     cur.cell.reset(bound * d);
+    cur.cellpack.reset(bound);
     prev.childstart.reset((size_t)prev.nb + 1);
     float quarter = 0.25f * prev.edge;
     F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
                prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
-               prev.childstart.get(), dstats);
+               cur.cellpack.get(), k, prev.childstart.get(), dstats);
     check_launch("build_level");
     cur.nb = -1;                       // until divide_finish
     cur.maxcount = -1;
@@ -755,7 +763,8 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     int nbx, const int *__restrict__ csx, int nbx_prev, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
     const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
     const float *__restrict__ ctrx, const float *__restrict__ ctry, int d, ClassifyParams cp,
-    const int *__restrict__ cellx, const int *__restrict__ celly, bool one_tree, unsigned long long *__restrict__ outliers,
+    const uint32_t *__restrict__ cellx, const uint32_t *__restrict__ celly, int depth, bool one_tree,
+    unsigned long long *__restrict__ outliers,
     unsigned long long *__restrict__ beyond,
     long long *__restrict__ cnt /* 3 arrays of nbx+1 */, const long long *__restrict__ pos /* 3 arrays of nbx+1 */,
     int *__restrict__ out_small, int *__restrict__ out_far, int *__restrict__ out_keep, int *__restrict__ rp_small,
@@ -780,6 +789,7 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     const int x = lo;
     const int t0 = keep_rowptr[x], t1 = keep_rowptr[x + 1];
     const int nx = offx[bx + 1] - offx[bx];
+    const uint32_t mycell = WRITE ? 0u : cellx[bx];
     float cx[kMaxD];
     for (int j = 0; j < d; j++) cx[j] = ctrx[(long long)bx * d + j];
     long long base0 = 0, base1 = 0, base2 = 0;
@@ -807,20 +817,18 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
                 const int size = nx + (offy[by + 1] - offy[by]);
                 c = classify_pair(cx, ctry + (long long)by * d, d, size, cp);
                 if (!WRITE && c == 1) {
-                    // the cell offset of a far pair must lie inside the M2L tables of the level
+                    // The cell offset of a far pair must lie inside the M2L tables of the level.  One tree: a pair is
+                    // regular if every offset from twice the parent's cell is in -2..3, or if it is a child of a
+                    // parent two cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere.
+                    // (cells from one packed word per box: one load per far pair instead of d)
+                    const uint32_t wy = celly[by], cmask = (1u << depth) - 1u;
                     bool outside = false;
-                    for (int j = 0; j < d; j++) {
-                        const int o = celly[(long long)by * d + j] - cellx[(long long)bx * d + j] - cp.omin[j];
-                        outside = outside || o < 0 || o >= kM2LOffsets;
-                    }
-                    if (outside) atomicAdd(beyond, 1ull);
-                }
-                if (!WRITE && c == 1 && one_tree) {
-                    // regular: every offset from twice the parent's cell in -2..3; or a child of a parent two
-                    // cells away along exactly one axis: -4, -3, 4 or 5 there and 0 or 1 elsewhere
                     int nout = 0, nmid = 0, nbad = 0;
                     for (int j = 0; j < d; j++) {
-                        int u = celly[(long long)by * d + j] - 2 * (cellx[(long long)bx * d + j] >> 1);
+                        const int yj = (int)((wy >> (j * depth)) & cmask), xj = (int)((mycell >> (j * depth)) & cmask);
+                        const int o = yj - xj - cp.omin[j];
+                        outside = outside || o < 0 || o >= kM2LOffsets;
+                        int u = yj - 2 * (xj >> 1);
                         if (u < -2 || u > 3) {
                             nout++;
                             if (u < -4 || u > 5) nbad++;
@@ -828,7 +836,8 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
                             nmid++;
                         }
                     }
-                    if (nout > 0 && (nout > 1 || nbad > 0 || nmid != d - 1)) atomicAdd(outliers, 1ull);
+                    if (outside) atomicAdd(beyond, 1ull);
+                    if (one_tree && nout > 0 && (nout > 1 || nbad > 0 || nmid != d - 1)) atomicAdd(outliers, 1ull);
                 }
             }
             const unsigned long long m0 = wave_ballot(c == 0), m1 = wave_ballot(c == 1), m2 = wave_ballot(c == 2);
@@ -969,13 +978,13 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     DBuf<long long> cnt((size_t)(3 * pend.stride));
     pend.pos.reset((size_t)(3 * pend.stride));
     for (int j = 0; j < kMaxD; j++) cp.omin[j] = j < d ? m2l_table_omin(tx.geo.origin[j], ty.geo.origin[j], lx.edge) : 0;
-    const int *cellx = lx.cell.get();
+    const uint32_t *cellx = lx.cellpack.get();
     unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
     unsigned long long *beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
     pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
     F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cell.get(), one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
+               cellx, ly.cellpack.get(), k, one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
     exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
@@ -1005,10 +1014,10 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     out.small_.rowptr.reset((size_t)pend.stride);
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
-    const int *cellx = lx.cell.get();
+    const uint32_t *cellx = lx.cellpack.get();
     F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cell.get(), one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr, (long long *)nullptr,
+               cellx, ly.cellpack.get(), k, one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr, (long long *)nullptr,
                (const long long *)pend.pos.get(),
                out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
                out.far.rowptr.get(), out.keep.rowptr.get());

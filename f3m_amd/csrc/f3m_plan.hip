@@ -671,6 +671,17 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     finish_stream(s);
 }
 
+// A call that fails may have queued work on the caller's stream and on the library's second stream, and the
+// buffers of that work have gone back to the pool while the error travelled up here: nothing may reuse them before
+// the device is idle.
+static void settle_after_error()
+{
+#ifndef F3M_CPU_EMU
+    (void)hipDeviceSynchronize();
+    (void)hipGetLastError();
+#endif
+}
+
 template <typename F>
 static int guarded(F f)
 {
@@ -679,9 +690,11 @@ static int guarded(F f)
         return 0;
     } catch (const Error &e) {
         g_error = e.what();
+        settle_after_error();
         return e.code;
     } catch (const std::exception &e) {
         g_error = e.what();
+        settle_after_error();
         return 99;
     }
 }
