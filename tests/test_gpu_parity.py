@@ -272,6 +272,53 @@ def test_stages_against_oracle(eng, oracle, name):
     assert rel_l2(got[sel], ora.apply(b, rows=rows)[sel]) < 1e-5
 
 
+@pytest.mark.parametrize("d,n,prm", [
+    (6, 60000, dict(ls=1.0, nr_of_interpolation=64, min_points=1000, small_field_points=200)),
+    (8, 100000, dict(ls=1.5, nr_of_interpolation=256, min_points=1000, small_field_points=300)),
+    (10, 120000, dict(ls=2.0, nr_of_interpolation=64, min_points=1000, small_field_points=100)),
+])
+def test_six_to_ten_dimensions_against_oracle(eng, oracle, d, n, prm):
+    """The reference exports its operator for 1 to 10 dimensions (F3M_src/pybinder_setup.cu:17-36).  Beyond five
+    the engine runs its general kernels (any tensor grid: 2^6, 2^8 and 2^6 x 1^4 nodes here; two matrix instructions
+    per near-field tile): box division and lists bit for bit, every stage and the product against the oracle on the
+    rows of eight boxes (the oracle's complete M2L would take minutes: up to 868 352 far pairs of 64^2 to 256^2 terms)."""
+    print("case d=%d" % d, flush=True)
+    rng = np.random.default_rng(d)
+    X = rng.random((n, d), dtype=f32)
+    b = rng.standard_normal((n, 1)).astype(f32)
+    plan = eng.Plan(dev(X), None, **prm)
+    ora = oracle.Plan(X, None, **prm)
+    assert_plan_matches_oracle(plan, ora)
+    L = ora.level(ora.nlevels - 1)
+    nb = len(L["offx"]) - 1
+    boxes = np.unique(np.linspace(0, nb - 1, 8).astype(int))
+    rows = np.concatenate([L["permx"][L["offx"][bx]:L["offx"][bx + 1]] for bx in boxes])
+    far_levels = 0
+    for k in range(1, plan.depth + 1):
+        sz = plan.level_sizes(k)
+        if sz["nsmall"]:
+            got = plan.near_level(k, "small", dev(b)).cpu().numpy()
+            assert rel_l2(got[rows], ora.near_level(k - 1, "small", b, rows=rows)[rows]) < 1e-5
+        if sz["nfar"]:
+            far_levels += 1
+            out, mom, loc = plan.far_level(k, dev(b), want_expansions=True)
+            o_out, o_mom, o_loc = ora.far_level(k - 1, b, rows=rows)
+            lvl = ora.level(k - 1)
+            mine = np.unique(canonical_box_of_point(lvl, "x")[rows])
+            assert rel_l2(mom.cpu().numpy(), np.moveaxis(o_mom, 2, 0)) < 1e-4
+            assert rel_l2(loc.cpu().numpy()[:, mine], np.moveaxis(o_loc, 2, 0)[:, mine]) < 1e-4
+            assert rel_l2(out.cpu().numpy()[rows], o_out[rows]) < 1e-4
+    assert far_levels >= 1
+    if plan.level_sizes(plan.depth)["nkeep"]:
+        got = plan.near_level(plan.depth, "keep", dev(b)).cpu().numpy()
+        assert rel_l2(got[rows], ora.near_level(plan.depth - 1, "keep", b, rows=rows)[rows]) < 1e-5
+    got = plan.apply(dev(b)).cpu().numpy()
+    want = ora.apply(b, rows=rows)
+    assert rel_l2(got[rows], want[rows]) < 1e-5
+    exact = oracle.exact_f64(X[rows], X, b, prm["ls"])
+    assert rel_l2(got[rows], exact) <= 1.5 * rel_l2(want[rows], exact) + 1e-7
+
+
 PRODUCT_NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5_243", "uniform3_ls0.1", "uniform3_ls10",
                  "normal3_ls0.1", "normal3_ls10"]
 # Where the reference algorithm itself (the oracle, same nodes and lengthscale) misses the 1e-3 of the
@@ -570,6 +617,19 @@ def test_edge_cases(eng, oracle):
         eng.kmvm(torch.from_numpy(X), None, torch.from_numpy(b))                      # host tensors
     with pytest.raises(AssertionError):
         eng.kmvm(dev(X), None, dev(b[:100]))
+
+
+def test_c_program_on_the_abi(eng):
+    """tests/abi_c/abi_smoke.c: a plain C program (HIP runtime for device memory, no Python in the process) calls
+    f3m_kmvm_f32, a plan forward and transposed, and the exact product through include/f3m.h."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "abi_c", "_build", "abi_smoke")
+    assert os.path.exists(exe), "tests/abi_c/build_smoke.py has not been run"
+    print("case C program", flush=True)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=120)
+    print(res.stdout, res.stderr, flush=True)
+    assert res.returncode == 0 and res.stdout.strip().endswith("OK"), res.stdout + res.stderr
 
 
 def test_reference_operator_classes(eng, oracle):
