@@ -84,3 +84,39 @@ def test_apply_without_allocation_refuses_what_does_not_fit(eng):
     assert e.value.code == 42 and "scratch" in str(e.value)
     assert torch.isnan(out).all()
     plan.close()
+
+
+def test_apply_without_allocation_under_graph_capture(eng):
+    """One of the callers the entry point is for: a HIP graph.  The call is captured once and replayed with
+    the program's own eager products and synchronisations between the replays; every replay must give the
+    eager result bit for bit, also after the input buffer's contents changed."""
+    import torch
+    print("case no-alloc: captured into a graph, 3-D 300000 points, 5 replays", flush=True)
+    rng = np.random.default_rng(33)
+    n = 300000
+    X = dev(rng.random((n, 3), dtype=f32))
+    b = dev(rng.standard_normal((n, 2)).astype(f32))
+    plan = eng.Plan(X, None, ls=0.7)
+    want = plan.apply(b)
+    out = torch.full((n, 2), float("nan"), device="cuda")
+    plan.apply_noalloc(b, out)                              # scratch address of this device is looked up here
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=torch.cuda.Stream()):
+        plan.apply_noalloc(b, out)
+    for replay in range(4):
+        out.fill_(float("nan"))
+        other = plan.apply(b)                               # eager work of the same library between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), replay
+        assert torch.equal(other, want)
+    b2 = dev(rng.standard_normal((n, 2)).astype(f32))
+    want2 = plan.apply(b2)
+    b.copy_(b2)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out, want2)
+    plan.close()
