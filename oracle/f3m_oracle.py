@@ -175,7 +175,7 @@ class Plan:
         self.work_near_pairs, self.work_far_pairs, self.work_interp_pts = w
 
     def __del__(self):
-        if getattr(self, "_h", None):
+        if getattr(self, "_h", None) and lib is not None:      # module globals are gone at interpreter exit
             lib().fo_plan_destroy(self._h)
             self._h = None
 

@@ -319,6 +319,85 @@ def test_six_to_ten_dimensions_against_oracle(eng, oracle, d, n, prm):
     assert rel_l2(got[rows], exact) <= 1.5 * rel_l2(want[rows], exact) + 1e-7
 
 
+def random_cloud(rng, kind, n, d):
+    if kind == "uniform":
+        return rng.random((n, d), dtype=f32)
+    if kind == "normal":
+        return rng.standard_normal((n, d)).astype(f32)
+    if kind == "clustered":
+        mu, sd = rng.random((8, d)) * 4, 0.02 + 0.3 * rng.random((8, d))
+        return np.concatenate([rng.normal(m, s, (n // 8 + 1, d)) for m, s in zip(mu, sd)])[:n].astype(f32)
+    if kind == "lattice":            # points on box faces at every level, and duplicates
+        m = max(2, int(round(n ** (1.0 / d))))
+        g = (np.stack(np.meshgrid(*[np.arange(m)] * d, indexing="ij"), -1).reshape(-1, d) / f32(m - 1)).astype(f32)
+        return np.concatenate([g, g[::3]])[:max(n, 10)]
+    if kind == "line":               # a noisy segment: deep, thin trees
+        return (rng.random((n, 1)) * rng.standard_normal((1, d)) + 1e-3 * rng.standard_normal((n, d))).astype(f32)
+    raise KeyError(kind)
+
+
+def random_configuration(case):
+    """One draw of (X, Y, b, parameters): dimension 1-6, five kinds of cloud, one tree or two, lengthscale 0.05-20,
+    node counts that are and are not full tensor grids, both cutoffs, variance compression, 1-5 columns."""
+    rng = np.random.default_rng(1000 + case)
+    d = int(rng.choice([1, 2, 3, 3, 3, 4, 5, 6]))
+    kind = str(rng.choice(["uniform", "normal", "clustered", "lattice", "line"]))
+    n = int(rng.integers(500, 40000 if d <= 3 else 25000))
+    two = bool(rng.random() < 0.35)
+    m = int(rng.integers(300, 30000)) if two else n
+    ls = float(np.exp(rng.uniform(np.log(0.05), np.log(20))))
+    nodes = int(rng.choice({1: [4, 8, 16], 2: [16, 36, 64, 100], 3: [8, 27, 64, 64, 125], 4: [16, 81, 256], 5: [32, 243],
+                            6: [64, 729]}[d]))
+    prm = dict(ls=ls, nr_of_interpolation=nodes, min_points=int(rng.choice([50, 200, 500, 1000, 2500])),
+               small_field_points=int(rng.choice([20, 100, 300, 1000])))
+    varc = bool(rng.random() < 0.25)
+    c = int(rng.choice([1, 1, 2, 3, 5]))
+    if varc:
+        prm.update(var_compression=True, eff_var_limit=float(rng.choice([0.1, 0.3, 1.0])))
+    X = random_cloud(rng, kind, n, d)
+    Y = random_cloud(rng, str(rng.choice(["uniform", "normal", "clustered"])), m, d) if two else None
+    if Y is not None and rng.random() < 0.5:      # sources spread over the targets' region
+        Y = (X.min(0) + (X.max(0) - X.min(0)) * rng.random((m, d))).astype(f32)
+    b = rng.standard_normal((X.shape[0] if Y is None else Y.shape[0], c)).astype(f32)
+    return X, Y, b, prm, kind
+
+
+# 32 of 540 draws that were run once in the same way (all of them agreed); the seeds are kept so that a failure names
+# its case.
+@pytest.mark.parametrize("case", [0, 3, 7, 11, 18, 20, 25, 28, 31, 34, 37, 52, 68, 77, 91, 104, 120, 133, 149, 162, 176, 188,
+                                  203, 240, 271, 305, 333, 364, 402, 447, 489, 530])
+def test_random_configurations_against_oracle(eng, oracle, case):
+    """Box division and lists bit for bit, the product no worse than 1.5x the oracle's error against the fp64 exact
+    product, the one-shot call with the bits of plan + apply, and for two trees the transposed product against the
+    oracle's product of the swapped clouds."""
+    X, Y, b, prm, kind = random_configuration(case)
+    print("case random %d: d=%d %s n=%d m=%s c=%d %s" % (case, X.shape[1], kind, X.shape[0],
+                                                         None if Y is None else Y.shape[0], b.shape[1], prm), flush=True)
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    ora = oracle.Plan(X, Y, **prm)
+    assert_plan_matches_oracle(plan, ora)
+    got = plan.apply(dev(b)).cpu().numpy()
+    want = ora.apply(b)
+    exact = oracle.exact_f64(X, X if Y is None else Y, b, prm["ls"])
+    assert np.isfinite(got).all()
+    if np.linalg.norm(exact) > 0:
+        assert rel_l2(got, exact) <= 1.5 * rel_l2(want, exact) + 3e-6, (rel_l2(got, exact), rel_l2(want, exact))
+    else:                                          # clouds many lengthscales apart: every term underflows
+        assert not got.any() and not want.any()
+    one = eng.kmvm(dev(X), None if Y is None else dev(Y), dev(b), **prm).cpu().numpy()
+    assert np.array_equal(one, got)
+    if Y is not None:
+        u = np.random.default_rng(case).standard_normal((X.shape[0], 1)).astype(f32)
+        got_t = plan.apply_transpose(dev(u)).cpu().numpy()
+        exact_t = oracle.exact_f64(Y, X, u, prm["ls"])
+        want_t = oracle.Plan(Y, X, **prm).apply(u)
+        if np.linalg.norm(exact_t) > 0:
+            assert rel_l2(got_t, exact_t) <= 1.5 * rel_l2(want_t, exact_t) + 3e-6
+        else:
+            assert not got_t.any()
+    plan.close()
+
+
 PRODUCT_NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5_243", "uniform3_ls0.1", "uniform3_ls10",
                  "normal3_ls0.1", "normal3_ls10"]
 # Where the reference algorithm itself (the oracle, same nodes and lengthscale) misses the 1e-3 of the
