@@ -143,7 +143,10 @@ void divide_discard(Tree &t);
 // The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts and scans (the
 // sizes of the small, far and keep list are then the last entries pos[(c+1)*stride - 1] of the three
 // scans; the number of far pairs outside the sibling-group tables is added to dtot[3] and of those outside
-// the M2L tables of the level to dtot[6], which the caller keeps zero between levels), lists_finish allocates from the fetched totals htot[0..3] and writes.
+// the M2L tables of the level to dtot[6], which the caller keeps zero between levels; the row statistics of the
+// small and the keep list -- x boxes with pairs, their points, their pieces of 128 and of 160 points -- are added
+// to the eight zeroed words drow), lists_finish allocates from the fetched totals htot[0..3], takes the fetched row
+// statistics hrow[0..7] and writes.
 // divide_launch likewise adds to dstats[0..1], zero on entry.
 struct ListsPending {
     DBuf<long long> pos;
@@ -152,9 +155,9 @@ struct ListsPending {
     bool active = false;
 };
 void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
-                  ListsPending &pend, long long *dtot, hipStream_t s);
+                  ListsPending &pend, long long *dtot, long long *drow /* 8 zeroed words or null */, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
-                  const ClassifyParams &cp, PlanLevel &out, long long *drow /* 8 zeroed words or null */, hipStream_t s);
+                  const ClassifyParams &cp, PlanLevel &out, const long long *hrow /* 8 words or null */, hipStream_t s);
 // out = `in` with the two boxes of every pair swapped, sorted by (by, bx) (a stable sort by `by` of a list that is
 // sorted by bx), its row pointers over the nby boxes of the Y level, and its row statistics for the near field
 void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipStream_t s);

@@ -852,11 +852,11 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     if (!WRITE && lane == 0) { cnt[bx] = c0; cnt[stride + bx] = c1; cnt[2 * stride + bx] = c2; }
 }
 
-// Row statistics of the small and the keep list of a level: out[4c .. 4c+3] (c = 0 small, 1 keep) += x
-// boxes with pairs, their points, their pieces of 128 and of 160 points (out is zero before).
+// Row statistics of the small and the keep list of a level from the per-box counts of the list builder's counting
+// pass (cnt: three arrays of `stride` entries, small, far, keep): out[4c .. 4c+3] (c = 0 small, 1 keep) += x boxes
+// with pairs, their points, their pieces of 128 and of 160 points (out is zero before).
 constexpr int kRowStatBlock = 256;
-__global__ void __launch_bounds__(kRowStatBlock) list_rowstats_kernel(const int *__restrict__ rowptr_small,
-                                                                       const int *__restrict__ rowptr_keep,
+__global__ void __launch_bounds__(kRowStatBlock) list_rowstats_kernel(const long long *__restrict__ cnt, long long stride,
                                                                        const int *__restrict__ offx, int nbx,
                                                                        unsigned long long *__restrict__ out)
 {
@@ -867,8 +867,7 @@ __global__ void __launch_bounds__(kRowStatBlock) list_rowstats_kernel(const int 
     if (b < nbx) {
         const unsigned long long n = (unsigned long long)(offx[b + 1] - offx[b]);
         for (int c = 0; c < 2; c++) {
-            const int *rp = c ? rowptr_keep : rowptr_small;
-            if (rp[b + 1] > rp[b]) {
+            if (cnt[(c ? 2 : 0) * stride + b] > 0) {
                 atomicAdd(&acc[4 * c + 0], 1ull);
                 atomicAdd(&acc[4 * c + 1], n);
                 atomicAdd(&acc[4 * c + 2], (n + 127) / 128);
@@ -962,7 +961,7 @@ void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipS
 }
 
 void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
-                  ListsPending &pend, long long *dtot, hipStream_t s)
+                  ListsPending &pend, long long *dtot, long long *drow, hipStream_t s)
 {
     const int d = tx.geo.d;
     const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
@@ -988,13 +987,23 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
     check_launch("lists_count");
     exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
+    if (drow != nullptr) {
+        F3M_LAUNCH(list_rowstats_kernel, cdiv(nbx, kRowStatBlock), kRowStatBlock, 0, s, cnt.get(), pend.stride, lx.off.get(), nbx,
+                   reinterpret_cast<unsigned long long *>(drow));
+        check_launch("list_rowstats");
+    }
 }
 
 void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
-                  const ClassifyParams &cp, PlanLevel &out, long long *drow, hipStream_t s)
+                  const ClassifyParams &cp, PlanLevel &out, const long long *hrow, hipStream_t s)
 {
     out.far.n = out.small_.n = out.keep.n = 0;
     if (!pend.active) return;
+    if (hrow != nullptr) {
+        PairList &sm = out.small_, &kp = out.keep;
+        sm.rows = hrow[0], sm.row_points = hrow[1], sm.items128 = hrow[2], sm.items160 = hrow[3];
+        kp.rows = hrow[4], kp.row_points = hrow[5], kp.items128 = hrow[6], kp.items160 = hrow[7];
+    }
     const int d = tx.geo.d;
     const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
@@ -1022,11 +1031,6 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
                out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
                out.far.rowptr.get(), out.keep.rowptr.get());
     check_launch("lists_write");
-    if (drow != nullptr) {
-        F3M_LAUNCH(list_rowstats_kernel, cdiv(nbx, kRowStatBlock), kRowStatBlock, 0, s, out.small_.rowptr.get(),
-                   out.keep.rowptr.get(), lx.off.get(), nbx, reinterpret_cast<unsigned long long *>(drow));
-        check_launch("list_rowstats");
-    }
     pend.pos.free();
     pend.active = false;
 }

@@ -201,7 +201,9 @@ static SideStream &side_stream()
 #endif
 
 // b_early (nullable, with c_early columns): the weights of the product that will follow at once (f3m_kmvm_f32);
-// their first column group is put into sorted order while the lists are built.
+// their first column group is put into sorted order while the lists are built.  With b_early the function returns
+// when the last kernels of the plan are queued, not when they are done: the product is queued behind them on the
+// same stream (every host-side figure of the plan is known by then), so the GPU does not wait for the host in between.
 static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y, long long M, const f3m_params *prm,
                              hipStream_t s, const float *b_early = nullptr, int c_early = 0)
 {
@@ -262,11 +264,17 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // box counts already call for it (it is dropped again if the keep list of depth k turns out empty).
     // Host record of a level, in 32-bit words: [0..5] pairs of the small, far and keep list (64 bits each),
     // [6,7] far pairs outside the sibling-group M2L tables, [8,9] boxes and largest box of the X tree's new level,
-    // [10,11] of the Y tree's, [12,13] far pairs outside the M2L tables of the level (must be none).  On the device the first three are the last entries of the list builder's
-    // scans; the counters behind [6..11] live in dres and are cleared by the readback that fetches them.
+    // [10,11] of the Y tree's, [12,13] far pairs outside the M2L tables of the level (must be none), [14,15] fullest
+    // cells at the sorted depth (first division only), [16..31] row statistics of the small and the keep list (eight
+    // 64-bit words: what the near field needs to shape its launches).  On the device the first three are the last
+    // entries of the list builder's scans; the counters behind [6..15] live in dres and are cleared by the readback
+    // that fetches them, the row statistics in drow, eight words per level.
     DBuf<int> dres(16);
     dev_fill(dres.get(), 0, 16 * sizeof(int), s);
-    alignas(8) int hres[16];
+    constexpr int kMaxLevels = 40;
+    DBuf<long long> drow((size_t)8 * kMaxLevels);
+    dev_fill(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s);
+    alignas(8) int hres[32];
     auto fetch_level = [&](const ListsPending *pend, bool division) {
         memset(hres, 0, sizeof(hres));
         ExportList L;
@@ -274,16 +282,12 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             for (int c = 0; c < 3; c++) L.add(pend->pos.get() + (c + 1) * pend->stride - 1, 2, 2 * c);
             L.add(dres.get() + 6, 2, 6, true);
             L.add(dres.get() + 12, 2, 12, true);
+            L.add(drow.get() + 8 * (P->levels.size() - 1), 16, 16);
         }
         if (division) L.add(dres.get() + 8, sym ? 2 : 4, 8, true);
         if (division && pend == nullptr) L.add(dres.get() + 14, 2, 14, true);      // first division: fullest sorted cells
         if (L.nseg > 0) fetch_segments(L, hres, s);
     };
-    // row statistics of the small and keep lists, 8 words per level; nothing at plan time depends on
-    // them, so they are fetched once at the end instead of with the per-level wait
-    constexpr int kMaxLevels = 40;
-    DBuf<long long> drow((size_t)8 * kMaxLevels);
-    dev_fill(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s);
     auto wants_division = [&]() {
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
@@ -368,7 +372,9 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             PlanLevel &L = P->levels.back();
             ClassifyParams cp = classify_params(*P, e);
             ListsPending pend;
-            lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()), s);
+            F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
+            lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()),
+                         drow.get() + 8 * (P->levels.size() - 1), s);
             const bool ahead = wants_division();
             if (ahead) { settle_early(); start_division(); }
 #ifndef F3M_CPU_EMU
@@ -378,9 +384,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             if (!ahead && early) prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
 #endif
             fetch_level(&pend, ahead);
-            F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
-                         drow.get() + 8 * (P->levels.size() - 1), s);
+                         reinterpret_cast<const long long *>(hres + 16), s);
             if (ahead) finish_division();
             L.num_nodes = prm->nr_of_interpolation;
             if (prm->var_compression && e * e * P->lcs < 0.01f)      // F3M_src/n_tree.cu:971-978,1022-1025
@@ -415,17 +420,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             F3M_HIP(hipMemcpyAsync(P->Yraw.get(), Y, sizeof(float) * (size_t)M * d, hipMemcpyDeviceToDevice, s));
         }
     }
-    if (!P->levels.empty()) {
-        std::vector<long long> hrow(8 * P->levels.size());
-        fetch_small(hrow.data(), drow.get(), hrow.size(), s);
-        for (size_t l = 0; l < P->levels.size(); l++) {
-            const long long *r = hrow.data() + 8 * l;
-            PairList &sm = P->levels[l].small_, &kp = P->levels[l].keep;
-            sm.rows = r[0], sm.row_points = r[1], sm.items128 = r[2], sm.items160 = r[3];
-            kp.rows = r[4], kp.row_points = r[5], kp.items128 = r[6], kp.items160 = r[7];
-        }
-    }
-    F3M_HIP(hipStreamSynchronize(s));
+    if (b_early == nullptr) F3M_HIP(hipStreamSynchronize(s));
     return P.release();
 }
 
