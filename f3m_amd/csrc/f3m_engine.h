@@ -28,6 +28,7 @@ struct TreeLevel {
     DBuf<int> cell;      // nb*d integer cell coordinates of the box at its depth
     DBuf<uint32_t> cellpack;   // nb: the same coordinates in one word, coordinate j in bits [j*depth, (j+1)*depth)
     DBuf<int> childstart;   // nb+1: compact id at depth+1 of each box's first child (set by the next level)
+    DBuf<int> parent;       // nb: compact id at depth-1 of each box's parent (the root: 0)
     // near-field source operands of this level (built on first use by near_field): per point, the
     // split-f16 matrix operand of its coordinates relative to its own box centre, scaled by nearops_sc
     mutable DBuf<unsigned char> nearops;

@@ -516,7 +516,7 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
                                    const int *__restrict__ cell_prev, float quarter, int *__restrict__ off,
                                    uint32_t *__restrict__ prefix, float *__restrict__ ctr, int *__restrict__ cell,
                                    uint32_t *__restrict__ cellpack, int depth,
-                                   int *__restrict__ childstart_prev, int *__restrict__ stats)
+                                   int *__restrict__ childstart_prev, int *__restrict__ parent, int *__restrict__ stats)
 {
     long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (nat > ncand) return;
@@ -533,6 +533,7 @@ __global__ void build_level_kernel(const int *__restrict__ natpos, const int *__
     int cnt = natpos[nat + 1] - natpos[nat];
     if (cnt > 0) {
         off[id] = natpos[nat];
+        parent[id] = q;
         prefix[id] = (prefix_prev[q] << d) | (uint32_t)child;
         uint32_t pack = 0u;
         for (int j = 0; j < d; j++) {
@@ -616,11 +617,12 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     cur.ctr.reset(bound * d);
     cur.cell.reset(bound * d);
     cur.cellpack.reset(bound);
+    cur.parent.reset(bound);
     prev.childstart.reset((size_t)prev.nb + 1);
     float quarter = 0.25f * prev.edge;
     F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
                prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
-               cur.cellpack.get(), k, prev.childstart.get(), dstats);
+               cur.cellpack.get(), k, prev.childstart.get(), cur.parent.get(), dstats);
     check_launch("build_level");
     cur.nb = -1;                       // until divide_finish
     cur.maxcount = -1;
@@ -760,7 +762,7 @@ constexpr int kListWaves = 4;   // wavefronts per workgroup
 
 template <bool WRITE>
 __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
-    int nbx, const int *__restrict__ csx, int nbx_prev, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
+    int nbx, const int *__restrict__ parentx, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
     const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
     const float *__restrict__ ctrx, const float *__restrict__ ctry, int d, ClassifyParams cp,
     const uint32_t *__restrict__ cellx, const uint32_t *__restrict__ celly, int depth, bool one_tree,
@@ -780,13 +782,7 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
         }
         return;
     }
-    // parent of bx: last x with csx[x] <= bx
-    int lo = 0, hi = nbx_prev;
-    while (hi - lo > 1) {
-        int mid = lo + ((hi - lo) >> 1);
-        if (csx[mid] <= bx) lo = mid; else hi = mid;
-    }
-    const int x = lo;
+    const int x = parentx[bx];
     const int t0 = keep_rowptr[x], t1 = keep_rowptr[x + 1];
     const int nx = offx[bx + 1] - offx[bx];
     const uint32_t mycell = WRITE ? 0u : cellx[bx];
@@ -964,7 +960,7 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
                   ListsPending &pend, long long *dtot, long long *drow, hipStream_t s)
 {
     const int d = tx.geo.d;
-    const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
+    const TreeLevel &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
     pend.active = false;
     if (keep_prev.n == 0) return;
@@ -981,7 +977,7 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
     unsigned long long *beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
     pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
-    F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+    F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
                cellx, ly.cellpack.get(), k, one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
                (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
@@ -1005,7 +1001,7 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
         kp.rows = hrow[4], kp.row_points = hrow[5], kp.items128 = hrow[6], kp.items160 = hrow[7];
     }
     const int d = tx.geo.d;
-    const TreeLevel &px = tx.lev[k - 1], &py = ty.lev[k - 1];
+    const TreeLevel &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
     const bool one_tree = &tx == &ty;
     const int nbx = lx.nb;
@@ -1024,7 +1020,7 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
     const uint32_t *cellx = lx.cellpack.get();
-    F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, px.childstart.get(), px.nb, py.childstart.get(),
+    F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),
                keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
                cellx, ly.cellpack.get(), k, one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr, (long long *)nullptr,
                (const long long *)pend.pos.get(),
