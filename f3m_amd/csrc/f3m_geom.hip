@@ -730,12 +730,13 @@ void lookup_boxes(const Tree &t, const TreeLevel &lev, const int *cells, long lo
 // y); only non-empty children exist here, so the filter step is implicit.
 
 // 0 small, 1 far, 2 keep, 3 dropped (F3M_src/1_d_conv.cu:927-952 and :983-1026)
-__device__ inline int classify_pair(const float *__restrict__ cx, const float *__restrict__ cy, int d, int size,
-                                    const ClassifyParams &cp)
+template <int D>
+__device__ inline int classify_pair(const float *__restrict__ cx, const float *__restrict__ cy, int size, const ClassifyParams &cp)
 {
     if (cp.do_init && size < 2 * cp.nr_interp) return 0;
     float acc = 0.f;
-    for (int j = 0; j < d; j++) {
+#pragma unroll
+    for (int j = 0; j < D; j++) {
         float dk = cy[j] - cx[j];
         float sq = dk * dk;
         acc = acc + sq;
@@ -760,11 +761,11 @@ __device__ inline int classify_pair(const float *__restrict__ cx, const float *_
 // pairs at the offsets that the scan of those counts gave (which are also the row pointers).
 constexpr int kListWaves = 4;   // wavefronts per workgroup
 
-template <bool WRITE>
+template <bool WRITE, int D>
 __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     int nbx, const int *__restrict__ parentx, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
     const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
-    const float *__restrict__ ctrx, const float *__restrict__ ctry, int d, ClassifyParams cp,
+    const float *__restrict__ ctrx, const float *__restrict__ ctry, ClassifyParams cp,
     const uint32_t *__restrict__ cellx, const uint32_t *__restrict__ celly, int depth, bool one_tree,
     unsigned long long *__restrict__ outliers,
     unsigned long long *__restrict__ beyond,
@@ -786,8 +787,10 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     const int t0 = keep_rowptr[x], t1 = keep_rowptr[x + 1];
     const int nx = offx[bx + 1] - offx[bx];
     const uint32_t mycell = WRITE ? 0u : cellx[bx];
-    float cx[kMaxD];
-    for (int j = 0; j < d; j++) cx[j] = ctrx[(long long)bx * d + j];
+    constexpr int d = D;
+    float cx[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) cx[j] = ctrx[(long long)bx * D + j];
     long long base0 = 0, base1 = 0, base2 = 0;
     if (WRITE) {
         base0 = pos[bx]; base1 = pos[stride + bx]; base2 = pos[2 * stride + bx];
@@ -811,7 +814,10 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
             int c = 3;
             if (there) {
                 const int size = nx + (offy[by + 1] - offy[by]);
-                c = classify_pair(cx, ctry + (long long)by * d, d, size, cp);
+                float cy[D];
+#pragma unroll
+                for (int j = 0; j < D; j++) cy[j] = ctry[(long long)by * D + j];
+                c = classify_pair<D>(cx, cy, size, cp);
                 if (!WRITE && c == 1) {
                     // The cell offset of a far pair must lie inside the M2L tables of the level.  One tree: a pair is
                     // regular if every offset from twice the parent's cell is in -2..3, or if it is a child of a
@@ -820,7 +826,8 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
                     const uint32_t wy = celly[by], cmask = (1u << depth) - 1u;
                     bool outside = false;
                     int nout = 0, nmid = 0, nbad = 0;
-                    for (int j = 0; j < d; j++) {
+#pragma unroll
+                    for (int j = 0; j < D; j++) {
                         const int yj = (int)((wy >> (j * depth)) & cmask), xj = (int)((mycell >> (j * depth)) & cmask);
                         const int o = yj - xj - cp.omin[j];
                         outside = outside || o < 0 || o >= kM2LOffsets;
@@ -977,10 +984,19 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
     unsigned long long *beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
     pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
-    F3M_LAUNCH((lists_kernel<false>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),
-               keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cellpack.get(), k, one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, (int *)nullptr,
-               (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);
+#define F3M_CASE(DD)                                                                                                          \
+    case DD:                                                                                                                  \
+        F3M_LAUNCH((lists_kernel<false, DD>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),    \
+                   keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), cp, \
+                   cellx, ly.cellpack.get(), k, one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, \
+                   (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);                            \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
     check_launch("lists_count");
     exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
     if (drow != nullptr) {
@@ -1020,12 +1036,20 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
     const uint32_t *cellx = lx.cellpack.get();
-    F3M_LAUNCH((lists_kernel<true>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),
-               keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), d, cp,
-               cellx, ly.cellpack.get(), k, one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr, (long long *)nullptr,
-               (const long long *)pend.pos.get(),
-               out.small_.pairs.get(), out.far.pairs.get(), out.keep.pairs.get(), out.small_.rowptr.get(),
-               out.far.rowptr.get(), out.keep.rowptr.get());
+#define F3M_CASE(DD)                                                                                                          \
+    case DD:                                                                                                                  \
+        F3M_LAUNCH((lists_kernel<true, DD>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),     \
+                   keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), cp, \
+                   cellx, ly.cellpack.get(), k, one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr,        \
+                   (long long *)nullptr, (const long long *)pend.pos.get(), out.small_.pairs.get(), out.far.pairs.get(),       \
+                   out.keep.pairs.get(), out.small_.rowptr.get(), out.far.rowptr.get(), out.keep.rowptr.get());                \
+        break;
+    switch (d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
     check_launch("lists_write");
     pend.pos.free();
     pend.active = false;
