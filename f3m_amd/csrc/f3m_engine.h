@@ -125,7 +125,7 @@ void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipS
 // keys, order (perm) and the root level; the coordinates are gathered by gather_tree_points once
 // every division is done (divisions may still refine the order inside the boxes)
 void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s);
-void gather_tree_points(Tree &t, const float *X, hipStream_t s);
+void gather_tree_points(Tree &t, const float *X, hipStream_t s, bool background = false);
 // One division in two steps, so that the host can wait once for several results: divide_launch starts
 // the kernels that build lev[k] from lev[k-1] and appends the level; divide_finish completes it with
 // the two numbers the kernels left in dstats (boxes, largest count) once the host has fetched them;
@@ -182,12 +182,13 @@ struct NodeSet {
 void make_nodes(NodeSet &ns, int d, int max_nodes, hipStream_t s);
 void set_node_offsets(NodeSet &ns, float edge, hipStream_t s);
 
-void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s);
+// background: the move runs beside latency-bound kernels of another stream and takes one workgroup per compute unit
+void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s, bool background = false);
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
 // ncol (1..4) neighbouring columns at once, one access per row; the scatter adds outs2 (same layout) if it is given
 void gather_columns(const float *b, const int *perm, long long n, int c, int col, int ncol, float *bs, long long bstride,
-                    hipStream_t s);
+                    hipStream_t s, bool background = false);
 void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
                      int ncol, float *out, hipStream_t s);
 

@@ -22,17 +22,45 @@ template <int D>
 __global__ void gather_points_kernel(const float *__restrict__ X, const int *__restrict__ perm, long long n,
                                      float *__restrict__ pts)
 {
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const fvec<D> row = *reinterpret_cast<const fvec<D> *>(X + (long long)perm[i] * D);
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const fvec<D> row = *reinterpret_cast<const fvec<D> *>(X + (long long)perm[i] * D);
 #pragma unroll
-    for (int j = 0; j < D; j++) pts[(long long)j * n + i] = row.v[j];
+        for (int j = 0; j < D; j++) pts[(long long)j * n + i] = row.v[j];
+    }
 }
-void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s)
+// Workgroups of a gather: one thread per row, or, for a move that runs in the background beside many small
+// latency-bound kernels (the level loop of the plan), one workgroup per compute unit that walks the rows in
+// strides: the random reads of a full-size launch fill the memory system's queues and the small kernels'
+// dependent loads then take several times as long (plan at N=1e7, 3-D: 1.05 -> 0.90 ms; 64 workgroups no
+// longer finish in time, 1024 disturb as much as all).
+static unsigned gather_grid(long long n, bool background)
+{
+    const unsigned full = cdiv(n, 256);
+    if (!background) return full;
+#ifndef F3M_CPU_EMU
+    static std::mutex mu;
+    static std::map<int, int> units;          // compute units per device
+    int dev = 0, cu = 0;
+    F3M_HIP(hipGetDevice(&dev));
+    {
+        std::lock_guard<std::mutex> g(mu);
+        auto it = units.find(dev);
+        if (it == units.end()) {
+            F3M_HIP(hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev));
+            it = units.emplace(dev, std::max(cu, 1)).first;
+        }
+        cu = it->second;
+    }
+    return std::min<unsigned>(full, (unsigned)cu);
+#else
+    return full;
+#endif
+}
+void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s, bool background)
 {
 #define F3M_CASE(DD)                                                                                  \
     case DD:                                                                                          \
-        F3M_LAUNCH((gather_points_kernel<DD>), cdiv(n, 256), 256, 0, s, X, perm, n, pts);             \
+        F3M_LAUNCH((gather_points_kernel<DD>), gather_grid(n, background), 256, 0, s, X, perm, n, pts); \
         break;
     switch (d) {
         F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -50,27 +78,27 @@ template <int NC>
 __global__ void gather_columns_kernel(const float *__restrict__ b, const int *__restrict__ perm, long long n, int c, int col,
                                       float *__restrict__ bs, long long bstride)
 {
-    long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
-    const fvec<NC> row = *reinterpret_cast<const fvec<NC> *>(b + (long long)perm[i] * c + col);
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+        const fvec<NC> row = *reinterpret_cast<const fvec<NC> *>(b + (long long)perm[i] * c + col);
 #pragma unroll
-    for (int q = 0; q < NC; q++) bs[q * bstride + i] = row.v[q];
+        for (int q = 0; q < NC; q++) bs[q * bstride + i] = row.v[q];
+    }
 }
 void gather_columns(const float *b, const int *perm, long long n, int c, int col, int ncol, float *bs, long long bstride,
-                    hipStream_t s)
+                    hipStream_t s, bool background)
 {
     switch (ncol) {
-    case 1: F3M_LAUNCH((gather_columns_kernel<1>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
-    case 2: F3M_LAUNCH((gather_columns_kernel<2>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
-    case 3: F3M_LAUNCH((gather_columns_kernel<3>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
-    case 4: F3M_LAUNCH((gather_columns_kernel<4>), cdiv(n, 256), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 1: F3M_LAUNCH((gather_columns_kernel<1>), gather_grid(n, background), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 2: F3M_LAUNCH((gather_columns_kernel<2>), gather_grid(n, background), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 3: F3M_LAUNCH((gather_columns_kernel<3>), gather_grid(n, background), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
+    case 4: F3M_LAUNCH((gather_columns_kernel<4>), gather_grid(n, background), 256, 0, s, b, perm, n, c, col, bs, bstride); break;
     default: throw Error(34, "1 to 4 columns at a time");
     }
     check_launch("gather_columns");
 }
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s)
 {
-    gather_columns(b, perm, n, c, col, 1, bs, 0, s);
+    gather_columns(b, perm, n, c, col, 1, bs, 0, s, false);
 }
 
 // out[perm[i]][col + q] = outs[q][i] (+ outs2[q][i] if outs2 is given: the far field's share when it was computed

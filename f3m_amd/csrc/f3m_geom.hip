@@ -276,15 +276,20 @@ void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipS
 // bit j set when the point lies in the upper half along dimension j (sign table of
 // F3M_src/1_d_conv.cu:895-897), which makes the natural child index of the reference the digit.
 
+template <int K> struct __attribute__((aligned(4))) point_row { float v[K]; };   // K floats at any 4-byte boundary
+
+template <int D>
 __global__ void morton_kernel(const float *__restrict__ X, long long n, Geo g, uint32_t *__restrict__ keys, int *__restrict__ idx)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const float side = (float)(1u << g.L);
     const int top = (1 << g.L) - 1;
-    int cell[kMaxD];
-    for (int j = 0; j < g.d; j++) {
-        float a = X[i * g.d + j] - g.origin[j];
+    const point_row<D> row = *reinterpret_cast<const point_row<D> *>(X + i * D);   // the row with one request
+    int cell[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) {
+        float a = row.v[j] - g.origin[j];
         float q = side * a;
         q = q / g.edge0;
         int c = (int)floorf(q);
@@ -293,8 +298,9 @@ __global__ void morton_kernel(const float *__restrict__ X, long long n, Geo g, u
     uint32_t key = 0;
     for (int l = g.L - 1; l >= 0; l--) {
         uint32_t digit = 0;
-        for (int j = 0; j < g.d; j++) digit |= (uint32_t)((cell[j] >> l) & 1) << j;
-        key = (key << g.d) | digit;
+#pragma unroll
+        for (int j = 0; j < D; j++) digit |= (uint32_t)((cell[j] >> l) & 1) << j;
+        key = (key << D) | digit;
     }
     keys[i] = key;
     idx[i] = (int)i;
@@ -458,7 +464,16 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     t.n = n;
     t.keys.reset((size_t)n);
     t.perm.reset((size_t)n);
-    F3M_LAUNCH(morton_kernel, cdiv(n, 256), 256, 0, s, X, n, geo, t.keys.get(), t.perm.get());
+#define F3M_CASE(DD)                                                                                          \
+    case DD:                                                                                                  \
+        F3M_LAUNCH((morton_kernel<DD>), cdiv(n, 256), 256, 0, s, X, n, geo, t.keys.get(), t.perm.get());       \
+        break;
+    switch (geo.d) {
+        F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
+        F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
+    default: throw Error(2, "dimension must be 1..10");
+    }
+#undef F3M_CASE
     check_launch("morton");
     // Only the leading 16 key bits are sorted at first: a division at depth k looks at the leading d*k
     // bits, and most trees stop before d*k exceeds 16.  divide_tree sorts further bits when it gets there.
@@ -483,10 +498,10 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     check_launch("root_level");
 }
 
-void gather_tree_points(Tree &t, const float *X, hipStream_t s)
+void gather_tree_points(Tree &t, const float *X, hipStream_t s, bool background)
 {
     t.pts.reset((size_t)t.n * t.geo.d);
-    gather_points(X, t.perm.get(), t.n, t.geo.d, t.pts.get(), s);
+    gather_points(X, t.perm.get(), t.n, t.geo.d, t.pts.get(), s, background);
 }
 
 // ------------------------------------------------------------------------------------------------

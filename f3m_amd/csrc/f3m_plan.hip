@@ -314,15 +314,16 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         SideStream &ss = side_stream();
         F3M_HIP(hipEventRecord(ss.fork, s));
         F3M_HIP(hipStreamWaitEvent(ss.stream, ss.fork, 0));
-        gather_tree_points(P->tx, X, ss.stream);
-        if (!sym) gather_tree_points(P->ty_, Y, ss.stream);
+        gather_tree_points(P->tx, X, ss.stream, /*background=*/true);
+        if (!sym) gather_tree_points(P->ty_, Y, ss.stream, /*background=*/true);
         if (b_early != nullptr && c_early >= 1) {
             const long long bstride = P->M + 32;
             P->early_ncol = c_early >= 3 ? std::min(c_early, 4) : c_early;
             const int nc = c_early >= 3 ? 4 : c_early;
             P->early_bs.reset((size_t)bstride * (c_early >= 2 ? 4 : 1));
             if (nc > P->early_ncol) dev_fill(P->early_bs.get(), 0, sizeof(float) * (size_t)bstride * nc, ss.stream);
-            gather_columns(b_early, P->ty->perm.get(), P->M, c_early, 0, P->early_ncol, P->early_bs.get(), bstride, ss.stream);
+            gather_columns(b_early, P->ty->perm.get(), P->M, c_early, 0, P->early_ncol, P->early_bs.get(), bstride, ss.stream,
+                           /*background=*/true);
             P->early_b = b_early;
             P->early_c = c_early;
         }
