@@ -154,9 +154,14 @@ struct ListsPending {
     long long stride = 0;
     unsigned grid = 0;
     bool active = false;
+    bool written = false;    // the writing pass has been queued (lists_write_early)
 };
 void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
                   ListsPending &pend, long long *dtot, long long *drow /* 8 zeroed words or null */, hipStream_t s);
+// queues the writing pass before the sizes are known, into lists allocated for an upper bound of the pairs, if that
+// bound is modest (returns whether it did; lists_finish then only records the sizes)
+bool lists_write_early(ListsPending &pend, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                       const ClassifyParams &cp, PlanLevel &out, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
                   const ClassifyParams &cp, PlanLevel &out, const long long *hrow /* 8 words or null */, hipStream_t s);
 // out = `in` with the two boxes of every pair swapped, sorted by (by, bx) (a stable sort by `by` of a list that is

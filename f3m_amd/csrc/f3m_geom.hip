@@ -1021,32 +1021,18 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     }
 }
 
-void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
-                  const ClassifyParams &cp, PlanLevel &out, const long long *hrow, hipStream_t s)
+// allocates the small, far and keep list for cap[0..2] pairs and queues the writing pass
+static void lists_write(ListsPending &pend, const long long *cap, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                        const ClassifyParams &cp, PlanLevel &out, hipStream_t s)
 {
-    out.far.n = out.small_.n = out.keep.n = 0;
-    if (!pend.active) return;
-    if (hrow != nullptr) {
-        PairList &sm = out.small_, &kp = out.keep;
-        sm.rows = hrow[0], sm.row_points = hrow[1], sm.items128 = hrow[2], sm.items160 = hrow[3];
-        kp.rows = hrow[4], kp.row_points = hrow[5], kp.items128 = hrow[6], kp.items160 = hrow[7];
-    }
     const int d = tx.geo.d;
     const TreeLevel &py = ty.lev[k - 1];
     const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
     const bool one_tree = &tx == &ty;
     const int nbx = lx.nb;
-    for (int c = 0; c < 3; c++) F3M_REQUIRE(tot[c] < (1ll << 31) - 2, 22, "interaction list too long (%lld)", tot[c]);
-    out.far.outliers = one_tree ? tot[3] : -1;
-    out.far.beyond_tables = tot[6];
-    F3M_REQUIRE(tot[6] == 0, 24, "%lld far pairs of depth %d lie outside the M2L tables (cell offsets beyond %d per dimension)",
-                tot[6], k, kM2LOffsets);
-    out.small_.n = tot[0];
-    out.far.n = tot[1];
-    out.keep.n = tot[2];
-    out.small_.pairs.reset((size_t)std::max<long long>(1, tot[0]) * 2);
-    out.far.pairs.reset((size_t)std::max<long long>(1, tot[1]) * 2);
-    out.keep.pairs.reset((size_t)std::max<long long>(1, tot[2]) * 2);
+    out.small_.pairs.reset((size_t)std::max<long long>(1, cap[0]) * 2);
+    out.far.pairs.reset((size_t)std::max<long long>(1, cap[1]) * 2);
+    out.keep.pairs.reset((size_t)std::max<long long>(1, cap[2]) * 2);
     out.small_.rowptr.reset((size_t)pend.stride);
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
@@ -1066,6 +1052,48 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     }
 #undef F3M_CASE
     check_launch("lists_write");
+}
+
+// A list cannot be longer than the candidates of the level, at most 4^d children pairs per keep pair of the level
+// above, nor than all box pairs.  Where three lists of that many pairs are a modest allocation the writing pass is
+// queued before the host has seen the sizes (it runs while the host waits for them).
+constexpr long long kEarlyListBytes = 64ll << 20;       // per list
+bool lists_write_early(ListsPending &pend, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                       const ClassifyParams &cp, PlanLevel &out, hipStream_t s)
+{
+    pend.written = false;
+    if (!pend.active) return false;
+    const int d = tx.geo.d;
+    const long long per_keep = d <= 15 ? (1ll << (2 * d)) : (1ll << 30);
+    long long cap = (long long)tx.lev[k].nb * (long long)ty.lev[k].nb;
+    if (keep_prev.n <= cap / per_keep) cap = keep_prev.n * per_keep;
+    if (cap * 8 > kEarlyListBytes) return false;
+    const long long caps[3] = {cap, cap, cap};
+    lists_write(pend, caps, keep_prev, tx, ty, k, cp, out, s);
+    pend.written = true;
+    return true;
+}
+
+void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
+                  const ClassifyParams &cp, PlanLevel &out, const long long *hrow, hipStream_t s)
+{
+    out.far.n = out.small_.n = out.keep.n = 0;
+    if (!pend.active) return;
+    if (hrow != nullptr) {
+        PairList &sm = out.small_, &kp = out.keep;
+        sm.rows = hrow[0], sm.row_points = hrow[1], sm.items128 = hrow[2], sm.items160 = hrow[3];
+        kp.rows = hrow[4], kp.row_points = hrow[5], kp.items128 = hrow[6], kp.items160 = hrow[7];
+    }
+    const bool one_tree = &tx == &ty;
+    for (int c = 0; c < 3; c++) F3M_REQUIRE(tot[c] < (1ll << 31) - 2, 22, "interaction list too long (%lld)", tot[c]);
+    out.far.outliers = one_tree ? tot[3] : -1;
+    out.far.beyond_tables = tot[6];
+    F3M_REQUIRE(tot[6] == 0, 24, "%lld far pairs of depth %d lie outside the M2L tables (cell offsets beyond %d per dimension)",
+                tot[6], k, kM2LOffsets);
+    if (!pend.written) lists_write(pend, tot, keep_prev, tx, ty, k, cp, out, s);
+    out.small_.n = tot[0];
+    out.far.n = tot[1];
+    out.keep.n = tot[2];
     pend.pos.free();
     pend.active = false;
 }

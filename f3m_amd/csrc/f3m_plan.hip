@@ -275,7 +275,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     DBuf<long long> drow((size_t)8 * kMaxLevels);
     dev_fill(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s);
     alignas(8) int hres[32];
-    auto fetch_level = [&](const ListsPending *pend, bool division) {
+    SegmentFetch fetch;
+    auto fetch_level_begin = [&](const ListsPending *pend, bool division) {
         memset(hres, 0, sizeof(hres));
         ExportList L;
         if (pend != nullptr && pend->active) {
@@ -286,8 +287,9 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         }
         if (division) L.add(dres.get() + 8, sym ? 2 : 4, 8, true);
         if (division && pend == nullptr) L.add(dres.get() + 14, 2, 14, true);      // first division: fullest sorted cells
-        if (L.nseg > 0) fetch_segments(L, hres, s);
+        fetch.begin(L, s);
     };
+    auto fetch_level_wait = [&]() { fetch.wait(hres, s); };
     auto wants_division = [&]() {
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
@@ -354,7 +356,8 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             if (!sym) max_run_launch(P->ty_, dres.get() + 15, s);
         }
 #endif
-        fetch_level(nullptr, true);
+        fetch_level_begin(nullptr, true);
+        fetch_level_wait();
         finish_division();
 #ifndef F3M_CPU_EMU
         if (two_streams) {
@@ -384,7 +387,11 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)
             if (!ahead && early) prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
 #endif
-            fetch_level(&pend, ahead);
+            // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
+            // host has them, wherever an upper bound of the sizes is a modest allocation: it then runs during the wait.
+            fetch_level_begin(&pend, ahead);
+            lists_write_early(pend, *keep, P->tx, *P->ty, k, cp, L, s);
+            fetch_level_wait();
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
                          reinterpret_cast<const long long *>(hres + 16), s);
             if (ahead) finish_division();

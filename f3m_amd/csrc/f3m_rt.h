@@ -21,6 +21,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -257,6 +258,15 @@ inline void fetch_segments(const ExportList &L, void *dst, hipStream_t s)
     F3M_LAUNCH((export_segments_kernel<64>), 1, 64, 0, s, L, static_cast<unsigned *>(dst));
     F3M_HIP(hipStreamSynchronize(s));
 }
+// a readback in two steps (the emulation has nothing to overlap: begin does it all)
+class SegmentFetch {
+public:
+    void begin(const ExportList &L, hipStream_t s) { words_ = L.total; buf_.assign((size_t)L.total, 0u); if (L.nseg > 0) fetch_segments(L, buf_.data(), s); }
+    void wait(void *dst, hipStream_t) { if (words_ > 0) memcpy(dst, buf_.data(), (size_t)words_ * 4); words_ = 0; }
+private:
+    std::vector<unsigned> buf_;
+    int words_ = 0;
+};
 #else
 constexpr size_t kPinnedBytes = 64 << 10, kPinnedHeader = 64;
 constexpr int kSpinLimitMs = 50;
@@ -334,6 +344,35 @@ inline void fetch_segments(const ExportList &L, void *dst, hipStream_t s)
     await_flag(blk.flag(), seq, s);
     memcpy(dst, blk.data(), (size_t)L.total * 4);
 }
+// The same readback in two steps: begin queues the kernel that gathers the words into pinned memory, wait returns
+// them; kernels queued on the stream in between run while the host waits.
+class SegmentFetch {
+public:
+    void begin(const ExportList &L, hipStream_t s)
+    {
+        words_ = 0;
+        if (L.nseg == 0) return;
+        if ((size_t)L.total * 4 > kPinnedBytes) throw Error(103, "readback record too large");
+        blk_.reset(new PinnedBlock());
+        seq_ = blk_->next_seq();
+        hipLaunchKernelGGL(export_segments_flag_kernel<64>, dim3(1), dim3(64), 0, s, L, static_cast<unsigned *>(blk_->data()),
+                           blk_->flag(), seq_);
+        F3M_HIP(hipGetLastError());
+        words_ = L.total;
+    }
+    void wait(void *dst, hipStream_t s)
+    {
+        if (words_ == 0) return;
+        await_flag(blk_->flag(), seq_, s);
+        memcpy(dst, blk_->data(), (size_t)words_ * 4);
+        words_ = 0;
+        blk_.reset();
+    }
+private:
+    std::unique_ptr<PinnedBlock> blk_;
+    unsigned seq_ = 0;
+    int words_ = 0;
+};
 template <typename T>
 inline void fetch_small(T *dst, const T *src, size_t n, hipStream_t s)
 {
