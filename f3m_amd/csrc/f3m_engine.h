@@ -121,10 +121,15 @@ void timer_begin(int stage, hipStream_t s);
 void timer_end(hipStream_t s);
 
 // --- f3m_geom.hip ---
-void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s);
-// keys, order (perm) and the root level; the coordinates are gathered by gather_tree_points once
-// every division is done (divisions may still refine the order inside the boxes)
-void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s);
+// Root geometry without a host wait before the sort: partial minima and maxima per tree (bounding_box_launch), their
+// reduction to the minima of X, of Y and the root edge in device memory (root_geometry_launch: 2 kMaxD + 1 floats),
+// Morton keys and their sort from those values (sort_tree_launch); the host fetches the same values meanwhile and
+// sets up the root level with them (root_level_launch).  The coordinates are gathered by gather_tree_points once
+// the order is final (divisions may still refine the order inside the boxes).
+unsigned bounding_box_launch(const float *X, long long n, int d, DBuf<float> &part, hipStream_t s);
+void root_geometry_launch(const float *partx, unsigned gridx, const float *party, unsigned gridy, int d, float *out, hipStream_t s);
+void sort_tree_launch(Tree &t, const float *X, long long n, int d, int L, const float *origin, const float *edge0p, hipStream_t s);
+void root_level_launch(Tree &t, const Geo &geo, hipStream_t s);
 void gather_tree_points(Tree &t, const float *X, hipStream_t s, bool background = false);
 // One division in two steps, so that the host can wait once for several results: divide_launch starts
 // the kernels that build lev[k] from lev[k-1] and appends the level; divide_finish completes it with

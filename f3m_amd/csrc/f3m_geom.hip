@@ -247,25 +247,66 @@ __global__ void __launch_bounds__(256) minmax_kernel(const float *__restrict__ X
     }
 }
 
-void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipStream_t s)
+// queues the partial minima and maxima of X (per workgroup and dimension) into `part`; returns their number
+unsigned bounding_box_launch(const float *X, long long n, int d, DBuf<float> &part, hipStream_t s)
 {
     const int prefix = (int)(((16 - reinterpret_cast<uintptr_t>(X) % 16) % 16) / 4);
     unsigned grid = (unsigned)d * kBBBlocksPerDim;                      // threads = 256 * grid: a multiple of d
     const unsigned need = cdiv(cdiv(n * d, 4), 256);
     if (need < grid) grid = (unsigned)d * std::max(1u, cdiv(need, d));
-    DBuf<float> part((size_t)grid * 2 * kMaxD);
+    part.reset((size_t)grid * 2 * kMaxD);
     F3M_LAUNCH(minmax_kernel, grid, 256, 0, s, X, n * d, d, std::min<long long>(prefix, n * d), part.get());
     check_launch("minmax");
-    std::vector<float> h((size_t)grid * 2 * kMaxD);
-    fetch_small(h.data(), part.get(), h.size(), s);
-    for (int j = 0; j < d; j++) {
-        mn[j] = h[j];
-        mx[j] = h[kMaxD + j];
-        for (unsigned b = 1; b < grid; b++) {
-            mn[j] = fminf(mn[j], h[((size_t)b * 2) * kMaxD + j]);
-            mx[j] = fmaxf(mx[j], h[((size_t)b * 2 + 1) * kMaxD + j]);
+    return grid;
+}
+
+// Root geometry on the device (F3M_src/n_tree.cu:25-46): per tree and dimension the minimum over the partial
+// results, the edge = largest extent over both trees, times 1.01.  out: minima of X (kMaxD), minima of Y (kMaxD; of X
+// again for one tree), edge0.  The Morton keys are computed from these values without the host having seen them.
+__global__ void __launch_bounds__(2 * kMaxD * 32) root_geometry_kernel(const float *__restrict__ partx, unsigned gridx,
+                                                                       const float *__restrict__ party, unsigned gridy, int d,
+                                                                       float *__restrict__ out)
+{
+    // 32 lanes per (tree, dimension): strided over the partial results, then combined inside the half wavefront
+    // (minimum and maximum do not depend on the order)
+    __shared__ float smn[2][kMaxD], smx[2][kMaxD];
+    const int combo = threadIdx.x / 32, sub = threadIdx.x % 32;
+    const int tree = combo / kMaxD, j = combo % kMaxD;
+    const float *part = (tree && party) ? party : partx;
+    const unsigned grid = (tree && party) ? gridy : gridx;
+    float mn = part[j < d ? j : 0], mx = part[kMaxD + (j < d ? j : 0)];          // the first block's: every lane starts there
+    if (j < d)
+        for (unsigned b = sub; b < grid; b += 32) {
+            mn = fminf(mn, part[((size_t)b * 2) * kMaxD + j]);
+            mx = fmaxf(mx, part[((size_t)b * 2 + 1) * kMaxD + j]);
         }
+#pragma unroll
+    for (int m = 16; m >= 1; m >>= 1) {
+        mn = fminf(mn, wave_shfl_xor_f(mn, m));
+        mx = fmaxf(mx, wave_shfl_xor_f(mx, m));
     }
+    if (sub == 0 && j < d) {
+        smn[tree][j] = mn;
+        smx[tree][j] = mx;
+        out[tree * kMaxD + j] = mn;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float e = smx[0][0] - smn[0][0];
+        for (int k = 1; k < d; k++) { const float r = smx[0][k] - smn[0][k]; if (r > e) e = r; }
+        if (party) {
+            float ye = smx[1][0] - smn[1][0];
+            for (int k = 1; k < d; k++) { const float r = smx[1][k] - smn[1][k]; if (r > ye) ye = r; }
+            if (ye > e) e = ye;
+        }
+        out[2 * kMaxD] = e * 1.01f;
+    }
+}
+
+void root_geometry_launch(const float *partx, unsigned gridx, const float *party, unsigned gridy, int d, float *out, hipStream_t s)
+{
+    F3M_LAUNCH(root_geometry_kernel, 1, 2 * kMaxD * 32, 0, s, partx, gridx, party, gridy, d, out);
+    check_launch("root_geometry");
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -278,20 +319,24 @@ void bounding_box(const float *X, long long n, int d, float *mn, float *mx, hipS
 
 template <int K> struct __attribute__((aligned(4))) point_row { float v[K]; };   // K floats at any 4-byte boundary
 
+// origin (D floats) and edge0 are read from device memory: the root geometry need not have reached the host
 template <int D>
-__global__ void morton_kernel(const float *__restrict__ X, long long n, Geo g, uint32_t *__restrict__ keys, int *__restrict__ idx)
+__global__ void morton_kernel(const float *__restrict__ X, long long n, const float *__restrict__ origin,
+                              const float *__restrict__ edge0p, int L, uint32_t *__restrict__ keys, int *__restrict__ idx)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
+    struct { int L; } g{L};
+    const float edge0 = *edge0p;
     const float side = (float)(1u << g.L);
     const int top = (1 << g.L) - 1;
     const point_row<D> row = *reinterpret_cast<const point_row<D> *>(X + i * D);   // the row with one request
     int cell[D];
 #pragma unroll
     for (int j = 0; j < D; j++) {
-        float a = row.v[j] - g.origin[j];
+        float a = row.v[j] - origin[j];
         float q = side * a;
-        q = q / g.edge0;
+        q = q / edge0;
         int c = (int)floorf(q);
         cell[j] = c < 0 ? 0 : (c > top ? top : c);
     }
@@ -458,17 +503,17 @@ __global__ void root_level_kernel(Geo g, int n, int *__restrict__ off, uint32_t 
     }
 }
 
-void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hipStream_t s)
+// keys and their order from the root geometry in device memory (origin: d floats, edge0p: one)
+void sort_tree_launch(Tree &t, const float *X, long long n, int d, int L, const float *origin, const float *edge0p, hipStream_t s)
 {
-    t.geo = geo;
     t.n = n;
     t.keys.reset((size_t)n);
     t.perm.reset((size_t)n);
-#define F3M_CASE(DD)                                                                                          \
-    case DD:                                                                                                  \
-        F3M_LAUNCH((morton_kernel<DD>), cdiv(n, 256), 256, 0, s, X, n, geo, t.keys.get(), t.perm.get());       \
+#define F3M_CASE(DD)                                                                                                    \
+    case DD:                                                                                                            \
+        F3M_LAUNCH((morton_kernel<DD>), cdiv(n, 256), 256, 0, s, X, n, origin, edge0p, L, t.keys.get(), t.perm.get());   \
         break;
-    switch (geo.d) {
+    switch (d) {
         F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
         F3M_CASE(6) F3M_CASE(7) F3M_CASE(8) F3M_CASE(9) F3M_CASE(10)
     default: throw Error(2, "dimension must be 1..10");
@@ -477,9 +522,15 @@ void build_sorted_tree(Tree &t, const float *X, long long n, const Geo &geo, hip
     check_launch("morton");
     // Only the leading 16 key bits are sorted at first: a division at depth k looks at the leading d*k
     // bits, and most trees stop before d*k exceeds 16.  divide_tree sorts further bits when it gets there.
-    t.sorted_from = std::max(0, geo.d * geo.L - 16);
-    radix_sort(t.keys, t.perm, n, t.sorted_from, geo.d * geo.L, s);
-    // root level (F3M_src/n_tree.cu:86-95)
+    t.sorted_from = std::max(0, d * L - 16);
+    radix_sort(t.keys, t.perm, n, t.sorted_from, d * L, s);
+}
+
+// the root level, once the host has the geometry (F3M_src/n_tree.cu:86-95)
+void root_level_launch(Tree &t, const Geo &geo, hipStream_t s)
+{
+    t.geo = geo;
+    const long long n = t.n;
     t.lev.clear();
     t.lev.reserve(40);
     t.lev.emplace_back();

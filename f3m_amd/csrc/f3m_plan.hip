@@ -147,13 +147,6 @@ static void check_device_ptr(const void *p, const char *name)
 #endif
 }
 
-static float root_edge(const float *mn, const float *mx, int d)
-{
-    float e = mx[0] - mn[0];
-    for (int j = 1; j < d; j++) { float r = mx[j] - mn[j]; if (r > e) e = r; }
-    return e;
-}
-
 static ClassifyParams classify_params(const f3m_plan &P, float edge)
 {
     ClassifyParams cp;
@@ -225,28 +218,33 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     Geo gx;
     memset(&gx, 0, sizeof(gx));
     if (need_tree) {
-        // root geometry (F3M_src/n_tree.cu:25-46)
-        float xmn[kMaxD], xmx[kMaxD], ymn[kMaxD], ymx[kMaxD];
-        bounding_box(X, N, d, xmn, xmx, s);
-        float edge = root_edge(xmn, xmx, d);
-        if (!sym) {
-            bounding_box(Y, M, d, ymn, ymx, s);
-            float ye = root_edge(ymn, ymx, d);
-            if (ye > edge) edge = ye;
-        }
+        // Root geometry (F3M_src/n_tree.cu:25-46), reduced on the device: the Morton keys and their sort are queued
+        // behind it and run while the same values travel to the host, which needs them from the root level on.
+        DBuf<float> partx, party, dgeo((size_t)2 * kMaxD + 1);
+        const unsigned npx = bounding_box_launch(X, N, d, partx, s);
+        const unsigned npy = sym ? 0u : bounding_box_launch(Y, M, d, party, s);
+        root_geometry_launch(partx.get(), npx, sym ? nullptr : party.get(), npy, d, dgeo.get(), s);
+        ExportList G;
+        G.add(dgeo.get(), 2 * kMaxD + 1, 0);
+        SegmentFetch geo_fetch;
+        geo_fetch.begin(G, s);
         gx.d = d;
-        gx.edge0 = edge * 1.01f;
-        F3M_REQUIRE(std::isfinite(gx.edge0), 10, "point coordinates are not finite");
         // key depth: past 31/d levels the reference's int32 grid keys overflow, past 16 its fp32
         // centres stop resolving cells; the tree is never deeper and what is left is summed exactly
         gx.L = std::min(31 / d, 16);
+        sort_tree_launch(P->tx, X, N, d, gx.L, dgeo.get(), dgeo.get() + 2 * kMaxD, s);
+        if (!sym) sort_tree_launch(P->ty_, Y, M, d, gx.L, dgeo.get() + kMaxD, dgeo.get() + 2 * kMaxD, s);
+        float hgeo[2 * kMaxD + 1];
+        geo_fetch.wait(hgeo, s);
+        gx.edge0 = hgeo[2 * kMaxD];
+        F3M_REQUIRE(std::isfinite(gx.edge0), 10, "point coordinates are not finite");
         if (gx.edge0 > 0.f) {
             Geo gy = gx;
-            for (int j = 0; j < d; j++) { gx.origin[j] = xmn[j]; gy.origin[j] = sym ? xmn[j] : ymn[j]; }
-            build_sorted_tree(P->tx, X, N, gx, s);
-            if (!sym) build_sorted_tree(P->ty_, Y, M, gy, s);
+            for (int j = 0; j < d; j++) { gx.origin[j] = hgeo[j]; gy.origin[j] = hgeo[kMaxD + j]; }
+            root_level_launch(P->tx, gx, s);
+            if (!sym) root_level_launch(P->ty_, gy, s);
         } else {
-            need_tree = false;
+            need_tree = false;      // every point at one place: the sort that was queued is simply not used
         }
     }
 
