@@ -1182,7 +1182,7 @@ __global__ void __launch_bounds__(64) p2m_q64_kernel(const float *__restrict__ y
             basis4(t, tn[k], tw[k], l[k], 1.f);
         }
         const float b = in ? bs[i] : 0.f;            // lanes past the end add nothing
-        __syncthreads();                             // the previous round has been read
+        __syncthreads();                             // the previous 64 points have been read by every lane
         *reinterpret_cast<float4 *>(sl0 + 4 * lane) = make_float4(l[0][0], l[0][1], l[0][2], l[0][3]);
         float *wrow = sw + 16 * lane + 16 * (lane >> 4);
 #pragma unroll
@@ -1245,7 +1245,7 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
             basis_1d(t, nt + N * k, nw + N * k, N, l[k], 1.f);
         }
         const float b = in ? bs[i] : 0.f;            // lanes past the end add nothing
-        __syncthreads();                             // the previous round has been read
+        __syncthreads();                             // the previous 64 points have been read by every lane
         // products over a range of dimensions, built dimension by dimension from the last (first one fastest)
         float h[NR], w[Q];
         h[0] = 1.f;
