@@ -326,10 +326,9 @@ __global__ void morton_kernel(const float *__restrict__ X, long long n, const fl
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    struct { int L; } g{L};
     const float edge0 = *edge0p;
-    const float side = (float)(1u << g.L);
-    const int top = (1 << g.L) - 1;
+    const float side = (float)(1u << L);
+    const int top = (1 << L) - 1;
     const point_row<D> row = *reinterpret_cast<const point_row<D> *>(X + i * D);   // the row with one request
     int cell[D];
 #pragma unroll
@@ -341,7 +340,7 @@ __global__ void morton_kernel(const float *__restrict__ X, long long n, const fl
         cell[j] = c < 0 ? 0 : (c > top ? top : c);
     }
     uint32_t key = 0;
-    for (int l = g.L - 1; l >= 0; l--) {
+    for (int l = L - 1; l >= 0; l--) {
         uint32_t digit = 0;
 #pragma unroll
         for (int j = 0; j < D; j++) digit |= (uint32_t)((cell[j] >> l) & 1) << j;
