@@ -36,5 +36,22 @@ def build(force=False, sanitize=False):
     return OUT
 
 
+def build_sanitize_driver():
+    """tests/cpu_emu/sanitize_driver.cpp and the kernel sources in one executable under AddressSanitizer and
+    UndefinedBehaviorSanitizer (an executable, so that the sanitizer runtime comes first without preloading anything).
+    Takes a minute or two to compile."""
+    out = os.path.join(HERE, "_build", "sanitize_driver")
+    srcs = [os.path.join(CSRC, s) for s in SRCS]
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    flags = ["-O1", "-g", "-std=c++17", "-DF3M_CPU_EMU", "-fsanitize=address,undefined", "-fno-omit-frame-pointer",
+             "-fno-sanitize-recover=undefined", "-ffp-contract=off", "-I", HERE, "-I", CSRC, "-w"]
+    cmd = ["g++"] + flags
+    for s in srcs:
+        cmd += ["-x", "c++", s]
+    cmd += ["-x", "c++", os.path.join(HERE, "sanitize_driver.cpp"), "-o", out, "-lpthread"]
+    subprocess.check_call(cmd)
+    return out
+
+
 if __name__ == "__main__":
     print(build(force=True))
