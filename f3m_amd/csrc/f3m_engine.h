@@ -222,8 +222,9 @@ void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
 void mark_far_boxes(const PairList &far, int nbx, int nby, int *fx, int *fy, hipStream_t s);
 void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, NodeSet &ns, const float *bs, float *mom,
                hipStream_t s);
+// beside_near: the launch will run beside the near field of another stream (small workgroups then)
 void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
-               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc /* overwritten */, hipStream_t s);
+               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc /* overwritten */, hipStream_t s, bool beside_near = false);
 void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
                hipStream_t s);
 // expansions moved between a level and the next deeper one: moments up (down = false, dst = parent

@@ -2035,7 +2035,7 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
 }
 
 void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
-               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc, hipStream_t s)
+               NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc, hipStream_t s, bool beside_near)
 {
     check_nodes(ns);
     const int P = ns.P;
@@ -2086,6 +2086,12 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             if (sibR2 <= 1024) {
                 sibGS = 1 << d;
                 while (sibGS * sibR2 > 1024) sibGS >>= 1;
+                // Beside the near field (whose wavefronts keep every compute unit full) only small workgroups find room:
+                // from four dimensions on, groups of four siblings then, one or two wavefronts (N=1e7: 4-D 15.1 -> 14.85 ms,
+                // 5-D 53.4 -> 51.8 ms per product; groups of eight: 14.9 and 54.8; alone on the GPU the whole family in
+                // one workgroup is faster, 2.1 against 3.0 ms in 4-D).
+                if (beside_near && d >= 4)
+                    while (sibGS > 4 || (sibGS > 1 && sibGS * sibR2 > 2 * kWave)) sibGS >>= 1;
                 // 3-D: 8 siblings x n2 lanes fill at most half a wavefront; two lanes then share a lane's nodes
                 const char *nosplit = getenv("F3M_SIB_SPLIT");   // F3M_SIB_SPLIT=0: testing aid
                 if (d == 3 && N % 2 == 0 && sibGS * sibR2 <= kWave / 2 && !(nosplit && atoi(nosplit) == 0)) { sibH = 2; sibR2 *= 2; }

@@ -461,7 +461,7 @@ static void far_level(f3m_plan *P, int level, const float *bs, float *outs, floa
 // Where a level has more nodes per dimension than the next deeper one (var_compression lowers the node
 // count of small boxes, F3M_src/n_tree.cu:971-978) the hand-over would not be exact, and that level
 // is interpolated from / evaluated at the points directly, as the reference does for every level.
-static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs, hipStream_t s)
+static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs, hipStream_t s, bool beside_near = false)
 {
     const int depth = (int)P->levels.size();
     // targets and sources of this product: the X and Y tree, or the other way round for K(X,Y)^T
@@ -494,7 +494,7 @@ static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs,
         NodeSet &ns = ns_of(k);
         const TreeLevel &lx = TX.lev[k];
         loc.reset((size_t)lx.nb * ns.P);
-        m2l_level(d, TX, lx, TY, TY.lev[k], far_of(k), ns, P->lcs, mode, mom[k].get(), loc.get(), s);
+        m2l_level(d, TX, lx, TY, TY.lev[k], far_of(k), ns, P->lcs, mode, mom[k].get(), loc.get(), s, beside_near);
         mom[k].free();
         if (pending) {
             NodeSet &nsp = ns_of(pending);
@@ -656,7 +656,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
 #ifndef F3M_CPU_EMU
                 if (overlap) { fs = side_stream().stream; fo = outs_far.get(); }
 #endif
-                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs);
+                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap);
             }
 #ifndef F3M_CPU_EMU
             if (overlap) {
