@@ -472,6 +472,14 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
     int b0 = box32[min(i0, M - 1) / 32], b0m = box32[pm / 32];
     while (off[b0 + 1] <= min(i0, M - 1)) b0++;      // at most the boxes that start inside 32 points
     while (off[b0m + 1] <= pm) b0m++;
+    if (need != nullptr) {
+        // no box between the one 31 points before this workgroup's first point and the one of its last point is
+        // wanted: nothing to do (a list of a shallow level names a few boxes, the launch covers every point)
+        const long long il = min(i0 + kOpsBlock - 1, M - 1);
+        int bl = box32[il / 32];
+        while (off[bl + 1] <= il) bl++;
+        if (need[bl + 1] - need[b0m] == 0) return;
+    }
     bounds[tid] = off[min(b0 + 1 + tid, nb)];       // starts of the following boxes; off[nb] = M closes the list
     __syncthreads();
     if (i >= stride) return;
