@@ -94,6 +94,7 @@ struct f3m_plan {
     DBuf<float> Xraw, Yraw;                // row-major copies, only when no division happened
     // one-shot products: the first column group of b, already in sorted order (gathered while the lists were built)
     DBuf<float> early_bs;
+    DBuf<float> early_outs, early_outs_far;   // the result arrays of that column group, cleared beside the last level's lists
     const float *early_b = nullptr;
     int early_c = 0, early_ncol = 0;
     std::map<std::pair<int, int>, std::unique_ptr<DBuf<float>>> shift_tabs;   // (parent nodes, child nodes)
@@ -383,7 +384,16 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             // No further division: this is the deepest level, whose near lists will be summed.  Its source operands
             // are prepared on the second stream (behind the moves of the points) while its lists are built here.
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)
-            if (!ahead && early) prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
+            if (!ahead && early) {
+                prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
+                if (P->early_b != nullptr) {       // and the result arrays of the product that follows are cleared there
+                    const int nc = P->early_c >= 3 ? 4 : P->early_c;
+                    P->early_outs.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
+                    P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
+                    dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
+                    dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
+                }
+            }
 #endif
             // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
             // host has them, wherever an upper bound of the sizes is a modest allocation: it then runs during the wait.
@@ -606,16 +616,26 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         const int ncol = std::min(nc, left);
         {
             Scope sc(kPerm, s);
+            bool cleared = false;
             if (col == 0 && !transposed && P->early_b == b && P->early_c == c && P->early_ncol == ncol && P->early_bs.size() > 0) {
                 std::swap(bs, P->early_bs);                 // this group's weights were put in order while the plan was built
                 P->early_b = nullptr;
                 P->early_bs.free();
+                if (P->early_outs.size() > 0) {             // and its result arrays cleared
+                    std::swap(outs, P->early_outs);
+                    if (overlap) std::swap(outs_far, P->early_outs_far);
+                    P->early_outs.free();
+                    P->early_outs_far.free();
+                    cleared = true;
+                }
             } else {
                 if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
                 gather_columns(b, TY.perm.get(), NS, c, col, ncol, bs.get(), bstride, s);
             }
-            dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
-            if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
+            if (!cleared) {
+                dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
+                if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
+            }
         }
         // Every temporary that is given back while this column group is being queued is parked until the streams
         // have joined: work queued on one stream may still use a block when host code of the other asks for memory.
