@@ -148,6 +148,16 @@ static void check_device_ptr(const void *p, const char *name)
 #endif
 }
 
+// start of a plan: the root pair (0,0), its row pointers (0,1), and zeroed counters
+__global__ void plan_init_kernel(int *__restrict__ pair, int *__restrict__ rowptr, int *__restrict__ counters, int ncounters,
+                                 int *__restrict__ stats, int nstats)
+{
+    const int t = threadIdx.x;
+    if (t < 2) { pair[t] = 0; rowptr[t] = t; }
+    for (int i = t; i < ncounters; i += blockDim.x) counters[i] = 0;
+    for (int i = t; i < nstats; i += blockDim.x) stats[i] = 0;
+}
+
 static ClassifyParams classify_params(const f3m_plan &P, float edge)
 {
     ClassifyParams cp;
@@ -249,11 +259,18 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         }
     }
 
+    // The root pair (0,0) with its row pointers (0,1), and the counters of the level loop, all cleared by one kernel:
+    // [0..1] pair, [2..3] row pointers, [4..19] counters of a level (dres), then eight 64-bit row statistics per level (drow)
+    constexpr int kMaxLevels = 40;
     PairList root;
     root.n = 1;
     root.pairs.reset(2);
-    dev_fill(root.pairs.get(), 0, 2 * sizeof(int), s);     // the root pair (0,0)
-    build_rowptr(root, 1, s);
+    root.rowptr.reset(2);
+    DBuf<int> dres(16);
+    DBuf<long long> drow((size_t)8 * kMaxLevels);
+    F3M_LAUNCH(plan_init_kernel, 1, 64, 0, s, root.pairs.get(), root.rowptr.get(), dres.get(), 16,
+               reinterpret_cast<int *>(drow.get()), 2 * 8 * kMaxLevels);
+    check_launch("plan_init");
     const PairList *keep = &root;
     P->levels.reserve(64);   // `keep` points into this vector: it must not reallocate
     // Loop of F3M_src/n_tree.cu:1075 (one tree) and :1099 (two trees): divide while the keep list is not
@@ -268,11 +285,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // 64-bit words: what the near field needs to shape its launches).  On the device the first three are the last
     // entries of the list builder's scans; the counters behind [6..15] live in dres and are cleared by the readback
     // that fetches them, the row statistics in drow, eight words per level.
-    DBuf<int> dres(16);
-    dev_fill(dres.get(), 0, 16 * sizeof(int), s);
-    constexpr int kMaxLevels = 40;
-    DBuf<long long> drow((size_t)8 * kMaxLevels);
-    dev_fill(drow.get(), 0, sizeof(long long) * 8 * kMaxLevels, s);
     alignas(8) int hres[32];
     SegmentFetch fetch;
     auto fetch_level_begin = [&](const ListsPending *pend, bool division) {
