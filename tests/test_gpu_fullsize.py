@@ -46,3 +46,23 @@ def test_n1e7_properties(name):
     assert err <= bound
     if meets:
         assert err <= 1e-3
+
+
+def test_n1e7_variance_compression():
+    """The reference's FALKON experiments run the operator with var_compression=True (experiments/
+    experiments_krr_a.py): the extra far-field shortcuts at full size, lengthscales 3 and 1 on the unit cube.  The
+    product stays within 1e-4 of the fp64 exact product on seeded rows (measured 1.8e-6 and 3.6e-5)."""
+    import torch
+    from f3m_amd import engine
+    print("case N=1e7 var_compression", flush=True)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    X = torch.rand(N, 3, generator=g, device="cuda")
+    b = torch.randn(N, 1, generator=g, device="cuda")
+    rows = torch.randint(0, N, (5000,), generator=torch.Generator().manual_seed(1)).cuda()
+    for ls, limit in ((3.0, 0.3), (1.0, 0.15)):
+        out = engine.kmvm(X, None, b, ls=ls, var_compression=True, eff_var_limit=limit)
+        assert torch.isfinite(out).all()
+        exact = engine.exact_f64(X[rows].contiguous(), X, b, ls)
+        err = rel_l2(out[rows].cpu().numpy(), exact.cpu().numpy())
+        print("ls=%g: rel-L2 on 5000 rows %.3e" % (ls, err), flush=True)
+        assert err < 1e-4
