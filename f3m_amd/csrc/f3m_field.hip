@@ -748,8 +748,19 @@ __global__ void near_reduce_kernel(const float *__restrict__ part, int nsplit, i
     const int i = offx[bx] + (wid - tileoff[bx]) * tile + r;
     if (i >= offx[bx + 1]) return;
     for (int c = 0; c < nc; c++) {
+        // slices in their order, eight loads in flight at a time (the loads do not depend on each other, the sum does)
+        const float *p = part + ((long long)c * nitems + wid) * tile + r;
+        const long long step = (long long)nc * nitems * tile;
         float sum = 0.f;
-        for (int sl = 0; sl < nsplit; sl++) sum += part[(((long long)sl * nc + c) * nitems + wid) * tile + r];
+        int sl = 0;
+        for (; sl + 8 <= nsplit; sl += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = p[(sl + u) * step];
+#pragma unroll
+            for (int u = 0; u < 8; u++) sum += v[u];
+        }
+        for (; sl < nsplit; sl++) sum += p[sl * step];
         outs[c * ostride + i] += sum;
     }
 }
