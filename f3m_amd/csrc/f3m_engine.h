@@ -169,6 +169,8 @@ bool lists_write_early(ListsPending &pend, const PairList &keep_prev, const Tree
                        const ClassifyParams &cp, PlanLevel &out, hipStream_t s);
 void lists_finish(ListsPending &pend, const long long *htot, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,
                   const ClassifyParams &cp, PlanLevel &out, const long long *hrow /* 8 words or null */, hipStream_t s);
+// moves lists that fill a small part of the block they were written into (lists_write_early) into blocks of their size
+void shrink_lists(PlanLevel &L, hipStream_t s);
 // out = `in` with the two boxes of every pair swapped, sorted by (by, bx) (a stable sort by `by` of a list that is
 // sorted by bx), its row pointers over the nby boxes of the Y level, and its row statistics for the near field
 void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipStream_t s);

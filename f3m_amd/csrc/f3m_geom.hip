@@ -1141,11 +1141,33 @@ void lists_finish(ListsPending &pend, const long long *tot, const PairList &keep
     F3M_REQUIRE(tot[6] == 0, 24, "%lld far pairs of depth %d lie outside the M2L tables (cell offsets beyond %d per dimension)",
                 tot[6], k, kM2LOffsets);
     if (!pend.written) lists_write(pend, tot, keep_prev, tx, ty, k, cp, out, s);
+    else {
+        // written ahead of the sizes into lists allocated for an upper bound: the bound must have held
+        const PairList *wl[3] = {&out.small_, &out.far, &out.keep};
+        for (int c = 0; c < 3; c++)
+            F3M_REQUIRE((size_t)tot[c] * 2 <= wl[c]->pairs.size(), 25, "interaction list of depth %d longer (%lld pairs) than its bound (%zu)",
+                        k, tot[c], wl[c]->pairs.size() / 2);
+    }
     out.small_.n = tot[0];
     out.far.n = tot[1];
     out.keep.n = tot[2];
     pend.pos.free();
     pend.active = false;
+}
+
+// Lists that were written ahead of their sizes sit in blocks allocated for an upper bound (up to 64 MiB per list).  A
+// plan that is kept gives the surplus back: a list that fills less than half of a block of more than 1 MiB moves into
+// a block of its own size.
+void shrink_lists(PlanLevel &L, hipStream_t s)
+{
+    PairList *wl[3] = {&L.small_, &L.far, &L.keep};
+    for (PairList *l : wl) {
+        const size_t need = (size_t)std::max<long long>(1, l->n) * 2;
+        if (l->pairs.size() * sizeof(int) <= ((size_t)1 << 20) || need * 2 > l->pairs.size()) continue;
+        DBuf<int> fit(need);
+        F3M_HIP(hipMemcpyAsync(fit.get(), l->pairs.get(), need * sizeof(int), hipMemcpyDeviceToDevice, s));
+        std::swap(l->pairs, fit);       // the old block goes back to the pool; work queued later on this stream may reuse it
+    }
 }
 
 }  // namespace f3m

@@ -448,7 +448,11 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             F3M_HIP(hipMemcpyAsync(P->Yraw.get(), Y, sizeof(float) * (size_t)M * d, hipMemcpyDeviceToDevice, s));
         }
     }
-    if (b_early == nullptr) F3M_HIP(hipStreamSynchronize(s));
+    if (b_early == nullptr) {
+        // a plan that is kept: lists written into blocks sized for an upper bound move into blocks of their own size
+        for (PlanLevel &L : P->levels) shrink_lists(L, s);
+        F3M_HIP(hipStreamSynchronize(s));
+    }
     return P.release();
 }
 
@@ -622,7 +626,13 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             }
         for (int k = same_nodes ? kd : ku; k <= kd; k++) ensure_box_table(TX.lev[k], NT, s);
     }
+    // A call whose temporaries come from an arena runs on one stream, so the temporaries of a column group (and of one
+    // column's far field) can take the place of the previous one's: the need does not grow with the number of columns,
+    // and the first group, which has the most columns, is the one that decides whether the product fits -- before
+    // anything has been written to `out`.
+    const size_t group_mark = arena_mark();
     for (int col = 0; col < c;) {
+        arena_rewind(group_mark);
         const int left = c - col;
         const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);   // columns of this pass (past `left`: zero weights)
         const int ncol = std::min(nc, left);
@@ -673,9 +683,13 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
                 near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
                            bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0);
-                if (per_level)
-                    for (int q = 0; q < ncol; q++)
+                if (per_level) {
+                    const size_t mark = arena_mark();
+                    for (int q = 0; q < ncol; q++) {
+                        arena_rewind(mark);
                         far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
+                    }
+                }
             }
             // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
             near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
@@ -688,7 +702,11 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
 #ifndef F3M_CPU_EMU
                 if (overlap) { fs = side_stream().stream; fo = outs_far.get(); }
 #endif
-                for (int q = 0; q < ncol; q++) far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap);
+                const size_t mark = arena_mark();
+                for (int q = 0; q < ncol; q++) {
+                    arena_rewind(mark);
+                    far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap);
+                }
             }
 #ifndef F3M_CPU_EMU
             if (overlap) {
@@ -706,10 +724,16 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
 
 // A call that fails may have queued work on the caller's stream and on the library's second stream, and the
 // buffers of that work have gone back to the pool while the error travelled up here: nothing may reuse them before
-// the device is idle.
+// the device is idle.  Not while the call's stream is being captured into a graph: nothing has run then, a device-wide
+// wait is an error during capture (and would invalidate it), and such a call takes its temporaries from static memory.
+static thread_local hipStream_t g_call_stream = nullptr;
 static void settle_after_error()
 {
 #ifndef F3M_CPU_EMU
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const bool capturing = hipStreamIsCapturing(g_call_stream, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+    (void)hipGetLastError();
+    if (capturing) return;
     (void)hipDeviceSynchronize();
     (void)hipGetLastError();
 #endif
@@ -865,7 +889,8 @@ static void *scratch_address()
 
 int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream)
 {
-    return guarded([&] {
+    g_call_stream = (hipStream_t)stream;
+    const int rc = guarded([&] {
         F3M_REQUIRE(plan != nullptr, 1, "plan is NULL");
         F3M_REQUIRE(c >= 1, 12, "b has no columns");
         // what the call needs at the least: the sorted copies of b and of the result
@@ -889,6 +914,8 @@ int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, vo
         }
         g_timer.enabled = timing;
     });
+    g_call_stream = nullptr;
+    return rc;
 }
 
 int f3m_plan_destroy(f3m_plan *plan)

@@ -88,6 +88,11 @@ struct ArenaScope {
     ArenaScope(const ArenaScope &) = delete;
     ArenaScope &operator=(const ArenaScope &) = delete;
 };
+// Position of the calling thread's arena, and a return to it: what was handed out since is handed out again.  Only for
+// temporaries whose kernels are all queued on one stream (a later kernel then reuses the memory after the earlier ones
+// are done) and whose host-side owners are gone.  No-ops without an arena.
+inline size_t arena_mark() { return g_arena != nullptr ? g_arena->used : 0; }
+inline void arena_rewind(size_t mark) { if (g_arena != nullptr) g_arena->used = mark; }
 inline void require_tables_may_be_built(const char *what)
 {
     if (g_arena != nullptr)
@@ -354,6 +359,7 @@ public:
         if (L.nseg == 0) return;
         if ((size_t)L.total * 4 > kPinnedBytes) throw Error(103, "readback record too large");
         blk_.reset(new PinnedBlock());
+        memset(blk_->data(), 0, (size_t)L.total * 4);      // words between the segments read as zero, not as what the block held before
         seq_ = blk_->next_seq();
         hipLaunchKernelGGL(export_segments_flag_kernel<64>, dim3(1), dim3(64), 0, s, L, static_cast<unsigned *>(blk_->data()),
                            blk_->flag(), seq_);

@@ -71,13 +71,20 @@ int f3m_plan_destroy(f3m_plan *plan);
 /* f3m_plan_apply without any device allocation.  No counterpart in the reference: it is for callers that
  * cannot allocate (a stream under HIP graph capture, a serving loop that must not touch the allocator, a
  * harness that forbids hipMalloc).  Same arguments and result as f3m_plan_apply.  Its temporaries live in
- * 128 MiB of static device memory that every GPU running the library holds until the process ends; a
- * product that needs more (roughly 4 (N + M) bytes per column group of up to 4 columns, plus the moments
- * and local expansions of the levels: N = M = 1e7 with one column just fits) is refused with error 42 and
- * nothing is written to out.  The plan's own tables are built by the first f3m_plan_apply with the same
- * number of columns, which must therefore have run once before (otherwise error 41).  All calls on a GPU
- * share the one scratch array: calls that overlap on one GPU race, also from different plans or threads.
- * The call waits for the stream like the others, except while the stream is being captured. */
+ * 128 MiB of static device memory that every GPU running the library holds until the process ends.  The
+ * need does not grow with c beyond four columns: the sorted copies of b and of the result for one group of
+ * columns (4 (N + M) bytes for c = 1, 16 (N + M) bytes for c >= 2), the partial sums of that group's near
+ * field, and the moments and local expansions of one column's far field; every further group and column
+ * reuses that memory (N = M = 1e7 with one column just fits).  A product that needs more is refused with
+ * error 42 while its first column group is being queued, before anything is written to out.  The plan's own
+ * tables are built by the first f3m_plan_apply with the same number of columns, which must therefore have
+ * run once before (otherwise error 41).  All calls on a GPU share the one scratch array: calls that overlap
+ * on one GPU race, also from different plans or threads.  The call waits for the stream like the others,
+ * except while the stream is being captured.  A captured call holds the addresses of the plan's tables: its
+ * graph may be replayed only while the plan lives and no other entry point has rebuilt those tables in the
+ * meantime (f3m_plan_near_level on a list the products do not sum, a product with another number of columns,
+ * a change of the library's F3M_* environment switches); an error raised during capture leaves the capture
+ * to the caller (the library then waits for nothing). */
 int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream);
 
 /* Introspection for parity tests (no counterpart is exported by the reference; the data are its

@@ -86,6 +86,51 @@ def test_apply_without_allocation_refuses_what_does_not_fit(eng):
     plan.close()
 
 
+def test_apply_without_allocation_many_columns(eng):
+    """The scratch need must not grow with the number of columns: every column group (and every column's far
+    field) reuses the memory of the one before.  N = 1e6 with c = 6 and c = 16: the first group of four columns takes
+    ~100 MB of the 128 MiB (sorted copies 32 MB, sliced near-field partial sums 67 MB), so a second group that did
+    not reuse it could not fit.  Results are those of f3m_plan_apply bit for bit."""
+    import torch
+    print("case no-alloc: 3-D 1000000 points, 6 and 16 columns", flush=True)
+    rng = np.random.default_rng(34)
+    n = 1_000_000
+    X = dev(rng.random((n, 3), dtype=f32))
+    plan = eng.Plan(X, None, ls=1.0)
+    for c in (6, 16):
+        b = dev(rng.standard_normal((n, c)).astype(f32))
+        want = plan.apply(b)
+        out = torch.full((n, c), float("nan"), device="cuda")
+        plan.apply_noalloc(b, out)
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), c
+    plan.close()
+
+
+def test_apply_without_allocation_refusal_writes_nothing(eng):
+    """A product whose sorted copies fit (64 MB: the check before any work) but whose first column group does not
+    (1.5e6 targets in ~13000 pieces of 128, sliced three ways for four columns: ~80 MB of partial sums on top) is
+    refused while that group is being queued: error 42, and `out` is untouched."""
+    import torch
+    from f3m_amd.capi import F3MError
+    print("case no-alloc: refusal inside the first column group", flush=True)
+    rng = np.random.default_rng(35)
+    X = dev(rng.random((1_500_000, 3), dtype=f32))
+    Y = dev(rng.random((2_500_000, 3), dtype=f32))
+    b = dev(rng.standard_normal((2_500_000, 6)).astype(f32))
+    plan = eng.Plan(X, Y, ls=1.0)
+    want = plan.apply(b)
+    out = torch.full((1_500_000, 6), float("nan"), device="cuda")
+    with pytest.raises(F3MError) as e:
+        plan.apply_noalloc(b, out)
+    torch.cuda.synchronize()
+    assert e.value.code == 42 and "scratch" in str(e.value)
+    assert torch.isnan(out).all()
+    # the library is in order afterwards: the same plan still multiplies, with the same bits
+    assert torch.equal(plan.apply(b), want)
+    plan.close()
+
+
 def test_apply_without_allocation_under_graph_capture(eng):
     """One of the callers the entry point is for: a HIP graph.  The call is captured once and replayed with
     the program's own eager products and synchronisations between the replays; every replay must give the
