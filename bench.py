@@ -7,7 +7,10 @@ A step is one complete product out = K(X,Y) b through the C ABI (box division + 
 near field + far field), inputs resident in HBM, like one `FFM(X) @ b` of the reference
 (experiments/experiments.py:72-77).  Prints one JSON line: the headline configuration (N = 1e7 uniform in
 [0,1]^3, ls = 1, 64 nodes per box) with the roofline of its dominant kernel and the CPU baseline, and under
-"extra" the time, error and near-field roofline fraction of every other benchmark configuration.
+"extra" the time, error and near-field roofline fraction of every other benchmark configuration, of the larger node
+grids of the reference's own sweep (5^3 and 6^3 nodes, and that sweep's protocol with var_compression), the smallest
+grid that reaches the 1e-3 target for each configuration that misses it at 64 nodes, and the kernel-ridge-regression
+configuration (FALKON, N = 1e7, M = 1e5 centres) when the device has the memory for it.
 """
 import argparse
 import json
@@ -22,6 +25,30 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak (vector or matrix pipe)
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "near_g_kernel_n1e7_uniform3d_counters.md")
+STATS_PROFILE = os.path.join(ROOT, "profiles", "near_g_kernel_n1e7_uniform3d_kernel_stats.md")
+ORACLE_ERRORS = os.path.join(ROOT, "tests", "golden", "fullsize_oracle_errors.json")
+CRITICAL_STAGES = ("plan", "near", "perm")          # on the caller's stream; the far field runs beside the near field
+
+
+def oracle_error(name, nodes=None):
+    """rel-L2 error of the CPU oracle (the restatement of the reference algorithm) against the fp64 exact product at
+    N = 1e7 on 256 seeded rows, from the committed fixture (written by tests/golden/make_fullsize_oracle_errors.py in
+    the build container: this script does not run the oracle outside cpu_baseline)."""
+    try:
+        rec = json.load(open(ORACLE_ERRORS)).get(name if nodes is None else "%s:%d" % (name, nodes))
+        return rec["oracle_rel_l2_vs_fp64_exact"] if rec else None
+    except (OSError, ValueError):
+        return None
+
+
+def profiled_near_launch_us():
+    """average duration of the near-field launch in the committed rocprofv3 kernel trace of this command (the first
+    table: default two-stream mode), microseconds"""
+    try:
+        m = re.search(r"\|\s*f3m::near_g_kernel<3, 4, 1>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
+        return float(m.group(1)) if m else None
+    except OSError:
+        return None
 
 
 def near_traffic_bytes():
@@ -56,12 +83,22 @@ def cpu_baseline(X, Y, b, ls, budget_s=15.0):
             "host_cpu_count": os.cpu_count()}
 
 
-def run_config(name, n, steps, warmup, subsample, keep_inputs=False):
+def split_stages(stage, steps):
+    """stage times per step: those of the caller's stream add up to the step (with the waits between them); the
+    far-field stages run on the second stream beside the near field, so theirs are elapsed times that overlap it"""
+    ms = {k: v / steps * 1e3 for k, v in stage.items()}
+    return {"critical_path": {k: ms[k] for k in CRITICAL_STAGES if k in ms},
+            "overlapped_elapsed": {k: v for k, v in ms.items() if k not in CRITICAL_STAGES},
+            "note": "critical_path: stages on the caller's stream; overlapped_elapsed: far-field stages on the second stream, "
+                    "running beside the near field (elapsed, not additive)"}
+
+
+def run_config(name, n, steps, warmup, subsample, keep_inputs=False, nodes=None, one_stream_steps=0):
     """Times `steps` products of one configuration; returns its record (and the inputs if asked)."""
     import numpy as np
     import torch
     from f3m_amd import engine, workloads
-    X, Y, b, prm = workloads.make(name, n, seed=1)
+    X, Y, b, prm = workloads.make(name, n, seed=1, nodes=nodes)
     d = X.shape[1]
     engine.set_timing(True)
     for _ in range(warmup):
@@ -89,18 +126,88 @@ def run_config(name, n, steps, warmup, subsample, keep_inputs=False):
     achieved = F * work["near_pairs"] * steps / max(near_t, 1e-12) / 1e12
     rec = {"ms_per_step": dt / steps * 1e3, "ms_per_step_median": statistics.median(per_step) * 1e3,
            "points_per_s": n / (dt / steps), "tree_depth": depth, "boxes": nbx,
-           "stage_ms_per_step": {k: v / steps * 1e3 for k, v in stage.items()},
+           "stage_ms_per_step": split_stages(stage, steps),
            "near": {"achieved_tflops": achieved, "frac": achieved / PEAK_FP32_TFLOPS, "launches_per_step": near_n // max(steps, 1),
                     "ms_per_step": near_t / steps * 1e3, "flops_per_pair": F},
            "work": work}
+    if one_stream_steps:
+        # the same product with everything on the caller's stream (F3M_OVERLAP=0): every stage alone on the GPU
+        os.environ["F3M_OVERLAP"] = "0"
+        try:
+            engine.kmvm(X, Y, b, **prm)
+            alone, t1 = {}, time.perf_counter()
+            for _ in range(one_stream_steps):
+                engine.kmvm(X, Y, b, **prm)
+                for k, v in engine.get_timing().items():
+                    alone[k] = alone.get(k, 0.0) + v[0]
+            rec["one_stream"] = {"ms_per_step": (time.perf_counter() - t1) / one_stream_steps * 1e3,
+                                 "stage_ms_per_step": {k: v / one_stream_steps * 1e3 for k, v in alone.items()},
+                                 "note": "F3M_OVERLAP=0: one stream, each stage alone on the GPU (additive)"}
+        finally:
+            del os.environ["F3M_OVERLAP"]
     if subsample:
         rows = torch.from_numpy(np.random.default_rng(1).choice(n, min(subsample, n), replace=False)).cuda()
         exact = engine.exact_f64(X[rows].double(), (X if Y is None else Y).double(), b.double(), prm["ls"])
         rec["rel_l2_error"] = float((out[rows].double() - exact).norm() / exact.norm())
         rec["rel_l2_rows"] = int(rows.numel())
         rec["meets_1e-3"] = rec["rel_l2_error"] <= 1e-3
-        rec["algorithm_error_at_this_config"] = workloads.ALGORITHM_ERROR_N1E7.get(name) if n == 10_000_000 else None
+        rec["algorithm_error_at_this_config"] = oracle_error(name, nodes) if n == 10_000_000 else None
     return (rec, (X, Y, b, prm)) if keep_inputs else rec
+
+
+def extra_record(r, steps):
+    return {"ms_per_step": r["ms_per_step"], "ms_per_step_median": r["ms_per_step_median"],
+            "rel_l2_error": r.get("rel_l2_error"), "meets_1e-3": r.get("meets_1e-3"),
+            "algorithm_error_at_this_config": r.get("algorithm_error_at_this_config"),
+            "near_frac": r["near"]["frac"], "near_ms": r["near"]["ms_per_step"],
+            "near_launches": r["near"]["launches_per_step"], "tree_depth": r["tree_depth"],
+            "stage_ms_per_step": r["stage_ms_per_step"], "steps": steps}
+
+
+def falkon_record():
+    """The kernel-ridge-regression configuration at its stated size (N = 1e7, M = 1e5 centres, 20 iterations), if the
+    device has the ~85 GiB it needs: times of the fit and of the engine products inside one iteration."""
+    import torch
+    from f3m_amd import engine
+    from f3m_amd.conjugate_gradient import FalkonOptions, custom_Falkon, custom_GaussianKernel
+    engine.release_cache()
+    torch.cuda.empty_cache()
+    free = torch.cuda.mem_get_info()[0] / 2 ** 30
+    if free < 100:
+        return {"skipped": "%.0f GiB of device memory free, 100 needed" % free}
+    n, m = 10_000_000, 100_000
+    g = torch.Generator().manual_seed(1)
+    X = 2 * torch.rand(n, 3, generator=g) - 1
+    y = torch.sin(3 * X[:, 0]) * torch.cos(2 * X[:, 1]) + X[:, 2] ** 2 + 0.1 * torch.randn(n, generator=g)
+    X, Y = X.cuda(), y[:, None].cuda()
+    opt = FalkonOptions()
+    kernel = custom_GaussianKernel(0.5, opt=opt, var_compression=False, interpolation_nr=64)
+    model = custom_Falkon(kernel, 1e-6, m, maxiter=20, seed=1, options=opt)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    model.fit(X, Y)
+    torch.cuda.synchronize()
+    t_fit = time.perf_counter() - t0
+    pred = model.predict(X)
+    mse = float(((pred - Y) ** 2).mean())
+    r2 = 1 - mse / float(((Y - Y.mean()) ** 2).mean())
+    C, v = model.ny_points_, torch.randn(m, 1, generator=g).cuda()
+    kernel.dmmv(X, C, v, None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        kernel.dmmv(X, C, v, None)
+    torch.cuda.synchronize()
+    t_dmmv = (time.perf_counter() - t0) / 5
+    rec = {"workload": "FALKON kernel ridge regression, N=1e7 uniform [-1,1]^3, M=1e5 centres, ls=0.5, penalty 1e-6, 20 CG iterations",
+           "fit_s": t_fit, "preconditioner_s": model.fit_times_[0], "cg_s": model.conjugate_gradient_time,
+           "cg_iterations": model.cg_iterations_, "cg_s_per_iteration": model.conjugate_gradient_time / max(1, model.cg_iterations_),
+           "engine_products_per_iteration_s": t_dmmv, "engine_products_per_iteration": "K_nm v and K_nm^T u on one plan",
+           "mse": mse, "r2": r2, "peak_device_memory_gib": torch.cuda.max_memory_allocated() / 2 ** 30}
+    del model, kernel, X, Y, pred
+    engine.release_cache()
+    torch.cuda.empty_cache()
+    return rec
 
 
 def main():
@@ -109,11 +216,12 @@ def main():
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--n", type=int, default=10_000_000)
-    ap.add_argument("--config", default="uniform3_ls1", help="headline configuration (a name of f3m_amd.workloads.CONFIGS)")
+    ap.add_argument("--config", default="uniform3_ls1", help="headline configuration (a name of f3m_amd.workloads.ALL_CONFIGS)")
     ap.add_argument("--subsample", type=int, default=100_000)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-accuracy", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="skip the other benchmark configurations")
+    ap.add_argument("--no-falkon", action="store_true", help="skip the kernel-ridge-regression configuration")
     ap.add_argument("--extra-steps", type=int, default=3)
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run one plain 1 GiB device copy (a kernel of known HBM traffic, to scale rocprof counters)")
@@ -129,7 +237,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     N, name = args.n, args.config
-    cfg = workloads.CONFIGS[name]
+    cfg = workloads.ALL_CONFIGS[name]
     d = cfg["d"]
 
     if args.copy_probe:
@@ -140,10 +248,12 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    rec, (X, Y, b, prm) = run_config(name, N, args.steps, args.warmup, 0 if args.no_accuracy else args.subsample, keep_inputs=True)
+    rec, (X, Y, b, prm) = run_config(name, N, args.steps, args.warmup, 0 if args.no_accuracy else args.subsample, keep_inputs=True,
+                                     one_stream_steps=0 if args.no_extra else 3)
     M = N if Y is None else Y.shape[0]
     tiles_per_wave = 5 if (N // max(rec["boxes"], 1) + 31) // 32 == 5 else 4     # the library's choice (near_field)
-    traffic, traffic_range = near_traffic_bytes() if (N == 10_000_000 and name == "uniform3_ls1") else (None, None)
+    headline = N == 10_000_000 and name == "uniform3_ls1"
+    traffic, traffic_range = near_traffic_bytes() if headline else (None, None)
     near = rec["near"]
     roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
@@ -154,6 +264,14 @@ def main():
                         "%.3e kernel evaluations/step; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE "
                         "(profiles/near_g_kernel_n1e7_uniform3d_counters.md)"
                         % (near["flops_per_pair"], near["launches_per_step"], near["ms_per_step"], rec["work"]["near_pairs"])}
+    prof_us = profiled_near_launch_us() if headline else None
+    if prof_us:
+        # the same fraction from the committed kernel trace's average launch (warm-up launch included): the low end
+        roofline["profile_avg_launch_us"] = prof_us
+        roofline["frac_from_profile"] = near["flops_per_pair"] * rec["work"]["near_pairs"] / (prof_us * 1e-6) / 1e12 / PEAK_FP32_TFLOPS
+    if "one_stream" in rec and rec["one_stream"]["stage_ms_per_step"].get("near"):
+        roofline["frac_one_stream"] = (near["flops_per_pair"] * rec["work"]["near_pairs"] /
+                                       (rec["one_stream"]["stage_ms_per_step"]["near"] * 1e-3) / 1e12 / PEAK_FP32_TFLOPS)
     res = {
         "metric": "KMVM points/sec at N=1e7 3D Gaussian (1 GPU); rel-L2 error vs fp64 exact",
         "value": rec["points_per_s"], "unit": "points/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -167,26 +285,39 @@ def main():
         "stage_ms_per_step": rec["stage_ms_per_step"],
         "work": rec["work"],
     }
-    for k in ("rel_l2_error", "rel_l2_rows"):
+    if "one_stream" in rec:
+        res["one_stream"] = rec["one_stream"]
+    for k in ("rel_l2_error", "rel_l2_rows", "algorithm_error_at_this_config"):
         if k in rec:
             res[k] = rec[k]
+    res["algorithm_error_source"] = ("CPU oracle (restatement of the reference algorithm) at N=1e7 on 256 seeded rows vs fp64 exact, "
+                                     "tests/golden/fullsize_oracle_errors.json")
     if not args.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline(X, Y, b, cfg["ls"])
     del X, Y, b
     if not args.no_extra:
-        # every other benchmark configuration at the same N: fewer steps, error on 1e4 seeded rows
+        # every other configuration at the same N: fewer steps, error on 1e4 seeded rows
+        sub = 0 if args.no_accuracy else 10_000
         extra = {}
-        for other in workloads.CONFIGS:
+        for other in workloads.ALL_CONFIGS:
             if other == name:
                 continue
             torch.cuda.empty_cache()
-            r = run_config(other, N, args.extra_steps, 1, 0 if args.no_accuracy else 10_000)
-            extra[other] = {"ms_per_step": r["ms_per_step"], "ms_per_step_median": r["ms_per_step_median"],
-                            "rel_l2_error": r.get("rel_l2_error"), "meets_1e-3": r.get("meets_1e-3"),
-                            "algorithm_error_at_this_config": r.get("algorithm_error_at_this_config"),
-                            "near_frac": r["near"]["frac"], "near_ms": r["near"]["ms_per_step"],
-                            "near_launches": r["near"]["launches_per_step"], "tree_depth": r["tree_depth"],
-                            "stage_ms_per_step": r["stage_ms_per_step"], "steps": args.extra_steps}
+            extra[other] = extra_record(run_config(other, N, args.extra_steps, 1, sub), args.extra_steps)
+        # configurations that miss the 1e-3 target at 64 nodes per box: the smallest grid of the reference's sweep that meets it
+        for other in workloads.NODE_VARIANTS_OF:
+            sweep = {}
+            for nodes in workloads.NODE_SWEEP[1:]:
+                torch.cuda.empty_cache()
+                r = extra_record(run_config(other, N, args.extra_steps, 1, sub, nodes=nodes), args.extra_steps)
+                sweep[str(nodes)] = r
+                if r["meets_1e-3"]:
+                    extra[other]["smallest_grid_meeting_1e-3"] = {"nodes": nodes, "ms_per_step": r["ms_per_step"],
+                                                                   "rel_l2_error": r["rel_l2_error"]}
+                    break
+            extra[other]["node_sweep"] = sweep
+        if not args.no_falkon and N == 10_000_000:
+            extra["falkon_krr"] = falkon_record()
         res["extra"] = extra
     print(json.dumps(res))
 

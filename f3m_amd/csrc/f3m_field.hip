@@ -1241,9 +1241,10 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
                                                          const float *__restrict__ nw, float factor, float *__restrict__ partial)
 {
     constexpr int NR = ipow(N, R), Q = ipow(N, D - R), G = 64 / Q, PG = (64 + G - 1) / G, QS = Q | 1, P = Q * NR;   // QS: odd row stride
-    static_assert(Q <= 64 && NR <= QS, "one wavefront holds the nodes of the last D-R dimensions");
+    static_assert(Q <= 64, "one wavefront holds the nodes of the last D-R dimensions");
     __shared__ float sh[64 * NR];
     __shared__ float sw[64 * QS];
+    float *const red = NR <= QS ? sw : sh;          // 64 * NR floats for the closing sum over the groups
     const int lane = threadIdx.x;
     if ((int)blockIdx.x >= tileoff[nb]) return;     // launched with an upper bound of the chunk count
     const int box = find_box(tileoff, nb, blockIdx.x);
@@ -1305,13 +1306,13 @@ __global__ void __launch_bounds__(64) p2m_tensor_kernel(const float *__restrict_
     // add the groups: lanes q, Q + q, 2Q + q, ... hold partial sums of the same nodes
     __syncthreads();
 #pragma unroll
-    for (int a = 0; a < NR; a++) sw[lane * NR + a] = g < G ? acc[a] : 0.f;
+    for (int a = 0; a < NR; a++) red[lane * NR + a] = g < G ? acc[a] : 0.f;
     __syncthreads();
     if (lane < Q) {
 #pragma unroll
         for (int a = 0; a < NR; a++) {
             float t = 0.f;
-            for (int gg = 0; gg < G; gg++) t += sw[(gg * Q + lane) * NR + a];
+            for (int gg = 0; gg < G; gg++) t += red[(gg * Q + lane) * NR + a];
             partial[(long long)blockIdx.x * P + a + NR * lane] = t;
         }
     }
@@ -1640,8 +1641,10 @@ __global__ void sib_class_count_kernel(const int *__restrict__ childstart, const
     cls[p] = c;
     atomicAdd(&hist[c], 1);
 }
+// (grids of 5 or 6 nodes per dimension, 3-D only: a workgroup is one wavefront, and a lane's 3 N^2 partial sums and
+// its moments in flight need more registers than a 1024-thread bound would leave)
 template <int D, int N, int H>
-__global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
+__global__ void __launch_bounds__((D == 3 && N >= 5) ? 64 : 1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
                                                         int R2, int GS, int nsub, int npass, const int *__restrict__ order,
                                                         const int *__restrict__ childstart,
                                                         const int *__restrict__ cell, const int *__restrict__ pairs,
@@ -1650,9 +1653,13 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
 {
     // H = 2: the n0 x n1 nodes of a lane are shared by two lanes, n1/2 values of a1 each (a workgroup of
     // 2^D siblings x R2 lanes would otherwise fill half a wavefront in 3-D); NN = nodes of a lane
+    // W: row length of the padded tables of the first two factors (rows are read as vectors of four)
     constexpr int NCODE = sib_codes(D), NEXT = sib_ext_codes(D), NN = N * N / H, NQ1 = N / H, NB = N <= 3 ? 4 : (D >= 4 ? 1 : 2);
+    constexpr int W = N <= 4 ? 4 : 8;
     static_assert(H == 1 || (H == 2 && N % 2 == 0), "the nodes of dimension 1 are split in halves");
     F3M_DYN_SHARED(float, smem);
+    // (every lambda below is forced inline: a call would take the partial sums, which are indexed by constants
+    // everywhere, out of the registers)
     const int tid = threadIdx.x, BD = blockDim.x, lane = tid & 63;
     // The regular table is filled and walked in npass parts (slabs of the last dimension, which is the
     // outermost of the walk), so that it takes NCODE / npass cells of LDS (the host asks for more than
@@ -1666,9 +1673,9 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     int *xkey = xord + NEXT;                                        // NEXT
     float *xbuf = smem + 2 * chunk + 4 * NEXT;                      // NN * BD: exchange buffer
     float *tabg = xbuf + NN * BD;                                   // ntab: E_j[o][a][q], row length sm.NT
-    float *tab01 = tabg + ((ntab + 3) & ~3);                        // 2 * 13 * N rows of 4: E_0, E_1 padded
-    float *zrow = tab01 + 2 * kM2LOffsets * N * 4;                  // N rows of zeros
-    int *sib = reinterpret_cast<int *>(zrow + N * 4);               // GS: compact id of each sibling or -1
+    float *tab01 = tabg + ((ntab + 3) & ~3);                        // 2 * 13 * N rows of W: E_0, E_1 padded
+    float *zrow = tab01 + 2 * kM2LOffsets * N * W;                  // N rows of zeros
+    int *sib = reinterpret_cast<int *>(zrow + N * W);               // GS: compact id of each sibling or -1
     // order (nullable): the parents sorted by the length of their far rows, longest first, so that the
     // workgroups that run longest start first
     const int px = order ? order[blockIdx.x / nsub] : blockIdx.x / nsub, sg = blockIdx.x % nsub;
@@ -1683,11 +1690,11 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
         xkey[e] = key;
     }
     for (int e = tid; e < ntab; e += BD) tabg[e] = tables[e];
-    for (int e = tid; e < 2 * kM2LOffsets * N * 4; e += BD) {
-        const int q = e & 3, a = (e >> 2) % N, o = (e / (4 * N)) % kM2LOffsets, j = e / (4 * N * kM2LOffsets);
+    for (int e = tid; e < 2 * kM2LOffsets * N * W; e += BD) {
+        const int q = e % W, a = (e / W) % N, o = (e / (W * N)) % kM2LOffsets, j = e / (W * N * kM2LOffsets);
         tab01[e] = q < N ? tables[((j * kM2LOffsets + o) * sm.NT + a) * sm.NT + q] : 0.f;
     }
-    for (int e = tid; e < N * 4; e += BD) zrow[e] = 0.f;
+    for (int e = tid; e < N * W; e += BD) zrow[e] = 0.f;
     if (tid < GS) sib[tid] = -1;
     __syncthreads();
     for (int e = tid; e < NEXT; e += BD) {                 // walking order of the extension cells
@@ -1709,7 +1716,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     for (int j = 0; j < D; j++) pc[j] = 2 * (cell[(long long)c0 * D + j] >> 1) - 2;
     __syncthreads();
     // fills part `pass` of the regular table (and, with part 0, the extension table) from the far rows
-    auto fill_tables = [&](int pass) {
+    auto fill_tables = [&](int pass) __attribute__((always_inline)) {
         for (int e = tid; e < chunk; e += BD) { tby[e] = 0; tmask[e] = 0u; }
         __syncthreads();
         for (int s2 = 0; s2 < GS; s2++) {
@@ -1752,6 +1759,26 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     }
     const float *mine = mom + (long long)NN * (live ? r2h : 0);
 
+    // the NN moments of a lane, four floats per load (a copy of the whole vector as one object keeps large ones out
+    // of registers)
+    auto load_moments = [](const float *src, fvec<NN> &v) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i + 4 <= NN; i += 4) {
+            const fvec<4> t = *reinterpret_cast<const fvec<4> *>(src + i);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v.v[i + e] = t.v[e];
+        }
+#pragma unroll
+        for (int i = NN & ~3; i < NN; i++) v.v[i] = src[i];
+    };
+    // one padded table row
+    auto load_row = [](const float *row, float (&ev)[W]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < W; u += 4) {
+            const float4 e = *reinterpret_cast<const float4 *>(row + u);
+            ev[u] = e.x; ev[u + 1] = e.y; ev[u + 2] = e.z; ev[u + 3] = e.w;
+        }
+    };
     float acc[D][NN];
 #pragma unroll
     for (int j = 0; j < D; j++)
@@ -1762,20 +1789,20 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     // box is paid by each of them on the compute unit's one scalar unit.
     int curpk = 0;
     bool have = false;
-    auto digit2 = [](int pk, int j) { return (pk >> (4 * j)) & 15; };      // digit j + 2
+    auto digit2 = [](int pk, int j) __attribute__((always_inline)) { return (pk >> (4 * j)) & 15; };      // digit j + 2
 
     // applies factor l+1 to acc[l], adds the result to acc[l+1] and clears acc[l]
-    auto flush = [&](auto level) {
+    auto flush = [&](auto level) __attribute__((always_inline)) {
         constexpr int l = decltype(level)::value, j = l + 1;
         if constexpr (j == 1) {
             int oi = digit2(curpk, 1) - cbit[1];
             oi = min(max(oi, 0), kM2LOffsets - 1);
-            const float *T1 = tab01 + ((kM2LOffsets + oi) * N) * 4;
+            const float *T1 = tab01 + ((kM2LOffsets + oi) * N) * W;
             if constexpr (H == 1) {
 #pragma unroll
                 for (int a1 = 0; a1 < N; a1++) {
-                    const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
-                    const float ev[4] = {e.x, e.y, e.z, e.w};
+                    float ev[W];
+                    load_row(T1 + a1 * W, ev);
 #pragma unroll
                     for (int a0 = 0; a0 < N; a0++) {
                         float t = acc[1][a0 + N * a1];
@@ -1790,8 +1817,8 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
                 float part[N * N];
 #pragma unroll
                 for (int a1 = 0; a1 < N; a1++) {
-                    const float4 e = *reinterpret_cast<const float4 *>(T1 + a1 * 4);
-                    const float ev[4] = {e.x, e.y, e.z, e.w};
+                    float ev[W];
+                    load_row(T1 + a1 * W, ev);
 #pragma unroll
                     for (int a0 = 0; a0 < N; a0++) {
                         float t = 0.f;
@@ -1829,14 +1856,14 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
 #pragma unroll
         for (int i = 0; i < NN; i++) acc[l][i] = 0.f;
     };
-    auto flush_upto = [&](int jt) {       // levels 0 .. jt-1, jt uniform over the workgroup
+    auto flush_upto = [&](int jt) __attribute__((always_inline)) {       // levels 0 .. jt-1, jt uniform over the workgroup
         if (jt > 0) flush(std::integral_constant<int, 0>());
         if constexpr (D > 2) { if (jt > 1) flush(std::integral_constant<int, 1>()); }
         if constexpr (D > 3) { if (jt > 2) flush(std::integral_constant<int, 2>()); }
         if constexpr (D > 4) { if (jt > 3) flush(std::integral_constant<int, 3>()); }
     };
     // one far box: pk = its packed digits (uniform), v = its moments at this lane's nodes
-    auto far_box = [&](int pk, unsigned smask, const fvec<NN> &v) {
+    auto far_box = [&](int pk, unsigned smask, const fvec<NN> &v) __attribute__((always_inline)) {
         if (have) {
             const int diff = (pk ^ curpk) >> 4;             // digits 1.. that change
             flush_upto(diff ? (31 - __builtin_clz(diff)) / 4 + 1 : 0);   // up to the highest of them
@@ -1846,11 +1873,11 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
         const bool part = live && ((smask >> sl) & 1u);
         int oi = digit2(pk, 0) - cbit[0];
         oi = min(max(oi, 0), kM2LOffsets - 1);
-        const float *T0 = part ? tab01 + (oi * N) * 4 : zrow;
+        const float *T0 = part ? tab01 + (oi * N) * W : zrow;
 #pragma unroll
         for (int a0 = 0; a0 < N; a0++) {
-            const float4 e = *reinterpret_cast<const float4 *>(T0 + a0 * 4);
-            const float ev[4] = {e.x, e.y, e.z, e.w};
+            float ev[W];
+            load_row(T0 + a0 * W, ev);
 #pragma unroll
             for (int q1 = 0; q1 < NQ1; q1++) {
                 float t = acc[0][a0 + N * q1];
@@ -1861,7 +1888,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
         }
     };
     // walks 64 table cells: ml, byl = this lane's cell; cellid = its id (regular code or extension entry)
-    auto walk64 = [&](unsigned ml, int byl, int cellid, auto ext) {
+    auto walk64 = [&](unsigned ml, int byl, int cellid, auto ext) __attribute__((always_inline)) {
         int pkl = 0;                                       // packed digits of this lane's cell
         {
             int dg[D];
@@ -1884,7 +1911,7 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
                 ls[u] = 0;
                 if (bal) { ls[u] = __ffsll(bal) - 1; bal &= bal - 1; cnt++; }
                 const int by = wave_readlane(byl, ls[u]);
-                v[u] = *reinterpret_cast<const fvec<NN> *>(mine + (long long)by * P);
+                load_moments(mine + (long long)by * P, v[u]);
             }
 #pragma unroll
             for (int u = 0; u < NB; u++) {
@@ -1912,10 +1939,16 @@ __global__ void __launch_bounds__(1024) m2l_sib_kernel(const float *__restrict__
     }
     if (have) flush_upto(D - 1);
     if (live) {
-        fvec<NN> r;
+        float *dst = loc + (long long)mybox * P + (long long)NN * r2h;
 #pragma unroll
-        for (int i = 0; i < NN; i++) r.v[i] = acc[D - 1][i];
-        *reinterpret_cast<fvec<NN> *>(loc + (long long)mybox * P + (long long)NN * r2h) = r;
+        for (int i = 0; i + 4 <= NN; i += 4) {
+            fvec<4> r;
+#pragma unroll
+            for (int e = 0; e < 4; e++) r.v[e] = acc[D - 1][i + e];
+            *reinterpret_cast<fvec<4> *>(dst + i) = r;
+        }
+#pragma unroll
+        for (int i = NN & ~3; i < NN; i++) dst[i] = acc[D - 1][i];
     }
 }
 
@@ -2039,6 +2072,14 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
         F3M_LAUNCH((p2m_tensor_kernel<3, 3, 1>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
                    ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
         check_launch("p2m_tensor");
+    } else if (nty > 0 && d == 3 && ns.n[0] == 5 && ns.n[1] == 5 && ns.n[2] == 5) {
+        F3M_LAUNCH((p2m_tensor_kernel<3, 5, 2>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
+                   ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
+        check_launch("p2m_tensor");
+    } else if (nty > 0 && d == 3 && ns.n[0] == 6 && ns.n[1] == 6 && ns.n[2] == 6) {
+        F3M_LAUNCH((p2m_tensor_kernel<3, 6, 2>), nty, 64, 0, s, ty.pts.get(), ty.n, bs, ly.off.get(), ly.ctr.get(), tiley.get(),
+                   ly.nb, ns.dt.get(), ns.dw.get(), factor, partial.get());
+        check_launch("p2m_tensor");
     } else if (nty > 0) {
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -2098,9 +2139,9 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         // parents: 0.30 against 0.55 ms at depth 5 of N=1e7; with fewer parents the per-box kernel has
         // more workgroups to offer)
         const bool enough_parents = sib_forced || !q64 || (lx.depth >= 1 && tx.lev[lx.depth - 1].nb >= 256);
-        if (m2l_mode == 0 && enough_parents && &tx == &ty && d >= 3 && d <= 5 && ns.n[0] == ns.n[1] && ns.n[0] >= 2 && ns.n[0] <= 4 &&
-            far.outliers == 0 && lx.depth >= 1) {
-            const int N = ns.n[0];
+        const bool sib_grid = ns.n[0] == ns.n[1] && ns.n[0] >= 2 && (ns.n[0] <= 4 || (d == 3 && ns.n[0] <= 6 && ns.n[2] == ns.n[0]));
+        if (m2l_mode == 0 && enough_parents && &tx == &ty && d >= 3 && d <= 5 && sib_grid && far.outliers == 0 && lx.depth >= 1) {
+            const int N = ns.n[0], W = N <= 4 ? 4 : 8;
             sibR2 = P / (N * N);
             if (sibR2 <= 1024) {
                 sibGS = 1 << d;
@@ -2123,13 +2164,16 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                     if (forced > 0 && np != forced && np != 6) continue;
                     sibPass = np;
                     shsib = sizeof(float) * (2 * (size_t)(sib_codes(d) / np) + 4 * (size_t)sib_ext_codes(d) + (size_t)(N * N / sibH) * bd +
-                                             (size_t)((ntab + 3) & ~3) + 2 * (size_t)kM2LOffsets * N * 4 + (size_t)N * 4) +
+                                             (size_t)((ntab + 3) & ~3) + 2 * (size_t)kM2LOffsets * N * W + (size_t)N * W) +
                             sizeof(int) * (size_t)sibGS;
                     if ((shsib <= 150 * 1024 && forced <= 0) || np == forced) break;
                 }
                 if (shsib > 150 * 1024) sibGS = 0;
             }
         }
+        if (getenv("F3M_DEBUG"))
+            fprintf(stderr, "m2l depth %d: %s (nodes %d, siblings per workgroup %d, lanes per sibling %d, table parts %d)\n", lx.depth,
+                    sibGS > 0 ? "sibling groups" : (q64 ? "4x4x4 per box" : "separable per box"), P, sibGS, sibR2, sibPass);
         if (sibGS > 0) {
             const TreeLevel &par = tx.lev[lx.depth - 1];
             const int nsub = (1 << d) / sibGS;
@@ -2169,7 +2213,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                    sibGS, nsub, sibPass, sibOrd, par.childstart.get(), lx.cell.get(), far.pairs.get(),                 \
                    far.rowptr.get(), mom, loc);                                                                        \
     }
-            F3M_SIB(3, 2, 2) F3M_SIB(3, 3, 1) F3M_SIB(3, 4, 2) F3M_SIB(3, 2, 1) F3M_SIB(3, 4, 1)
+            F3M_SIB(3, 2, 2) F3M_SIB(3, 3, 1) F3M_SIB(3, 4, 2) F3M_SIB(3, 2, 1) F3M_SIB(3, 4, 1) F3M_SIB(3, 5, 1) F3M_SIB(3, 6, 1)
             F3M_SIB(4, 2, 1) F3M_SIB(4, 3, 1) F3M_SIB(4, 4, 1)
             F3M_SIB(5, 2, 1) F3M_SIB(5, 3, 1) F3M_SIB(5, 4, 1)
 #undef F3M_SIB
@@ -2356,6 +2400,22 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<3, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_tensor");
+        return;
+    }
+    if (flag == nullptr && d == 3 && ns.n[0] == 5 && ns.n[1] == 5 && ns.n[2] == 5) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH((l2p_tensor_kernel<3, 5>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+        timer_end(s);
+        check_launch("l2p_tensor");
+        return;
+    }
+    if (flag == nullptr && d == 3 && ns.n[0] == 6 && ns.n[1] == 6 && ns.n[2] == 6) {
+        timer_begin(kL2P, s);
+        F3M_LAUNCH((l2p_tensor_kernel<3, 6>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
                    lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
         timer_end(s);
         check_launch("l2p_tensor");
@@ -2555,6 +2615,73 @@ __global__ void __launch_bounds__(kShiftQWaves * 64) shift_q64_kernel(const floa
     if (!DOWN) dst[(long long)b * 64 + lane] = acc;
 }
 
+// The same transfer for any grid of N nodes per dimension on both levels, one wavefront per parent box (a workgroup
+// of one wavefront finds room beside the near field's wavefronts; the general kernel's workgroup of one lane per node
+// does not).  The expansion of a child passes through two LDS buffers, one 1-D factor at a time; lane l owns the
+// elements l, l + 64, ... of every stage.
+template <bool DOWN, int D, int N>
+__global__ void __launch_bounds__(64) shift_tensor_kernel(const float *__restrict__ tables, int nbp,
+                                                           const int *__restrict__ childstart, const int *__restrict__ cellc,
+                                                           const float *__restrict__ src, float *__restrict__ dst)
+{
+    constexpr int P = ipow(N, D), K = (P + 63) / 64, NTAB = D * 2 * N * N;
+    __shared__ float tab[NTAB];             // T_j[s][m][a], m = parent node, a = child node
+    __shared__ float buf[2][P];
+    const int lane = threadIdx.x, b = blockIdx.x;
+    if (b >= nbp) return;
+    for (int e = lane; e < NTAB; e += 64) tab[e] = tables[e];
+    float acc[K], par[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        const int e = lane + 64 * k;
+        acc[k] = 0.f;
+        par[k] = (DOWN && e < P) ? src[(long long)b * P + e] : 0.f;
+    }
+    for (int c = childstart[b]; c < childstart[b + 1]; c++) {
+        __syncthreads();                    // the previous child's last stage has been read
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int e = lane + 64 * k;
+            if (e < P) buf[0][e] = DOWN ? par[k] : src[(long long)c * P + e];
+        }
+        __syncthreads();
+        int stride = 1;
+#pragma unroll
+        for (int j = 0; j < D; j++) {
+            const int sg = cellc[(long long)c * D + j] & 1;
+            const float *T = tab + (j * 2 + sg) * N * N;
+            const float *in = buf[j & 1];
+            float *out = buf[(j & 1) ^ 1];
+#pragma unroll
+            for (int k = 0; k < K; k++) {
+                const int e = lane + 64 * k;
+                if (e < P) {
+                    const int q = (e / stride) % N;
+                    const float *sp = in + (e - q * stride);
+                    float sum = 0.f;
+#pragma unroll
+                    for (int r = 0; r < N; r++) sum = fmaf(DOWN ? T[r * N + q] : T[q * N + r], sp[r * stride], sum);
+                    if (j == D - 1) {
+                        if (DOWN) dst[(long long)c * P + e] += sum;
+                        else acc[k] += sum;
+                    } else {
+                        out[e] = sum;
+                    }
+                }
+            }
+            stride *= N;
+            if (j < D - 1) __syncthreads();
+        }
+    }
+    if (!DOWN) {
+#pragma unroll
+        for (int k = 0; k < K; k++) {
+            const int e = lane + 64 * k;
+            if (e < P) dst[(long long)b * P + e] = acc[k];
+        }
+    }
+}
+
 bool nodes_nest(const NodeSet &coarse, const NodeSet &fine)
 {
     if (coarse.d != fine.d) return false;
@@ -2598,7 +2725,27 @@ void shift_level(bool down, const TreeLevel &parent, const TreeLevel &child, con
     timer_begin(down ? kL2P : kP2M, s);
     const bool q64 = d == 3 && sm.Pp == 64 && sm.Pc == 64 && sm.NTp == 4 && sm.NTc == 4 && nsp.n[0] == 4 && nsp.n[1] == 4 &&
                      nsc.n[0] == 4 && nsc.n[1] == 4;
-    if (q64 && down)
+    // the same N nodes along every dimension on both levels: one wavefront per parent
+    int same = nsp.n[0];
+    for (int j = 0; j < d; j++)
+        if (nsp.n[j] != same || nsc.n[j] != same) same = 0;
+    bool done = false;
+#define F3M_SHIFT_T(DD, NNODE)                                                                                         \
+    if (!done && !q64 && d == DD && same == NNODE) {                                                                   \
+        if (down)                                                                                                      \
+            F3M_LAUNCH((shift_tensor_kernel<true, DD, NNODE>), parent.nb, 64, 0, s, tab, parent.nb,                    \
+                       parent.childstart.get(), child.cell.get(), src, dst);                                           \
+        else                                                                                                           \
+            F3M_LAUNCH((shift_tensor_kernel<false, DD, NNODE>), parent.nb, 64, 0, s, tab, parent.nb,                   \
+                       parent.childstart.get(), child.cell.get(), src, dst);                                           \
+        done = true;                                                                                                   \
+    }
+    F3M_SHIFT_T(3, 3) F3M_SHIFT_T(3, 5) F3M_SHIFT_T(3, 6) F3M_SHIFT_T(4, 3) F3M_SHIFT_T(5, 3)
+#undef F3M_SHIFT_T
+    if (getenv("F3M_DEBUG"))
+        fprintf(stderr, "shift %s depth %d: %s\n", down ? "down" : "up", parent.depth, done ? "one wavefront per parent" : (q64 ? "4x4x4" : "general"));
+    if (done) {
+    } else if (q64 && down)
         F3M_LAUNCH((shift_q64_kernel<true>), cdiv(parent.nb, kShiftQWaves), kShiftQWaves * 64, 0, s, tab, parent.nb,
                    parent.childstart.get(), child.cell.get(), src, dst);
     else if (q64)

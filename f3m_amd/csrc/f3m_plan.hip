@@ -182,7 +182,6 @@ static ClassifyParams classify_params(const f3m_plan &P, float edge)
 // A second stream per device, on which the far field of a product runs beside the near field (which is bound
 // by vector-ALU issue and leaves the memory system and the latency-bound far-field kernels room), with the two
 // events that fork it from and join it to the caller's stream.  Default priority, kept for the life of the process.
-#ifndef F3M_CPU_EMU
 struct SideStream {
     hipStream_t stream = nullptr;
     hipEvent_t fork = nullptr, join = nullptr;
@@ -202,7 +201,6 @@ static SideStream &side_stream()
     }
     return ss;
 }
-#endif
 
 // b_early (nullable, with c_early columns): the weights of the product that will follow at once (f3m_kmvm_f32);
 // their first column group is put into sorted order while the lists are built.  With b_early the function returns
@@ -321,7 +319,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // While work is queued on both streams, blocks that host code gives back are parked (a kernel of the other stream
     // may still use them, and the pool would hand them to the next request); they return to the pool at the end.
     ParkingLot lot;
-#ifndef F3M_CPU_EMU
     const bool two_streams = g_arena == nullptr && !(getenv("F3M_OVERLAP") && atoi(getenv("F3M_OVERLAP")) == 0);
     auto start_early_moves = [&]() {
         SideStream &ss = side_stream();
@@ -353,24 +350,18 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             P->early_bs.free();
         }
     };
-#else
-    auto settle_early = [&]() {};
-#endif
     if (need_tree && wants_division()) {
         settle_early();
         start_division();
-#ifndef F3M_CPU_EMU
         // with the first division's counts, the fullest cell at the depth that the sorted key bits resolve
         // (words [14], [15] of the record)
         if (two_streams) {
             max_run_launch(P->tx, dres.get() + 14, s);
             if (!sym) max_run_launch(P->ty_, dres.get() + 15, s);
         }
-#endif
         fetch_level_begin(nullptr, true);
         fetch_level_wait();
         finish_division();
-#ifndef F3M_CPU_EMU
         if (two_streams) {
             // A tree whose fullest cell at that depth still calls for division will need more key bits sorted: now,
             // rather than in the middle of the level loop, so that the order of the points is final from here on
@@ -379,7 +370,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             if (!sym && (float)hres[15] > prm->min_points) sort_more_bits(P->ty_, s);
             start_early_moves();
         }
-#endif
         for (;;) {
             const int k = (int)P->tx.lev.size() - 1;
             const float e = P->tx.lev[k].edge;
@@ -392,7 +382,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                          drow.get() + 8 * (P->levels.size() - 1), s);
             const bool ahead = wants_division();
             if (ahead) { settle_early(); start_division(); }
-#ifndef F3M_CPU_EMU
             // No further division: this is the deepest level, whose near lists will be summed.  Its source operands
             // are prepared on the second stream (behind the moves of the points) while its lists are built here.
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)
@@ -406,7 +395,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
                 }
             }
-#endif
             // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
             // host has them, wherever an upper bound of the sizes is a modest allocation: it then runs during the wait.
             fetch_level_begin(&pend, ahead);
@@ -430,12 +418,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             break;
         }
     }
-#ifndef F3M_CPU_EMU
     if (early) {
         F3M_HIP(hipEventRecord(side_stream().join, side_stream().stream));
         F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));       // the work of the second stream is part of the plan
     }
-#endif
     if (need_tree && !early) {
         gather_tree_points(P->tx, X, s);
         if (!sym) gather_tree_points(P->ty_, Y, s);
@@ -602,14 +588,12 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     // scattered (F3M_OVERLAP=0: one stream).  Not for a call whose temporaries come from an arena (it would need
     // one more array of N floats per column) and not for the per-level cross-check.
     bool overlap = false;
-#ifndef F3M_CPU_EMU
     {
         bool any_far = false;
         for (int k = 1; k <= depth; k++) any_far = any_far || (transposed ? P->levels[k - 1].farT.n : P->levels[k - 1].far.n) > 0;
         const char *oe = getenv("F3M_OVERLAP");
         overlap = any_far && !per_level && g_arena == nullptr && !(oe && atoi(oe) == 0);
     }
-#endif
     DBuf<float> outs_far;
     if (overlap) {
         outs_far.reset((size_t)ostride * width);
@@ -664,7 +648,6 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         {
             ParkingLot lot;
             lot.start();
-#ifndef F3M_CPU_EMU
             if (overlap) {
                 // The near field's own tables first (kept with the plan from then on), so that its long launches
                 // follow without delay; the streams part after that: the far field then runs beside those launches.
@@ -676,7 +659,6 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 F3M_HIP(hipEventRecord(side_stream().fork, s));
                 F3M_HIP(hipStreamWaitEvent(side_stream().stream, side_stream().fork, 0));
             }
-#endif
             // the near field first: it is the long pole, and the host needs a while to queue the far field's many
             // small kernels
             for (int k = 1; k <= depth; k++) {
@@ -699,21 +681,17 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             if (!per_level) {
                 hipStream_t fs = s;
                 float *fo = outs.get();
-#ifndef F3M_CPU_EMU
                 if (overlap) { fs = side_stream().stream; fo = outs_far.get(); }
-#endif
                 const size_t mark = arena_mark();
                 for (int q = 0; q < ncol; q++) {
                     arena_rewind(mark);
                     far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap);
                 }
             }
-#ifndef F3M_CPU_EMU
             if (overlap) {
                 F3M_HIP(hipEventRecord(side_stream().join, side_stream().stream));
                 F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
             }
-#endif
             Scope sc(kPerm, s);
             scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
         }

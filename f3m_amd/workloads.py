@@ -36,16 +36,9 @@ for _n in NODE_SWEEP:
                                                       var_compression=True, eff_var_limit=0.9, small_field_points=_n)
 ALL_CONFIGS = dict(CONFIGS, **MORE_CONFIGS)
 
-# rel-L2 error of the product against the fp64 exact product that the F3M algorithm itself has at these
-# node counts and lengthscales at N = 1e7 (measured with this engine, which matches the CPU restatement of
-# the reference algorithm to 1e-5 on clouds of the same kind at sizes that restatement can run); the
-# full-size tests allow 1.5x these.  Where the figure is above 1e-3 the algorithm at 64 nodes per box does
-# not reach the 1e-3 target at that lengthscale, whatever computes it.
-ALGORITHM_ERROR_N1E7 = {
-    "uniform3_ls1": 3.4e-6, "uniform3_ls0.1": 1.4e-3, "uniform3_ls10": 6e-7,
-    "normal3_ls1": 1.1e-3, "normal3_ls0.1": 1.4e-3, "normal3_ls10": 1.0e-6,
-    "clustered3_xy_ls0.5": 1.5e-3, "uniform4_81nodes": 1.0e-4, "uniform5_243nodes": 7.7e-4,
-}
+# configurations whose error at 64 nodes per box is above the 1e-3 target (the algorithm's own error there): the
+# benchmark also runs them at the larger grids of NODE_SWEEP and reports the smallest that meets the target
+NODE_VARIANTS_OF = ("uniform3_ls0.1", "normal3_ls1", "normal3_ls0.1", "clustered3_xy_ls0.5")
 
 
 def make(name, n, seed=1, columns=1, device="cuda", nodes=None):

@@ -15,6 +15,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <functional>
 #include <vector>
 
@@ -36,16 +37,94 @@ typedef void *hipStream_t;
 enum { hipSuccess = 0, hipErrorInvalidValue = 1, hipErrorOutOfMemory = 2 };
 enum hipMemcpyKind { hipMemcpyHostToDevice, hipMemcpyDeviceToHost, hipMemcpyDeviceToDevice, hipMemcpyDefault };
 
+// Streams.  The caller's stream (any handle the program did not create, normally null) runs its work at once, in
+// program order.  A stream that the program CREATES is lazy: its work is queued and runs only when something waits
+// for it -- an event of that stream that another stream or the host waits for, a synchronisation -- which is the
+// latest moment the HIP model allows.  Host code that gives a buffer back, or reuses it on the caller's stream, while
+// work of a created stream still needs it therefore computes with the wrong data here, and the tests see it.
+// F3M_EMU_STREAMS=eager makes created streams run at once as well (the earliest schedule).
+namespace emu {
+struct Stream {
+    std::deque<std::function<void()>> q;
+    size_t queued = 0, done = 0;
+    void run_until(size_t target)
+    {
+        while (done < target && !q.empty()) {
+            std::function<void()> f = std::move(q.front());
+            q.pop_front();
+            done++;
+            f();
+        }
+    }
+};
+struct Event {
+    Stream *stream = nullptr;     // lazy stream the event was recorded on (null: recorded on an eager stream, complete)
+    size_t pos = 0;               // work of that stream queued before the event
+};
+inline std::vector<Stream *> &streams() { static std::vector<Stream *> v; return v; }
+inline Stream *lazy(void *s)
+{
+    for (Stream *t : streams()) if (t == s) return t;
+    return nullptr;
+}
+inline bool eager_streams()
+{
+    const char *e = getenv("F3M_EMU_STREAMS");
+    return e && !strcmp(e, "eager");
+}
+// runs f now, or queues it if `stream` is a lazy stream
+inline void submit(void *stream, std::function<void()> f)
+{
+    Stream *st = lazy(stream);
+    if (st && !eager_streams()) { st->q.push_back(std::move(f)); st->queued++; }
+    else f();
+}
+inline void drain_all() { for (Stream *t : streams()) t->run_until(t->queued); }
+}  // namespace emu
+typedef emu::Event *hipEvent_t;
+enum { hipStreamNonBlocking = 1, hipEventDisableTiming = 2 };
+
 inline hipError_t hipMalloc(void **p, size_t n) { *p = malloc(n ? n : 1); return *p ? hipSuccess : hipErrorOutOfMemory; }
 inline hipError_t hipFree(void *p) { free(p); return hipSuccess; }
-inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { memcpy(d, s, n); return hipSuccess; }
-inline hipError_t hipMemcpyAsync(void *d, const void *s, size_t n, hipMemcpyKind, hipStream_t) { memcpy(d, s, n); return hipSuccess; }
-inline hipError_t hipMemsetAsync(void *d, int v, size_t n, hipStream_t) { memset(d, v, n); return hipSuccess; }
-inline hipError_t hipStreamSynchronize(hipStream_t) { return hipSuccess; }
-inline hipError_t hipDeviceSynchronize() { return hipSuccess; }
+inline hipError_t hipMemcpy(void *d, const void *s, size_t n, hipMemcpyKind) { emu::drain_all(); memcpy(d, s, n); return hipSuccess; }
+inline hipError_t hipMemcpyAsync(void *d, const void *s, size_t n, hipMemcpyKind, hipStream_t st)
+{
+    emu::submit(st, [=]() { memcpy(d, s, n); });
+    return hipSuccess;
+}
+inline hipError_t hipMemsetAsync(void *d, int v, size_t n, hipStream_t st)
+{
+    emu::submit(st, [=]() { memset(d, v, n); });
+    return hipSuccess;
+}
+inline hipError_t hipStreamSynchronize(hipStream_t st)
+{
+    if (emu::Stream *t = emu::lazy(st)) t->run_until(t->queued);
+    return hipSuccess;
+}
+inline hipError_t hipDeviceSynchronize() { emu::drain_all(); return hipSuccess; }
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline const char *hipGetErrorString(hipError_t) { return "emu"; }
 inline hipError_t hipGetDevice(int *d) { *d = 0; return hipSuccess; }
+inline hipError_t hipStreamCreateWithFlags(hipStream_t *s, unsigned) { emu::Stream *t = new emu::Stream(); emu::streams().push_back(t); *s = t; return hipSuccess; }
+inline hipError_t hipEventCreateWithFlags(hipEvent_t *e, unsigned) { *e = new emu::Event(); return hipSuccess; }
+inline hipError_t hipEventRecord(hipEvent_t e, hipStream_t st)
+{
+    emu::Stream *t = emu::eager_streams() ? nullptr : emu::lazy(st);
+    e->stream = t;
+    e->pos = t ? t->queued : 0;
+    return hipSuccess;
+}
+// the waiting stream may not pass the event: an eager stream (or the host) makes the event's stream catch up now, a
+// lazy stream does so when it gets there
+inline hipError_t hipStreamWaitEvent(hipStream_t st, hipEvent_t e, unsigned)
+{
+    emu::Stream *src = e->stream;
+    if (!src) return hipSuccess;
+    const size_t pos = e->pos;
+    emu::submit(st, [=]() { src->run_until(pos); });
+    return hipSuccess;
+}
 
 namespace emu {
 
@@ -224,9 +303,14 @@ inline void launch_k(unsigned grid, unsigned block, size_t shmem, K kernel, A...
 {
     launch(grid, block, shmem, [=]() { kernel(args...); });
 }
+template <typename K, typename... A>
+inline void launch_on(void *stream, unsigned grid, unsigned block, size_t shmem, K kernel, A... args)
+{
+    submit(stream, [=]() { launch(grid, block, shmem, [=]() { kernel(args...); }); });
+}
 }  // namespace emu
 #define F3M_EMU_LAUNCH(kernel, grid, block, shmem, stream, ...) \
-    emu::launch_k((unsigned)(grid), (unsigned)(block), (size_t)(shmem), kernel, __VA_ARGS__)
+    emu::launch_on((void *)(stream), (unsigned)(grid), (unsigned)(block), (size_t)(shmem), kernel, __VA_ARGS__)
 
 struct float4 { float x, y, z, w; };
 inline float4 make_float4(float x, float y, float z, float w) { return float4{x, y, z, w}; }

@@ -214,6 +214,36 @@ def test_m2l_forms_agree(monkeypatch, d, n, P, mp):
     assert rel_l2(grouped, direct) < 3e-6
 
 
+@pytest.mark.parametrize("P", [125, 216])
+def test_grids_of_five_and_six_nodes_per_dimension(oracle, monkeypatch, P):
+    """5 x 5 x 5 and 6 x 6 x 6 nodes (the grids of the reference's own sweep, experiments/experiments.py:47-49) on
+    their one-wavefront kernels: interpolation, sibling-group M2L, transfers between two levels, evaluation.  A thin
+    slab keeps the near field small for the emulation: 8 x 8 x 1 boxes of ~230 points at depth 3, far pairs at depths
+    2 and 3, half of every family of siblings missing."""
+    rng = np.random.default_rng(9)
+    X = (rng.random((15000, 3)) * np.array([1.0, 1.0, 1e-3])).astype(f32)
+    b = rng.standard_normal((15000, 1)).astype(f32)
+    prm = dict(ls=0.6, min_points=300, nr_of_interpolation=P, small_field_points=300)
+    eng = ee.Plan(X, None, **prm)
+    ora = oracle.Plan(X, None, **prm)
+    assert_plan_matches_oracle(eng, ora)
+    far_levels = [k for k in range(1, eng.depth + 1) if eng.level_sizes(k)["nfar"]]
+    assert len(far_levels) >= 2
+    for k in far_levels:                                  # P2M and M2L of every level against the oracle
+        out, mom, loc = eng.far_level(k, b, P)
+        o_out, o_mom, o_loc = ora.far_level(k - 1, b)
+        assert rel_l2(mom, np.moveaxis(o_mom, 2, 0)) < 1e-4
+        assert rel_l2(loc, np.moveaxis(o_loc, 2, 0)) < 1e-4
+        assert rel_l2(out, o_out) < 1e-4
+    sweeps = eng.apply(b)                                 # one interpolation, transfers between the levels, one evaluation
+    assert rel_l2(sweeps, ora.apply(b)) < 1e-5
+    monkeypatch.setenv("F3M_FAR", "levels")
+    assert 0 < rel_l2(sweeps, eng.apply(b)) < 3e-6
+    monkeypatch.delenv("F3M_FAR")
+    monkeypatch.setenv("F3M_M2L", "direct")
+    assert 0 < rel_l2(sweeps, eng.apply(b)) < 3e-6
+
+
 @pytest.mark.parametrize("parts", [2, 6])
 def test_m2l_sibling_table_in_parts(monkeypatch, parts):
     """the sibling-group M2L can fill and walk its table of far cells in several parts (for tables that do not fit LDS whole):

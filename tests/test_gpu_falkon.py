@@ -47,10 +47,11 @@ def test_falkon_matches_closed_form_and_fits():
     print("dmmv vs dense fp64: %.3e" % rel_dmmv, flush=True)
     assert rel_dmmv < 1e-3
     # With lambda = 1e-6 the Nystrom system is ill conditioned: the ~1e-4 relative error of the engine's
-    # products moves the coefficients along weakly determined directions, so predictions are compared
-    # loosely and the fit itself tightly (the CG + preconditioner arithmetic is pinned against the closed
-    # form with a dense kernel in tests/test_falkon_cpu.py).
-    assert rel < 0.1
+    # products moves the coefficients along weakly determined directions, so the pin of the operator is the
+    # dmmv check above and the fit is held tightly below; the predictions themselves agree with the closed form
+    # to the level the fp32 solves allow (1e-2 in tests/test_falkon_cpu.py, where the CG + preconditioner
+    # arithmetic is pinned against the closed form with a dense kernel).
+    assert rel < 1e-2                       # measured 1.1e-3
     assert mse < 1.05 * mse_ref + 1e-4
     ss_tot = float(((Y.double() - Y.double().mean()) ** 2).mean())
     assert 1 - mse / ss_tot > 0.9           # R^2 on the synthetic target (noise sd 0.1, signal var ~0.4)
@@ -100,3 +101,56 @@ def test_blocked_preconditioner_matches_whole_matrix_form_on_the_gpu():
         assert float((dense @ x - v).norm() / v.norm()) < 1e-3          # each solve inverts its own factor
         xt = fac.solve(v, transpose=True)
         assert float((dense.T @ xt - v).norm() / v.norm()) < 1e-3
+
+
+def test_falkon_at_the_benchmark_size():
+    """The kernel-ridge-regression configuration at its stated size: N = 1e7 points, M = 1e5 Nystrom centres, 20
+    conjugate-gradient iterations (reference protocol: conjugate_gradient/custom_falkon.py:119-244, experiments/
+    experiments_krr_a.py:49-97).  The tile-by-tile fp32 preconditioner holds two 40 GB factors: the test skips on a
+    device with less than 100 GiB free.  Checks: quality of the fit (R^2 >= 0.96, mse within 5 % of the noise
+    variance 0.01), and both engine products of the operator, K_nm v and K_nm^T u on the plan of the fit, against
+    the fp64 exact products on 2000 seeded rows each (< 1e-3)."""
+    import torch
+    from f3m_amd import engine
+    from f3m_amd.conjugate_gradient import FalkonOptions, custom_Falkon, custom_GaussianKernel
+    print("case falkon n=1e7 M=1e5", flush=True)
+    engine.release_cache()
+    torch.cuda.empty_cache()
+    free = torch.cuda.mem_get_info()[0] / 2 ** 30
+    if free < 100:
+        pytest.skip("%.0f GiB of device memory free, 100 needed" % free)
+    n, M, lam, sigma = 10_000_000, 100_000, 1e-6, 0.5
+    X, Y = _problem(n, seed=1)
+    opt = FalkonOptions()
+    kernel = custom_GaussianKernel(sigma, opt=opt, var_compression=False, interpolation_nr=64)
+    model = custom_Falkon(kernel, lam, M, maxiter=20, seed=1, options=opt)
+    model.fit(X, Y)
+    pred = model.predict(X)
+    mse = float(((pred - Y) ** 2).mean())
+    r2 = 1 - mse / float(((Y - Y.mean()) ** 2).mean())
+    print("fit: preconditioner %.1f s, CG %.2f s (%d iterations), mse %.5f, R^2 %.4f, peak device memory %.1f GiB"
+          % (model.fit_times_[0], model.conjugate_gradient_time, model.cg_iterations_, mse, r2,
+             torch.cuda.max_memory_allocated() / 2 ** 30), flush=True)
+    assert model.cg_iterations_ == 20
+    assert r2 >= 0.96
+    assert mse <= 1.05 * 0.01
+    # the two products of one iteration, on the plan of (X, centres) that the fit used
+    C = model.ny_points_
+    del model, pred
+    torch.cuda.empty_cache()
+    g = torch.Generator().manual_seed(11)
+    v, u = torch.randn(M, 1, generator=g).cuda(), torch.randn(n, 1, generator=g).cuda()
+    rows = torch.randint(0, n, (2000,), generator=g).cuda()
+    cols = torch.randint(0, M, (2000,), generator=g).cuda()
+    Kv = kernel.mmv(X, C, v)
+    Ktu = kernel.dmmv(X, C, None, u)
+    Xd, Cd = X.double(), C.double()
+    exact_rows = engine.exact_f64(Xd[rows].contiguous(), Cd, v.double(), sigma)
+    exact_cols = engine.exact_f64(Cd[cols].contiguous(), Xd, u.double(), sigma)
+    e1 = float((Kv[rows].double() - exact_rows).norm() / exact_rows.norm())
+    e2 = float((Ktu[cols].double() - exact_cols).norm() / exact_cols.norm())
+    print("K_nm v on 2000 rows: %.3e, K_nm^T u on 2000 rows: %.3e (vs fp64 exact)" % (e1, e2), flush=True)
+    assert e1 < 1e-3 and e2 < 1e-3
+    del kernel, X, Y, Xd, Cd
+    engine.release_cache()
+    torch.cuda.empty_cache()

@@ -51,6 +51,9 @@ def clouds(name, rng):
     if name == "uniform5_1024":      # 4^5 nodes: the siblings of a box do not fit one workgroup and are split in two
         return rng.random((1500000, 5), dtype=f32), None, dict(ls=1.5, nr_of_interpolation=1024, min_points=1000,
                                                                 small_field_points=300)
+    if name in ("uniform3_125", "uniform3_216"):     # the larger grids of the reference's own sweep (experiments/
+        # experiments.py:47-49): 390 points per box at depth 3, far pairs at depths 2 and 3
+        return rng.random((200000, 3), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=int(name.split("_")[1]))
     if name == "uniform2":
         return rng.random((80000, 2), dtype=f32), None, dict(ls=0.2)
     if name == "uniform1":
@@ -69,7 +72,8 @@ NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5", "unif
 # Clouds whose complete far field would keep the CPU oracle busy for minutes (far pairs x 243^2 kernel
 # evaluations): the oracle computes the target rows of a few boxes only (same sums, restricted to those rows)
 # and the GPU results are compared on them.
-ROW_BOXES = {"uniform5_243": [0, 17, 333, 512, 800, 1023]}
+ROW_BOXES = {"uniform5_243": [0, 17, 333, 512, 800, 1023], "uniform3_125": [0, 7, 100, 255, 256, 300, 480, 511],
+             "uniform3_216": [0, 7, 100, 255, 256, 300, 480, 511]}
 
 
 def selected_rows(name, level):
@@ -229,12 +233,12 @@ def test_exact_kernels(eng, oracle, d):
 
 
 @pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform5_243",
-                                  "uniform3_varcomp"])
+                                  "uniform3_varcomp", "uniform3_125", "uniform3_216"])
 def test_stages_against_oracle(eng, oracle, name):
     print("case stages", name, flush=True)
     rng = np.random.default_rng(7)
     X, Y, prm = clouds(name, rng)
-    if name not in ("uniform5", "uniform5_243"):          # the 5-D clouds need their points to have far pairs
+    if name not in ("uniform5", "uniform5_243", "uniform3_125", "uniform3_216"):   # these need their points to have far pairs
         X = X[:30000]
         Y = None if Y is None else Y[:12000]
     M = X.shape[0] if Y is None else Y.shape[0]
@@ -264,7 +268,7 @@ def test_stages_against_oracle(eng, oracle, name):
             assert rel_l2(mom.cpu().numpy(), np.moveaxis(o_mom, 2, 0)) < 1e-4     # P2M
             assert rel_l2(loc, o_loc) < 1e-4                                      # M2L
             assert rel_l2(out.cpu().numpy()[sel], o_out[sel]) < 1e-4              # L2P
-    assert far_levels >= (2 if name == "uniform5_243" else 1)
+    assert far_levels >= (2 if name in ("uniform5_243", "uniform3_125", "uniform3_216") else 1)
     if plan.level_sizes(plan.depth)["nkeep"]:
         got = plan.near_level(plan.depth, "keep", dev(b)).cpu().numpy()
         assert rel_l2(got[sel], ora.near_level(plan.depth - 1, "keep", b, rows=rows)[sel]) < 1e-5
@@ -432,7 +436,8 @@ def test_product_error_vs_fp64_exact(eng, oracle, name):
         assert err <= 1e-3, (err, err_oracle)
 
 
-@pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform5_1024", "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["uniform4", "uniform5", "uniform5_243", "uniform5_1024", "uniform3_varcomp", "uniform3_125",
+                                  "uniform3_216"])
 def test_m2l_forms_agree(eng, monkeypatch, name):
     """Sibling-group separable M2L (default for one tree, d >= 3) against the per-box separable form
     and the direct form of the reference (F3M_src/1_d_conv.cu:741-817): same sums up to rounding."""
@@ -551,7 +556,8 @@ def test_m2l_children_of_parent_pairs_kept_on_the_far_threshold(eng, monkeypatch
     assert 0 < rel_l2(grouped, per_box) < 2e-6
 
 
-@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform5", "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform5", "uniform3_varcomp", "uniform3_125",
+                                  "uniform3_216", "uniform4", "uniform5_243"])
 def test_far_sweeps_match_per_level_interpolation(eng, monkeypatch, name):
     """Default: points interpolated once, moments and local expansions moved between levels.
     F3M_FAR=levels: every level interpolated from the points like the reference
