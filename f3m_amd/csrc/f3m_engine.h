@@ -204,6 +204,17 @@ void gather_columns(const float *b, const int *perm, long long n, int c, int col
 void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
                      int ncol, float *out, hipStream_t s);
 
+// Results added straight into the caller's array instead of the sorted one: out[perm[i] * c + col + q] += value by a
+// hardware atomic addition.  The array is cleared before, and at most two values are added to an element (the near
+// field's sum and the far field's), so the result does not depend on which comes first: 0 + a + b = 0 + b + a.
+struct DirectOut {
+    const int *perm = nullptr;
+    float *out = nullptr;         // null: not used, results go to the sorted array
+    int c = 0, col = 0, ncol = 0; // row length of out, first column and number of columns of this pass
+};
+// whether near_field would take this list in one launch of the matrix-pipe kernel with one wavefront per work item
+// (the condition for DirectOut: every target is then written by exactly one wavefront)
+bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList &list, float lcs, int nc);
 // builds the table "box of every 32nd point" of a level now, on stream s, if it does not exist yet (kernels of
 // the near field and of L2P start from it; when those run on different streams the table must exist before)
 void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s);
@@ -214,7 +225,7 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 // prepare_only: build the tables of the list that are kept with the plan (tile table, source operands), launch nothing else
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc = 1, long long bstride = 0,
-                long long ostride = 0, bool only_list = false, bool prepare_only = false);
+                long long ostride = 0, bool only_list = false, bool prepare_only = false, const DirectOut *direct = nullptr);
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);
@@ -227,8 +238,9 @@ void p2m_level(int d, const Tree &ty, const TreeLevel &ly, const int *flag, Node
 // beside_near: the launch will run beside the near field of another stream (small workgroups then)
 void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, float lcs, int m2l_mode, const float *mom, float *loc /* overwritten */, hipStream_t s, bool beside_near = false);
+// direct (nullable, one column: direct->col is the column): results go to the caller's array
 void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
-               hipStream_t s);
+               hipStream_t s, const DirectOut *direct = nullptr);
 // expansions moved between a level and the next deeper one: moments up (down = false, dst = parent
 // moments, overwritten) or local expansions down (down = true, dst = child expansions, added to)
 bool nodes_nest(const NodeSet &coarse, const NodeSet &fine);

@@ -535,6 +535,16 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
 // no barriers: wavefronts are independent.  Rows past the end of a box are neutralised by a zero
 // weight (the exponent of any two vectors is -|x''-y'|^2 <= 0, so exp2 stays finite).
 constexpr int kNearWavesPerBlock = 2;
+// value of sorted point i, column q of the pass, added into the caller's array (see DirectOut)
+__device__ __forceinline__ void direct_add(const DirectOut &dout, long long i, int q, float value)
+{
+    float *p = dout.out + (long long)dout.perm[i] * dout.c + dout.col + q;
+#ifdef F3M_CPU_EMU
+    *p += value;
+#else
+    unsafeAtomicAdd(p, value);          // one hardware instruction (no compare-and-swap loop); out is ordinary device memory
+#endif
+}
 struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floats at any 4-byte boundary
 
 // NC right-hand sides at once: the exponential of a pair is computed once and multiplies NC weights
@@ -545,7 +555,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
     const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
-    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order)
+    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = near_insts(D);
@@ -730,7 +740,8 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             float total = acc[q][c] + wave_shfl_xor_f(acc[q][c], 32);
             if (half == 0 && i < x1) {
                 if (nsplit > 1) part[(((long long)slice * NC + c) * nitems + wid) * (TPW * 32) + q * 32 + col] = total;
-                else outs[c * ostride + i] += total;
+                else if (dout.out == nullptr) outs[c * ostride + i] += total;
+                else if (c < dout.ncol) direct_add(dout, i, c, total);
             }
         }
     }
@@ -820,9 +831,28 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
     build_near_operands(d, ty, ly, sqrtf(lcs * kLog2e), nullptr, s);
 }
 
+// the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
+// the list, the exact number of work items (else -1)
+static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact)
+{
+    const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
+    tpw = ((avg_points + 31) / 32 == 5 && nc == 1) ? 5 : 4;
+    if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
+    items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
+}
+
+bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList &list, float lcs, int nc)
+{
+    if (list.n == 0 || !near_on_matrix_pipe(d, lcs, lx.edge)) return false;
+    int tpw;
+    long long items_exact;
+    near_shape(tx, lx, list, nc, tpw, items_exact);
+    return items_exact >= 16384;          // fewer work items: the lists are cut into slices with partial sums
+}
+
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride,
-                bool only_list, bool prepare_only)
+                bool only_list, bool prepare_only, const DirectOut *direct)
 {
     if (list.n == 0) return;
     F3M_REQUIRE(nc == 1 || nc == 2 || nc == 4, 34, "near field takes 1, 2 or 4 columns at a time");
@@ -846,10 +876,9 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // (N=1e7, d=4, 153 points per box: 16.9 -> 15.6 ms at the time)
     // Where the plan has counted the rows of the list, "typical" is the mean over the listed boxes and the
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
-    const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
-    int tpw = ((avg_points + 31) / 32 == 5 && nc == 1) ? 5 : 4;
-    if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
-    const long long items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
+    int tpw;
+    long long items_exact;
+    near_shape(tx, lx, list, nc, tpw, items_exact);
     // From five dimensions on the work items are long and their lists differ a lot in length (3^5 boxes around
     // an interior box, 2^5 around a corner): the boxes with the longest lists go first, which shortens the
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
@@ -901,6 +930,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         }
         DBuf<float> part;
         if (nsplit > 1) part.reset((size_t)nsplit * nc * ntiles * tpw * 32);   // every slot of a live work item is written
+        F3M_REQUIRE(direct == nullptr || nsplit == 1, 35, "direct output needs a near field of one wavefront per work item");
+        const DirectOut dout = direct ? *direct : DirectOut();
         int nblk = (int)cdiv((long long)ntiles * nsplit, kNearWavesPerBlock);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
@@ -910,22 +941,22 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
             F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else if (nc == 4)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else if (nc == 2)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 2>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else                                                                                                          \
             F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
                        tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord);                                         \
+                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -940,6 +971,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         }
     } else {
         if (prepare_only) return;
+        F3M_REQUIRE(direct == nullptr, 35, "direct output needs the matrix-pipe near field");
         timer_begin(kNear, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
@@ -1641,10 +1673,11 @@ __global__ void sib_class_count_kernel(const int *__restrict__ childstart, const
     cls[p] = c;
     atomicAdd(&hist[c], 1);
 }
-// (grids of 5 or 6 nodes per dimension, 3-D only: a workgroup is one wavefront, and a lane's 3 N^2 partial sums and
-// its moments in flight need more registers than a 1024-thread bound would leave)
-template <int D, int N, int H>
-__global__ void __launch_bounds__((D == 3 && N >= 5) ? 64 : 1024) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
+// MAXT: the largest workgroup the instance is launched with.  It sets the registers a lane may use: 128 under the
+// general bound of 1024 threads, which a lane's 3 N^2 partial sums and its moments in flight exceed by far at 5 or 6
+// nodes per dimension; those grids (3-D only, workgroups of one wavefront) have instances bound to 64 threads.
+template <int D, int N, int H, int MAXT>
+__global__ void __launch_bounds__(MAXT) m2l_sib_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, NodeMeta nm,
                                                         int R2, int GS, int nsub, int npass, const int *__restrict__ order,
                                                         const int *__restrict__ childstart,
                                                         const int *__restrict__ cell, const int *__restrict__ pairs,
@@ -1963,7 +1996,7 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict_
                                                          const int *__restrict__ off, const float *__restrict__ ctr,
                                                          const int *__restrict__ tileoff, int nb, NodeMeta nm,
                                                          const float *__restrict__ nt, const float *__restrict__ nw,
-                                                         float factor, const float *__restrict__ loc)
+                                                         float factor, const float *__restrict__ loc, DirectOut dout)
 {
     F3M_DYN_SHARED(float, smem);
     const int S1p = nm.S1 | 1;               // odd stride: lanes hit distinct LDS banks
@@ -2007,7 +2040,8 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_kernel(const float *__restrict_
             idx[k] = 0;
         }
     }
-    outs[i] += acc;
+    if (dout.out == nullptr) outs[i] += acc;
+    else direct_add(dout, i, 0, acc);
 }
 
 void mark_far_boxes(const PairList &far, int nbx, int nby, int *fx, int *fy, hipStream_t s)
@@ -2199,23 +2233,27 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
                 check_launch("sib_class_place");
             }
             const int *sibOrd = ordered ? sibOrder.get() : (const int *)nullptr;
+            // (instances bound to 128 threads for the groups of four siblings that run beside the near field, 4-D and 5-D,
+            // have no spilled values but one wavefront per SIMD less: same time, not kept)
+            const int maxt = (d == 3 && ns.n[0] >= 5) ? 64 : 1024;
 #ifndef F3M_CPU_EMU
-#define F3M_SIB_ATTR(DD, NNODE, HH)                                                                                    \
-    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE, HH>),                        \
+#define F3M_SIB_ATTR(DD, NNODE, HH, MT)                                                                                \
+    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE, HH, MT>),                    \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shsib));
 #else
-#define F3M_SIB_ATTR(DD, NNODE, HH)
+#define F3M_SIB_ATTR(DD, NNODE, HH, MT)
 #endif
-#define F3M_SIB(DD, NNODE, HH)                                                                                         \
-    if (d == DD && ns.n[0] == NNODE && sibH == HH) {                                                                   \
-        F3M_SIB_ATTR(DD, NNODE, HH)                                                                                    \
-        F3M_LAUNCH((m2l_sib_kernel<DD, NNODE, HH>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2,      \
+#define F3M_SIB(DD, NNODE, HH, MT)                                                                                     \
+    if (d == DD && ns.n[0] == NNODE && sibH == HH && maxt == MT) {                                                     \
+        F3M_SIB_ATTR(DD, NNODE, HH, MT)                                                                                \
+        F3M_LAUNCH((m2l_sib_kernel<DD, NNODE, HH, MT>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2,  \
                    sibGS, nsub, sibPass, sibOrd, par.childstart.get(), lx.cell.get(), far.pairs.get(),                 \
                    far.rowptr.get(), mom, loc);                                                                        \
     }
-            F3M_SIB(3, 2, 2) F3M_SIB(3, 3, 1) F3M_SIB(3, 4, 2) F3M_SIB(3, 2, 1) F3M_SIB(3, 4, 1) F3M_SIB(3, 5, 1) F3M_SIB(3, 6, 1)
-            F3M_SIB(4, 2, 1) F3M_SIB(4, 3, 1) F3M_SIB(4, 4, 1)
-            F3M_SIB(5, 2, 1) F3M_SIB(5, 3, 1) F3M_SIB(5, 4, 1)
+            F3M_SIB(3, 2, 2, 1024) F3M_SIB(3, 3, 1, 1024) F3M_SIB(3, 4, 2, 1024) F3M_SIB(3, 2, 1, 1024) F3M_SIB(3, 4, 1, 1024)
+            F3M_SIB(3, 5, 1, 64) F3M_SIB(3, 6, 1, 64)
+            F3M_SIB(4, 2, 1, 1024) F3M_SIB(4, 3, 1, 1024) F3M_SIB(4, 4, 1, 1024)
+            F3M_SIB(5, 2, 1, 1024) F3M_SIB(5, 3, 1, 1024) F3M_SIB(5, 4, 1, 1024)
 #undef F3M_SIB
 #undef F3M_SIB_ATTR
         } else if (q64) {
@@ -2275,7 +2313,7 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restr
                                                              const int *__restrict__ off, const float *__restrict__ ctr,
                                                              int nb, const int *__restrict__ box32,
                                                              const float *__restrict__ nt, const float *__restrict__ nw,
-                                                             float factor, const float *__restrict__ loc)
+                                                             float factor, const float *__restrict__ loc, DirectOut dout)
 {
     __shared__ int bounds[kL2PBlock];
     const int tid = threadIdx.x;
@@ -2309,7 +2347,8 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_q64_kernel(const float *__restr
         inner = fmaf(l[0][3], r.w, inner);
         acc = fmaf(l[1][h & 3] * l[2][h >> 2], inner, acc);
     }
-    outs[i] += acc;
+    if (dout.out == nullptr) outs[i] += acc;
+    else direct_add(dout, i, 0, acc);
 }
 
 // The same for other tensor grids of N nodes per dimension: the weights of the nodes of dimensions >= 1
@@ -2319,7 +2358,7 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_tensor_kernel(const float *__re
                                                                 const int *__restrict__ off, const float *__restrict__ ctr,
                                                                 int nb, const int *__restrict__ box32,
                                                                 const float *__restrict__ nt, const float *__restrict__ nw,
-                                                                float factor, const float *__restrict__ loc)
+                                                                float factor, const float *__restrict__ loc, DirectOut dout)
 {
     constexpr int Q = ipow(N, D - 1), P = Q * N;
     __shared__ int bounds[kL2PBlock];
@@ -2363,12 +2402,14 @@ __global__ void __launch_bounds__(kL2PBlock) l2p_tensor_kernel(const float *__re
         for (int e = 1; e < N; e++) inner = fmaf(l[0][e], r.v[e], inner);
         acc = fmaf(w[j], inner, acc);
     }
-    outs[i] += acc;
+    if (dout.out == nullptr) outs[i] += acc;
+    else direct_add(dout, i, 0, acc);
 }
 
 void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, NodeSet &ns, const float *loc, float *outs,
-               hipStream_t s)
+               hipStream_t s, const DirectOut *direct)
 {
+    const DirectOut dout = direct ? *direct : DirectOut();
     check_nodes(ns);
     const int P = ns.P;
     NodeMeta nm = meta_of(ns);
@@ -2376,7 +2417,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 4 && ns.n[1] == 4 && ns.n[2] == 4) {
         timer_begin(kL2P, s);
         F3M_LAUNCH(l2p_q64_kernel, cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_q64");
         return;
@@ -2384,7 +2425,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 4 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<4, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2392,7 +2433,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 5 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3 && ns.n[3] == 3 && ns.n[4] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<5, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2400,7 +2441,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 3 && ns.n[1] == 3 && ns.n[2] == 3) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<3, 3>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2408,7 +2449,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 5 && ns.n[1] == 5 && ns.n[2] == 5) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<3, 5>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2416,7 +2457,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
     if (flag == nullptr && d == 3 && ns.n[0] == 6 && ns.n[1] == 6 && ns.n[2] == 6) {
         timer_begin(kL2P, s);
         F3M_LAUNCH((l2p_tensor_kernel<3, 6>), cdiv(tx.n, kL2PBlock), kL2PBlock, 0, s, tx.pts.get(), tx.n, outs, lx.off.get(),
-                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc);
+                   lx.ctr.get(), lx.nb, box_table(lx, tx.n, s), ns.dt.get(), ns.dw.get(), factor, loc, dout);
         timer_end(s);
         check_launch("l2p_tensor");
         return;
@@ -2437,7 +2478,7 @@ void l2p_level(int d, const Tree &tx, const TreeLevel &lx, const int *flag, Node
 #define F3M_CASE(DD)                                                                                                   \
     case DD:                                                                                                           \
         F3M_LAUNCH((l2p_kernel<DD>), ntx, kL2PBlock, shl, s, tx.pts.get(), tx.n, outs, lx.off.get(), lx.ctr.get(),     \
-                   tilex.get(), lx.nb, nm, ns.dt.get(), ns.dw.get(), factor, loc);                                     \
+                   tilex.get(), lx.nb, nm, ns.dt.get(), ns.dw.get(), factor, loc, dout);                                     \
         break;
     if (ntx > 0) {
         timer_begin(kL2P, s);

@@ -97,6 +97,7 @@ struct f3m_plan {
     DBuf<float> early_outs, early_outs_far;   // the result arrays of that column group, cleared beside the last level's lists
     const float *early_b = nullptr;
     int early_c = 0, early_ncol = 0;
+    float *early_out = nullptr;               // the caller's result array, cleared beside the last level's lists (N x early_c floats)
     std::map<std::pair<int, int>, std::unique_ptr<DBuf<float>>> shift_tabs;   // (parent nodes, child nodes)
     const float *shift_table(int nodes_parent, int nodes_child, hipStream_t s)
     {
@@ -207,12 +208,13 @@ static SideStream &side_stream()
 // when the last kernels of the plan are queued, not when they are done: the product is queued behind them on the
 // same stream (every host-side figure of the plan is known by then), so the GPU does not wait for the host in between.
 static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y, long long M, const f3m_params *prm,
-                             hipStream_t s, const float *b_early = nullptr, int c_early = 0)
+                             hipStream_t s, const float *b_early = nullptr, int c_early = 0, float *out_early = nullptr)
 {
     bool sym = (Y == nullptr || Y == X);
     check_params(d, N, M, sym, prm);
     check_device_ptr(X, "X");
     if (!sym) check_device_ptr(Y, "Y");
+    if (out_early != nullptr) check_device_ptr(out_early, "out");       // it is written before the product checks it
     std::unique_ptr<f3m_plan> P(new f3m_plan());
     P->d = d; P->symmetric = sym; P->N = N; P->M = sym ? N : M; P->prm = *prm;
     P->lcs = 1 / (2 * prm->ls * prm->ls);                        // F3M_src/n_tree.cu:1060
@@ -393,6 +395,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
                     dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
                     dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
+                    if (out_early != nullptr) {     // and the caller's array, for a product that adds its results straight into it
+                        dev_fill(out_early, 0, sizeof(float) * (size_t)P->N * P->early_c, side_stream().stream);
+                        P->early_out = out_early;
+                    }
                 }
             }
             // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
@@ -473,7 +479,10 @@ static void far_level(f3m_plan *P, int level, const float *bs, float *outs, floa
 // Where a level has more nodes per dimension than the next deeper one (var_compression lowers the node
 // count of small boxes, F3M_src/n_tree.cu:971-978) the hand-over would not be exact, and that level
 // is interpolated from / evaluated at the points directly, as the reference does for every level.
-static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs, hipStream_t s, bool beside_near = false)
+// direct (nullable): the one evaluation at the points adds into the caller's array (only where the node counts of the
+// levels allow the single evaluation)
+static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs, hipStream_t s, bool beside_near = false,
+                     const DirectOut *direct = nullptr)
 {
     const int depth = (int)P->levels.size();
     // targets and sources of this product: the X and Y tree, or the other way round for K(X,Y)^T
@@ -514,13 +523,14 @@ static void far_tree(f3m_plan *P, bool transposed, const float *bs, float *outs,
                 const float *tab = P->shift_table(P->levels[pending - 1].num_nodes, P->levels[k - 1].num_nodes, s);
                 shift_level(true, TX.lev[pending], lx, nsp, ns, tab, prev.get(), loc.get(), s);
             } else {
+                F3M_REQUIRE(direct == nullptr, 36, "direct output with more than one evaluation of the far field");
                 l2p_level(d, TX, TX.lev[pending], nullptr, nsp, prev.get(), outs, s);
             }
         }
         std::swap(loc, prev);
         pending = k;
     }
-    l2p_level(d, TX, TX.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s);
+    l2p_level(d, TX, TX.lev[pending], nullptr, ns_of(pending), prev.get(), outs, s, direct);
 }
 
 // The lists seen from the Y boxes, for the transposed product (built once, on its first use).
@@ -594,9 +604,47 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         const char *oe = getenv("F3M_OVERLAP");
         overlap = any_far && !per_level && g_arena == nullptr && !(oe && atoi(oe) == 0);
     }
+    // Where the whole near field is one launch in which every target belongs to one wavefront, and the far field is
+    // evaluated at the points once, both add their sums straight into the caller's array (cleared before; two additions
+    // per element, so their order does not matter) and the pass that scatters the sorted results is not needed: the
+    // scattered writes happen inside the two long kernels instead of after them.  F3M_DIRECT=0 turns it off.
+    bool direct = false;
+    if (overlap && !(getenv("F3M_DIRECT") && atoi(getenv("F3M_DIRECT")) == 0)) {
+        int ku = 0, kd = 0;
+        bool same_nodes = true;
+        for (int k = 1; k <= depth; k++)
+            if ((transposed ? P->levels[k - 1].farT.n : P->levels[k - 1].far.n) > 0) {
+                if (kd && P->levels[k - 1].num_nodes != P->levels[kd - 1].num_nodes) same_nodes = false;
+                if (!ku) ku = k;
+                kd = k;
+            }
+        int nlists = 0;
+        direct = same_nodes;
+        for (int k = 1; k <= depth && direct; k++) {
+            const PairList *ls[2] = {&small_of(k), k == depth ? &keep_of(depth) : nullptr};
+            for (const PairList *l : ls) {
+                if (l == nullptr || l->n == 0) continue;
+                nlists++;
+                // every column group of this product (four columns while three or more are left, then two or one)
+                for (int left = c; left > 0 && direct;) {
+                    const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);
+                    direct = near_single_pass(P->d, TX, TX.lev[k], *l, P->lcs, nc);
+                    left -= std::min(nc, left);
+                }
+            }
+        }
+        direct = direct && nlists == 1;          // (without a near field to hide them, the atomic additions of the far field alone take longer than the pass they replace: 0.50 against 0.13 + 0.17 ms)
+    }
+    if (direct) {
+        if (!(P->early_out == out && P->early_c == c && !transposed)) {
+            Scope sc(kPerm, s);
+            dev_fill(out, 0, sizeof(float) * (size_t)NT * c, s);
+        }
+        P->early_out = nullptr;
+    }
     DBuf<float> outs_far;
     if (overlap) {
-        outs_far.reset((size_t)ostride * width);
+        if (!direct) outs_far.reset((size_t)ostride * width);
         // The one table that kernels of both streams read has to exist before the streams part: L2P starts from the
         // box table of the deepest level with far pairs (and of every level with far pairs where the node counts
         // change between levels, since such levels are evaluated at the points themselves).
@@ -629,7 +677,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 P->early_bs.free();
                 if (P->early_outs.size() > 0) {             // and its result arrays cleared
                     std::swap(outs, P->early_outs);
-                    if (overlap) std::swap(outs_far, P->early_outs_far);
+                    if (overlap && !direct) std::swap(outs_far, P->early_outs_far);
                     P->early_outs.free();
                     P->early_outs_far.free();
                     cleared = true;
@@ -638,7 +686,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 if (nc > ncol) dev_fill(bs.get(), 0, sizeof(float) * (size_t)bstride * nc, s);
                 gather_columns(b, TY.perm.get(), NS, c, col, ncol, bs.get(), bstride, s);
             }
-            if (!cleared) {
+            if (!cleared && !direct) {
                 dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
                 if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
             }
@@ -661,10 +709,13 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             }
             // the near field first: it is the long pole, and the host needs a while to queue the far field's many
             // small kernels
+            DirectOut dnear;
+            if (direct) { dnear.perm = TX.perm.get(); dnear.out = out; dnear.c = c; dnear.col = col; dnear.ncol = ncol; }
+            const DirectOut *dn = direct ? &dnear : nullptr;
             for (int k = 1; k <= depth; k++) {
                 // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
                 near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
-                           bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0);
+                           bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0, false, dn);
                 if (per_level) {
                     const size_t mark = arena_mark();
                     for (int q = 0; q < ncol; q++) {
@@ -675,7 +726,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             }
             // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
             near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
-                       outs.get(), P->lcs, s, nc, bstride, ostride);
+                       outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
             // the far field: beside the near field on the second stream into its own array, or after it on the one
             // stream; either way a result is (near sums) + (far sum)
             if (!per_level) {
@@ -685,7 +736,10 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 const size_t mark = arena_mark();
                 for (int q = 0; q < ncol; q++) {
                     arena_rewind(mark);
-                    far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap);
+                    DirectOut dfar = dnear;
+                    dfar.col = col + q;
+                    dfar.ncol = 1;
+                    far_tree(P, transposed, bs.get() + q * bstride, fo + q * ostride, fs, overlap, direct ? &dfar : nullptr);
                 }
             }
             if (overlap) {
@@ -693,7 +747,8 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 F3M_HIP(hipStreamWaitEvent(s, side_stream().join, 0));
             }
             Scope sc(kPerm, s);
-            scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
+            if (!direct)
+                scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
         }
         col += ncol;
     }
@@ -750,7 +805,7 @@ int f3m_kmvm_f32(int d, const float *X, int64_t N, const float *Y, int64_t M, co
     return guarded([&] {
         hipStream_t s = (hipStream_t)stream;
         g_timer.reset();
-        std::unique_ptr<f3m_plan> P(plan_create(d, X, N, Y, M, params, s, b, c));
+        std::unique_ptr<f3m_plan> P(plan_create(d, X, N, Y, M, params, s, b, c, out));
         plan_apply(P.get(), b, c, out, s);
         g_timer.collect();
     });
