@@ -215,6 +215,13 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     check_device_ptr(X, "X");
     if (!sym) check_device_ptr(Y, "Y");
     if (out_early != nullptr) check_device_ptr(out_early, "out");       // it is written before the product checks it
+    // (a caller that passes overlapping b and out against the interface's rule at least keeps the old order: all of
+    // b is read before the first write to out)
+    if (out_early != nullptr && b_early != nullptr) {
+        const char *b0 = reinterpret_cast<const char *>(b_early), *o0 = reinterpret_cast<const char *>(out_early);
+        const size_t bb = sizeof(float) * (size_t)(sym ? N : M) * (size_t)std::max(c_early, 0), ob = sizeof(float) * (size_t)N * (size_t)std::max(c_early, 0);
+        if (b0 < o0 + ob && o0 < b0 + bb) out_early = nullptr;
+    }
     std::unique_ptr<f3m_plan> P(new f3m_plan());
     P->d = d; P->symmetric = sym; P->N = N; P->M = sym ? N : M; P->prm = *prm;
     P->lcs = 1 / (2 * prm->ls * prm->ls);                        // F3M_src/n_tree.cu:1060
@@ -609,7 +616,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     // per element, so their order does not matter) and the pass that scatters the sorted results is not needed: the
     // scattered writes happen inside the two long kernels instead of after them.  F3M_DIRECT=0 turns it off.
     bool direct = false;
-    if (overlap && !(getenv("F3M_DIRECT") && atoi(getenv("F3M_DIRECT")) == 0)) {
+    const bool b_out_overlap = reinterpret_cast<const char *>(b) < reinterpret_cast<const char *>(out) + sizeof(float) * (size_t)NT * c &&
+                               reinterpret_cast<const char *>(out) < reinterpret_cast<const char *>(b) + sizeof(float) * (size_t)NS * c;
+    if (overlap && !b_out_overlap && !(getenv("F3M_DIRECT") && atoi(getenv("F3M_DIRECT")) == 0)) {
         int ku = 0, kd = 0;
         bool same_nodes = true;
         for (int k = 1; k <= depth; k++)
@@ -635,6 +644,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         }
         direct = direct && nlists == 1;          // (without a near field to hide them, the atomic additions of the far field alone take longer than the pass they replace: 0.50 against 0.13 + 0.17 ms)
     }
+    // F3M_DIRECT=2 (testing aid): fail where the results cannot go straight into the caller's array
+    F3M_REQUIRE(direct || !(getenv("F3M_DIRECT") && atoi(getenv("F3M_DIRECT")) == 2), 37,
+                "F3M_DIRECT=2: this product does not qualify for direct output");
     if (direct) {
         if (!(P->early_out == out && P->early_c == c && !transposed)) {
             Scope sc(kPerm, s);

@@ -5,7 +5,8 @@
  * the duration of the call and never modified except `out`.  `stream` is a hipStream_t passed as
  * void* (NULL = the default stream).  Every function returns 0 on success or a positive error
  * code; f3m_last_error() then returns a message for the calling thread.  Calls are synchronous:
- * the stream is idle when they return.  One call at a time per device (the engine keeps a cache of
+ * the stream is idle when they return.  `out` must not overlap X, Y or b (it may be written before the
+ * inputs have been read for the last time).  One call at a time per device (the engine keeps a cache of
  * device buffers, per device, that concurrent calls would share).  The device of the pointers must be
  * the calling thread's current device (hipSetDevice), for plans during create, apply and destroy.
  *

@@ -631,6 +631,36 @@ def test_repeated_products_have_the_same_bits(eng):
             assert np.array_equal(plans[i].apply(b).cpu().numpy(), first[i]), (rep, i, "plan")
 
 
+@pytest.mark.parametrize("c", [1, 3, 6])
+def test_results_added_straight_into_the_output_array(eng, monkeypatch, c):
+    """Where the near field is one launch with one wavefront per work item and the far field is evaluated once, both
+    add their sums straight into the caller's array (atomic additions into a cleared array, two per element) instead
+    of going through sorted arrays and a scatter pass.  Same bits as the scatter form (a + b either way), for the
+    one-shot call and for a kept plan, with one, three (padded to four) and six (four + two) columns; and the same
+    bits again when repeated."""
+    import torch
+    from f3m_amd.capi import F3MError
+    print("case direct output, %d columns" % c, flush=True)
+    rng = np.random.default_rng(41)
+    n = 2_600_000                                   # 4096 boxes of ~635 points: 20480 work items of 128 targets
+    X = dev(rng.random((n, 3), dtype=f32))
+    b = dev(rng.standard_normal((n, c)).astype(f32))
+    monkeypatch.setenv("F3M_DIRECT", "0")
+    want = eng.kmvm(X, None, b, ls=1.0)
+    monkeypatch.setenv("F3M_DIRECT", "2")           # fails if the product does not take the direct path
+    got = eng.kmvm(X, None, b, ls=1.0)
+    assert torch.equal(got, want)
+    plan = eng.Plan(X, None, ls=1.0)
+    assert torch.equal(plan.apply(b), want)
+    assert torch.equal(plan.apply(b), want)
+    plan.close()
+    # a cloud whose near field is cut into slices does not qualify
+    small = dev(rng.random((100000, 3), dtype=f32))
+    with pytest.raises(F3MError) as e:
+        eng.kmvm(small, None, dev(rng.standard_normal((100000, 1)).astype(f32)), ls=1.0)
+    assert e.value.code == 37
+
+
 def test_inputs_at_any_four_byte_alignment(eng):
     """Views that start in the middle of an allocation (12-byte rows) are not 16-byte aligned."""
     rng = np.random.default_rng(17)
