@@ -31,9 +31,10 @@ struct TreeLevel {
     DBuf<int> parent;       // nb: compact id at depth-1 of each box's parent (the root: 0)
     // near-field source operands of this level (built on first use by near_field): per point, the
     // split-f16 matrix operand of its coordinates relative to its own box centre, scaled by nearops_sc
-    mutable DBuf<unsigned char> nearops;
+    // Two tables, each built at most once and never replaced (a launch recorded into a graph keeps its address):
+    // nearops_all holds every box, nearops only the source boxes of the level's one near list.
+    mutable DBuf<unsigned char> nearops, nearops_all;
     mutable float nearops_sc = 0.f;
-    mutable bool nearops_partial = false;   // built for the source boxes of one list only
     // grid key -> box id table of this level (built on first use by lookup_boxes)
     // box of every 32nd point (npoints/32 + 2 entries, built on first use by box_table): kernels that
     // take points in fixed-size pieces start from here instead of searching the offsets
@@ -87,7 +88,7 @@ struct PairList {
 };
 
 struct ClassifyParams {
-    int omin[kMaxD];     // m2l_table_omin per dimension (set by lists_launch)
+    int omin[kMaxD];     // m2l_table_omin per dimension (set by level_launch)
     int nr_interp;
     int small_limit;
     int var_comp;
@@ -131,29 +132,29 @@ void root_geometry_launch(const float *partx, unsigned gridx, const float *party
 void sort_tree_launch(Tree &t, const float *X, long long n, int d, int L, const float *origin, const float *edge0p, hipStream_t s);
 void root_level_launch(Tree &t, const Geo &geo, hipStream_t s);
 void gather_tree_points(Tree &t, const float *X, hipStream_t s, bool background = false);
-// One division in two steps, so that the host can wait once for several results: divide_launch starts
-// the kernels that build lev[k] from lev[k-1] and appends the level; divide_finish completes it with
-// the two numbers the kernels left in dstats (boxes, largest count) once the host has fetched them;
-// divide_discard drops a level that turned out not to be needed.
-void divide_launch(Tree &t, int *dstats, hipStream_t s);
+// The division to a new depth is queued by level_launch (below) and appended to the tree with its box count and
+// largest count still unknown; divide_finish completes it with the two numbers the kernels left in dstats once the
+// host has fetched them; divide_discard drops a level that turned out not to be needed.
 // Levels whose boxes the sorted key bits resolve; the count of the fullest cell at that depth (added to *dout by
 // atomicMax, *dout zero before): if it exceeds the division threshold the tree will go deeper than the sorted bits
 // reach, and sort_more_bits (eight more key bits; the levels built so far stay valid) is due sooner or later.
 int sorted_levels(const Tree &t);
 void max_run_launch(const Tree &t, int *dout, hipStream_t s);
 void sort_more_bits(Tree &t, hipStream_t s);
-// whether the next divide_launch will first sort more key bits (and thereby replace the key and order arrays)
+// whether the next division will first sort more key bits (and thereby replace the key and order arrays)
 bool divide_will_sort(const Tree &t);
 void divide_finish(Tree &t, const int *hstats);
 void divide_discard(Tree &t);
-// The lists of depth k from the keep list of depth k-1, likewise: lists_launch counts and scans (the
-// sizes of the small, far and keep list are then the last entries pos[(c+1)*stride - 1] of the three
-// scans; the number of far pairs outside the sibling-group tables is added to dtot[3] and of those outside
-// the M2L tables of the level to dtot[6], which the caller keeps zero between levels; the row statistics of the
-// small and the keep list -- x boxes with pairs, their points, their pieces of 128 and of 160 points -- are added
-// to the eight zeroed words drow), lists_finish allocates from the fetched totals htot[0..3], takes the fetched row
-// statistics hrow[0..7] and writes.
-// divide_launch likewise adds to dstats[0..1], zero on entry.
+// One step of the level loop, queued as one group of launches: the counting pass of the lists of depth k from the keep
+// list of depth k-1 (keep_prev; null or empty: no lists) and, if `divide`, the division of both trees to depth k+1
+// (dstats_x, dstats_y: two zeroed words each, to which the kernels add the new level's boxes and largest count).  The
+// two are independent, so their kernels share launches: one for the counting pass and the candidates' point ranges,
+// one set for all the scans.  After it the sizes of the small, far and keep list are the last entries
+// pos[(c+1)*stride - 1] of the three scans; the number of far pairs outside the sibling-group tables has been added to
+// dtot[3] and of those outside the M2L tables of the level to dtot[6], which the caller keeps zero between levels; the
+// row statistics of the small and the keep list -- x boxes with pairs, their points, their pieces of 128 and of 160
+// points -- have been added to the eight zeroed words drow (nullable).  lists_finish allocates from the fetched totals
+// htot[0..3], takes the fetched row statistics hrow[0..7] and writes.
 struct ListsPending {
     DBuf<long long> pos;
     long long stride = 0;
@@ -161,8 +162,8 @@ struct ListsPending {
     bool active = false;
     bool written = false;    // the writing pass has been queued (lists_write_early)
 };
-void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
-                  ListsPending &pend, long long *dtot, long long *drow /* 8 zeroed words or null */, hipStream_t s);
+void level_launch(const PairList *keep_prev, Tree &tx, Tree &ty, int k, ClassifyParams &cp, ListsPending &pend,
+                  long long *dtot, long long *drow, bool divide, int *dstats_x, int *dstats_y, hipStream_t s);
 // queues the writing pass before the sizes are known, into lists allocated for an upper bound of the pairs, if that
 // bound is modest (returns whether it did; lists_finish then only records the sizes)
 bool lists_write_early(ListsPending &pend, const PairList &keep_prev, const Tree &tx, const Tree &ty, int k,

@@ -787,16 +787,20 @@ static bool near_on_matrix_pipe(int d, float lcs, float edge)
 
 // The split-f16 source operands of a level, kept with it.  only (nullable): operands are needed for the source boxes
 // of this list alone (at most levels a small part of the boxes); otherwise for every box.
-static void build_near_operands(int d, const Tree &ty, const TreeLevel &ly, float sc, const PairList *only, hipStream_t s)
+// Returns the table to use: the one of every box if it exists, else (for a list that is the level's only one) the table
+// of that list's source boxes; whichever is missing is built, none is ever rebuilt.
+static const h8 *build_near_operands(int d, const Tree &ty, const TreeLevel &ly, float sc, const PairList *only, hipStream_t s)
 {
     const bool only_list = only != nullptr;
-    if (ly.nearops.size() != 0 && ly.nearops_sc == sc && !(ly.nearops_partial && !only_list)) return;
+    F3M_REQUIRE(ly.nearops_sc == 0.f || ly.nearops_sc == sc, 38, "near-field operands of a level asked for with another lengthscale");
+    if (ly.nearops_all.size() != 0) return reinterpret_cast<const h8 *>(ly.nearops_all.get());
+    if (only_list && ly.nearops.size() != 0) return reinterpret_cast<const h8 *>(ly.nearops.get());
     const int NS = near_insts(d);
     const long long stride = ty.n + 32;
     require_tables_may_be_built("the near-field source operands of a level");
-    ly.nearops.reset((size_t)NS * 2 * stride * 16);
+    DBuf<unsigned char> &table = only_list ? ly.nearops : ly.nearops_all;
+    table.reset((size_t)NS * 2 * stride * 16);
     ly.nearops_sc = sc;
-    ly.nearops_partial = only_list;
     DBuf<int> need;
     if (only_list) {
         DBuf<int> fy((size_t)ly.nb);
@@ -812,7 +816,7 @@ static void build_near_operands(int d, const Tree &ty, const TreeLevel &ly, floa
         F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
                    ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
                    only_list ? need.get() : (const int *)nullptr, box32,                                              \
-                   reinterpret_cast<h8 *>(ly.nearops.get()));                                                         \
+                   reinterpret_cast<h8 *>(table.get()));                                                              \
         break;
     switch (d) {
         F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -821,6 +825,7 @@ static void build_near_operands(int d, const Tree &ty, const TreeLevel &ly, floa
     }
 #undef F3M_CASE
     check_launch("near_operands");
+    return reinterpret_cast<const h8 *>(table.get());
 }
 
 // The operands of every box of a level, ahead of the near field (the plan calls this for its deepest level, beside
@@ -915,7 +920,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
         const long long stride = ty.n + 32;
-        build_near_operands(d, ty, ly, sc, only_list ? &list : nullptr, s);
+        const h8 *srcops = build_near_operands(d, ty, ly, sc, only_list ? &list : nullptr, s);
         if (prepare_only) return;
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
@@ -939,22 +944,22 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     case DD:                                                                                                          \
         if (tpw == 5)                                                                                                 \
             F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else if (nc == 4)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else if (nc == 2)                                                                                             \
             F3M_LAUNCH((near_g_kernel<DD, 4, 2>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         else                                                                                                          \
             F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, reinterpret_cast<const h8 *>(ly.nearops.get()), stride, bs, bstride, outs, \
+                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
                        tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
         break;

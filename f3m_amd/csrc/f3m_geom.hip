@@ -190,6 +190,164 @@ void exclusive_scan_i64(const long long *in, long long n, long long *out, hipStr
     exclusive_scan<long long, long long>(in, n, out, s);
 }
 
+// Several independent scans in one set of launches (the level loop's: the three list counts of depth k, and per tree the
+// "candidate box is not empty" flags of depth k+1).  A channel of kind 0 scans n 64-bit values into n+1 64-bit
+// outputs; a channel of kind 1 scans the flags in[i+1] > in[i] of n+1 non-decreasing 32-bit entries into n+1 32-bit
+// outputs.  One tile launch; where a channel has more than one tile, a launch that scans the tile sums (one workgroup
+// per channel, so at most kScanTile tiles per channel) and one that adds them.
+// Folded in: the row statistics of the small and the keep list (channels rs_ch[0], rs_ch[1] of kind 0, or -1): x boxes
+// with pairs, their points, their pieces of 128 and of 160 points, added to rowstat[4c .. 4c+3] (zero before).
+constexpr int kMaxScanCh = 5;
+struct ScanChannel {
+    const void *in;
+    void *out;
+    long long n;
+    int kind;
+    unsigned tile0, ntiles;
+};
+struct ScanJob {
+    ScanChannel ch[kMaxScanCh];
+    int nch = 0;
+    unsigned blocks = 0;
+    const int *offx = nullptr;
+    unsigned long long *rowstat = nullptr;
+    int rs_ch[2] = {-1, -1};
+    void add(const void *in, void *out, long long n, int kind)
+    {
+        if (nch >= kMaxScanCh) throw Error(103, "too many scan channels");
+        const unsigned nt = cdiv(n + 1, kScanTile);
+        ch[nch++] = ScanChannel{in, out, n, kind, blocks, nt};
+        blocks += nt;
+    }
+};
+
+__global__ void __launch_bounds__(kScanBlock) multi_scan_tile_kernel(ScanJob job, long long *__restrict__ tilesum)
+{
+    __shared__ long long sh[kScanBlock];
+    __shared__ unsigned long long rs[4];
+    int c = 0;
+    while (c + 1 < job.nch && blockIdx.x >= job.ch[c + 1].tile0) c++;
+    const ScanChannel ch = job.ch[c];
+    const int tid = threadIdx.x;
+    const long long n = ch.n;
+    const long long base = (long long)(blockIdx.x - ch.tile0) * kScanTile + (long long)tid * kScanItems;
+    const int rsi = (job.rowstat != nullptr && c == job.rs_ch[0]) ? 0 : ((job.rowstat != nullptr && c == job.rs_ch[1]) ? 1 : -1);
+    if (tid < 4) rs[tid] = 0;
+    long long v[kScanItems];
+    long long sum = 0;
+    if (ch.kind == 0) {
+        const long long *in = static_cast<const long long *>(ch.in);
+#pragma unroll
+        for (int e = 0; e < kScanItems; e++) { const long long i = base + e; v[e] = i < n ? in[i] : 0; sum += v[e]; }
+    } else {
+        const int *in = static_cast<const int *>(ch.in);
+#pragma unroll
+        for (int e = 0; e < kScanItems; e++) { const long long i = base + e; v[e] = (i < n && in[i + 1] > in[i]) ? 1 : 0; sum += v[e]; }
+    }
+    sh[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanBlock; off <<= 1) {
+        long long t = (tid >= off) ? sh[tid - off] : 0;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    long long run = sh[tid] - sum;
+    if (ch.kind == 0) {
+        long long *out = static_cast<long long *>(ch.out);
+#pragma unroll
+        for (int e = 0; e < kScanItems; e++) { const long long i = base + e; if (i <= n) out[i] = run; run += v[e]; }
+    } else {
+        int *out = static_cast<int *>(ch.out);
+#pragma unroll
+        for (int e = 0; e < kScanItems; e++) { const long long i = base + e; if (i <= n) out[i] = (int)run; run += v[e]; }
+    }
+    if (tid == kScanBlock - 1) tilesum[blockIdx.x] = sh[tid];
+    if (rsi >= 0) {                                   // uniform over the workgroup
+        unsigned long long r0 = 0, r1 = 0, r2 = 0, r3 = 0;
+#pragma unroll
+        for (int e = 0; e < kScanItems; e++) {
+            const long long i = base + e;
+            if (i < n && v[e] > 0) {
+                const unsigned long long np = (unsigned long long)(job.offx[i + 1] - job.offx[i]);
+                r0 += 1; r1 += np; r2 += (np + 127) / 128; r3 += (np + 159) / 160;
+            }
+        }
+        if (r0) { atomicAdd(&rs[0], r0); atomicAdd(&rs[1], r1); atomicAdd(&rs[2], r2); atomicAdd(&rs[3], r3); }
+        __syncthreads();
+        if (tid < 4 && rs[tid]) atomicAdd(&job.rowstat[4 * rsi + tid], rs[tid]);
+    }
+}
+
+// tile sums of every channel -> their exclusive prefixes, in place; one workgroup per channel
+__global__ void __launch_bounds__(kScanBlock) multi_scan_sums_kernel(ScanJob job, long long *__restrict__ tilesum)
+{
+    __shared__ long long sh[kScanBlock];
+    const ScanChannel ch = job.ch[blockIdx.x];
+    const int tid = threadIdx.x;
+    long long *ts = tilesum + ch.tile0;
+    long long v[kScanItems];
+    long long sum = 0;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        const unsigned i = (unsigned)tid * kScanItems + e;
+        v[e] = i < ch.ntiles ? ts[i] : 0;
+        sum += v[e];
+    }
+    sh[tid] = sum;
+    __syncthreads();
+    for (int off = 1; off < kScanBlock; off <<= 1) {
+        long long t = (tid >= off) ? sh[tid - off] : 0;
+        __syncthreads();
+        sh[tid] += t;
+        __syncthreads();
+    }
+    long long run = sh[tid] - sum;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++) {
+        const unsigned i = (unsigned)tid * kScanItems + e;
+        if (i < ch.ntiles) ts[i] = run;
+        run += v[e];
+    }
+}
+
+__global__ void __launch_bounds__(kScanBlock) multi_scan_add_kernel(ScanJob job, const long long *__restrict__ tilesum)
+{
+    int c = 0;
+    while (c + 1 < job.nch && blockIdx.x >= job.ch[c + 1].tile0) c++;
+    const ScanChannel ch = job.ch[c];
+    if (ch.ntiles == 1) return;                       // nothing to add
+    const long long add = tilesum[blockIdx.x];
+    long long i = (long long)(blockIdx.x - ch.tile0) * kScanTile + threadIdx.x;
+#pragma unroll
+    for (int e = 0; e < kScanItems; e++, i += kScanBlock)
+        if (i <= ch.n) {
+            if (ch.kind == 0) static_cast<long long *>(ch.out)[i] += add;
+            else static_cast<int *>(ch.out)[i] += (int)add;
+        }
+}
+
+// queues the scans of a job; false (nothing queued) if a channel has more tiles than one workgroup can scan
+static bool multi_scan(const ScanJob &job, hipStream_t s)
+{
+    if (job.nch == 0) return true;
+    unsigned most = 0;
+    for (int c = 0; c < job.nch; c++) most = std::max(most, job.ch[c].ntiles);
+    if (most > (unsigned)kScanTile) return false;
+    if (const char *e = getenv("F3M_LEVEL_SCANS"))      // F3M_LEVEL_SCANS=separate: the path of levels too large for this one (testing aid)
+        if (!strcmp(e, "separate")) return false;
+    DBuf<long long> tilesum((size_t)job.blocks);
+    F3M_LAUNCH(multi_scan_tile_kernel, job.blocks, kScanBlock, 0, s, job, tilesum.get());
+    check_launch("multi_scan_tile");
+    if (most > 1) {
+        F3M_LAUNCH(multi_scan_sums_kernel, job.nch, kScanBlock, 0, s, job, tilesum.get());
+        check_launch("multi_scan_sums");
+        F3M_LAUNCH(multi_scan_add_kernel, job.blocks, kScanBlock, 0, s, job, (const long long *)tilesum.get());
+        check_launch("multi_scan_add");
+    }
+    return true;
+}
+
 // ------------------------------------------------------------------------------------------------
 // bounding box (F3M_src/n_tree.cu:28-31,42-43: per-dimension min and max)
 
@@ -558,21 +716,29 @@ void gather_tree_points(Tree &t, const float *X, hipStream_t s, bool background)
 // One division (F3M_src/n_tree.cu:98-179).  Candidates are the 2^d children of every box, natural
 // index = parent*2^d + child; their point ranges are found by binary search in the sorted keys.
 
-__global__ void child_bounds_kernel(const uint32_t *__restrict__ keys, const uint32_t *__restrict__ prefix_prev,
-                                    const int *__restrict__ off_prev, long long ncand, int d, int shift, long long n,
-                                    int *__restrict__ natpos)
+// (a device function with its workgroup index as an argument: the level loop launches it together with the list
+// builder's counting pass in one grid)
+struct BoundsArgs {
+    const uint32_t *keys, *prefix_prev;
+    const int *off_prev;
+    long long ncand, n;
+    int d, shift;
+    int *natpos;
+    unsigned grid;              // workgroups of 256 threads (0: nothing to do)
+};
+__device__ inline void child_bounds_body(unsigned blk, const BoundsArgs &a)
 {
-    long long nat = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (nat > ncand) return;
-    if (nat == ncand) { natpos[nat] = (int)n; return; }
-    int q = (int)(nat >> d);
-    uint32_t target = (prefix_prev[q] << d) | (uint32_t)(nat & ((1 << d) - 1));
-    int lo = off_prev[q], hi = off_prev[q + 1];
+    long long nat = (long long)blk * 256 + threadIdx.x;
+    if (nat > a.ncand) return;
+    if (nat == a.ncand) { a.natpos[nat] = (int)a.n; return; }
+    int q = (int)(nat >> a.d);
+    uint32_t target = (a.prefix_prev[q] << a.d) | (uint32_t)(nat & ((1 << a.d) - 1));
+    int lo = a.off_prev[q], hi = a.off_prev[q + 1];
     while (lo < hi) {
         int mid = lo + ((hi - lo) >> 1);
-        if ((keys[mid] >> shift) < target) lo = mid + 1; else hi = mid;
+        if ((a.keys[mid] >> a.shift) < target) lo = mid + 1; else hi = mid;
     }
-    natpos[nat] = lo;
+    a.natpos[nat] = lo;
 }
 
 // stats[0] = number of non-empty children, stats[1] = largest count
@@ -654,7 +820,17 @@ bool divide_will_sort(const Tree &t)
     return t.geo.d * (t.geo.L - k) < t.sorted_from;
 }
 
-void divide_launch(Tree &t, int *dstats, hipStream_t s)
+// The division to the next depth in three steps, so that the level loop can queue the first two together with the
+// list builder's counting pass and scans: divide_prepare sorts further key bits if the depth needs them, allocates
+// the new level and describes the search for the candidates' point ranges; (the ranges are found and the "not empty"
+// flags scanned by the caller's launches;) divide_build queues the kernel that fills the level and appends it.
+struct DividePending {
+    DBuf<int> natpos, cid;
+    TreeLevel cur;
+    long long ncand = 0;
+    bool active = false;
+};
+static BoundsArgs divide_prepare(Tree &t, DividePending &dp, hipStream_t s)
 {
     const int d = t.geo.d;
     const int k = (int)t.lev.size();   // depth being built
@@ -667,15 +843,13 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
         radix_sort(t.keys, t.perm, t.n, t.sorted_from, d * t.geo.L, s);
     }
     TreeLevel &prev = t.lev[k - 1];
-    long long ncand = (long long)prev.nb << d;
+    const long long ncand = (long long)prev.nb << d;
     F3M_REQUIRE(ncand < (1ll << 31) - 2, 20, "too many candidate boxes at depth %d (%lld)", k, ncand);
-    DBuf<int> natpos((size_t)ncand + 1), cid((size_t)ncand + 1);
-    F3M_LAUNCH(child_bounds_kernel, cdiv(ncand + 1, 256), 256, 0, s, t.keys.get(), prev.prefix.get(), prev.off.get(), ncand,
-               d, shift, t.n, natpos.get());
-    check_launch("child_bounds");
-    exclusive_scan_nonempty(natpos.get(), ncand, cid.get(), s);      // compact id = number of non-empty candidates before
+    dp.ncand = ncand;
+    dp.natpos.reset((size_t)ncand + 1);
+    dp.cid.reset((size_t)ncand + 1);
     size_t bound = (size_t)std::min<long long>(ncand, t.n);
-    TreeLevel cur;
+    TreeLevel &cur = dp.cur;
     cur.depth = k;
     cur.off.reset(bound + 1);
     cur.prefix.reset(bound);
@@ -684,8 +858,21 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     cur.cellpack.reset(bound);
     cur.parent.reset(bound);
     prev.childstart.reset((size_t)prev.nb + 1);
+    dp.active = true;
+    BoundsArgs a;
+    a.keys = t.keys.get(); a.prefix_prev = prev.prefix.get(); a.off_prev = prev.off.get();
+    a.ncand = ncand; a.n = t.n; a.d = d; a.shift = shift; a.natpos = dp.natpos.get();
+    a.grid = cdiv(ncand + 1, 256);
+    return a;
+}
+static void divide_build(Tree &t, DividePending &dp, int *dstats, hipStream_t s)
+{
+    const int d = t.geo.d;
+    const int k = (int)t.lev.size();
+    TreeLevel &prev = t.lev[k - 1];
+    TreeLevel &cur = dp.cur;
     float quarter = 0.25f * prev.edge;
-    F3M_LAUNCH(build_level_kernel, cdiv(ncand + 1, 256), 256, 0, s, natpos.get(), cid.get(), ncand, d, prev.prefix.get(),
+    F3M_LAUNCH(build_level_kernel, cdiv(dp.ncand + 1, 256), 256, 0, s, dp.natpos.get(), dp.cid.get(), dp.ncand, d, prev.prefix.get(),
                prev.ctr.get(), prev.cell.get(), quarter, cur.off.get(), cur.prefix.get(), cur.ctr.get(), cur.cell.get(),
                cur.cellpack.get(), k, prev.childstart.get(), cur.parent.get(), dstats);
     check_launch("build_level");
@@ -693,6 +880,7 @@ void divide_launch(Tree &t, int *dstats, hipStream_t s)
     cur.maxcount = -1;
     cur.edge = prev.edge * 0.5f;
     t.lev.push_back(std::move(cur));
+    dp.active = false;
 }
 
 void divide_finish(Tree &t, const int *hstats)
@@ -827,8 +1015,8 @@ __device__ inline int classify_pair(const float *__restrict__ cx, const float *_
 constexpr int kListWaves = 4;   // wavefronts per workgroup
 
 template <bool WRITE, int D>
-__global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
-    int nbx, const int *__restrict__ parentx, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
+__device__ inline void lists_body(
+    unsigned blk, int nbx, const int *__restrict__ parentx, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
     const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
     const float *__restrict__ ctrx, const float *__restrict__ ctry, ClassifyParams cp,
     const uint32_t *__restrict__ cellx, const uint32_t *__restrict__ celly, int depth, bool one_tree,
@@ -839,7 +1027,7 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
     int *__restrict__ rp_far, int *__restrict__ rp_keep)
 {
     const int lane = threadIdx.x & 63;
-    const int bx = blockIdx.x * kListWaves + (threadIdx.x >> 6);
+    const int bx = (int)blk * kListWaves + (threadIdx.x >> 6);
     if (bx > nbx) return;
     const long long stride = (long long)nbx + 1;
     if (bx == nbx) {                               // the closing entry of the row pointers
@@ -918,6 +1106,49 @@ __global__ void __launch_bounds__(kListWaves * 64) lists_kernel(
         }
     }
     if (!WRITE && lane == 0) { cnt[bx] = c0; cnt[stride + bx] = c1; cnt[2 * stride + bx] = c2; }
+}
+
+// the writing pass on its own
+template <int D>
+__global__ void __launch_bounds__(kListWaves * 64) lists_write_kernel(
+    int nbx, const int *__restrict__ parentx, const int *__restrict__ csy, const int *__restrict__ keep_pairs,
+    const int *__restrict__ keep_rowptr, const int *__restrict__ offx, const int *__restrict__ offy,
+    const float *__restrict__ ctrx, const float *__restrict__ ctry, ClassifyParams cp, int depth, bool one_tree,
+    const long long *__restrict__ pos, int *__restrict__ out_small, int *__restrict__ out_far, int *__restrict__ out_keep,
+    int *__restrict__ rp_small, int *__restrict__ rp_far, int *__restrict__ rp_keep)
+{
+    lists_body<true, D>(blockIdx.x, nbx, parentx, csy, keep_pairs, keep_rowptr, offx, offy, ctrx, ctry, cp, nullptr, nullptr, depth,
+                        one_tree, nullptr, nullptr, nullptr, pos, out_small, out_far, out_keep, rp_small, rp_far, rp_keep);
+}
+
+// One launch for the two independent things a step of the level loop starts with: the counting pass of the lists of
+// depth k (workgroups [0, la.grid)) and the point ranges of the candidate boxes of depth k+1, for one tree or two
+// (workgroups after that).  Either part may be absent (grid 0).
+struct ListsCountArgs {
+    int nbx;
+    const int *parentx, *csy, *keep_pairs, *keep_rowptr, *offx, *offy;
+    const float *ctrx, *ctry;
+    ClassifyParams cp;
+    const uint32_t *cellx, *celly;
+    int depth;
+    bool one_tree;
+    unsigned long long *outliers, *beyond;
+    long long *cnt;
+    unsigned grid;
+};
+template <int D>
+__global__ void __launch_bounds__(kListWaves * 64) level_count_kernel(ListsCountArgs la, BoundsArgs b0, BoundsArgs b1)
+{
+    unsigned blk = blockIdx.x;
+    if (blk < la.grid) {
+        lists_body<false, D>(blk, la.nbx, la.parentx, la.csy, la.keep_pairs, la.keep_rowptr, la.offx, la.offy, la.ctrx, la.ctry,
+                             la.cp, la.cellx, la.celly, la.depth, la.one_tree, la.outliers, la.beyond, la.cnt, nullptr, nullptr,
+                             nullptr, nullptr, nullptr, nullptr, nullptr);
+        return;
+    }
+    blk -= la.grid;
+    if (blk < b0.grid) { child_bounds_body(blk, b0); return; }
+    child_bounds_body(blk - b0.grid, b1);
 }
 
 // Row statistics of the small and the keep list of a level from the per-box counts of the list builder's counting
@@ -1028,33 +1259,51 @@ void transpose_list(const PairList &in, const TreeLevel &ly, PairList &out, hipS
     out.rows = (long long)h[0], out.row_points = (long long)h[1], out.items128 = (long long)h[2], out.items160 = (long long)h[3];
 }
 
-void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int k, ClassifyParams &cp,
-                  ListsPending &pend, long long *dtot, long long *drow, hipStream_t s)
+void level_launch(const PairList *keep_prev, Tree &tx, Tree &ty, int k, ClassifyParams &cp, ListsPending &pend,
+                  long long *dtot, long long *drow, bool divide, int *dstats_x, int *dstats_y, hipStream_t s)
 {
     const int d = tx.geo.d;
-    const TreeLevel &py = ty.lev[k - 1];
-    const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
-    pend.active = false;
-    if (keep_prev.n == 0) return;
-    F3M_REQUIRE(keep_prev.n < (1ll << 31) - 2, 21, "keep list too long (%lld)", keep_prev.n);
-    F3M_REQUIRE((1 << d) < (1 << 21), 21, "too many children per box");
-    pend.active = true;
     const bool one_tree = &tx == &ty;
-    const int nbx = lx.nb;
-    pend.stride = (long long)nbx + 1;
-    DBuf<long long> cnt((size_t)(3 * pend.stride));
-    pend.pos.reset((size_t)(3 * pend.stride));
-    for (int j = 0; j < kMaxD; j++) cp.omin[j] = j < d ? m2l_table_omin(tx.geo.origin[j], ty.geo.origin[j], lx.edge) : 0;
-    const uint32_t *cellx = lx.cellpack.get();
-    unsigned long long *outl = reinterpret_cast<unsigned long long *>(dtot + 3);
-    unsigned long long *beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
-    pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
+    pend.active = false;
+    const bool lists = keep_prev != nullptr && keep_prev->n > 0;
+    // the counting pass of the lists of depth k
+    ListsCountArgs la;
+    memset(&la, 0, sizeof(la));
+    DBuf<long long> cnt;
+    if (lists) {
+        const TreeLevel &py = ty.lev[k - 1];
+        const TreeLevel &lx = tx.lev[k], &ly = ty.lev[k];
+        F3M_REQUIRE(keep_prev->n < (1ll << 31) - 2, 21, "keep list too long (%lld)", keep_prev->n);
+        F3M_REQUIRE((1 << d) < (1 << 21), 21, "too many children per box");
+        pend.active = true;
+        const int nbx = lx.nb;
+        pend.stride = (long long)nbx + 1;
+        cnt.reset((size_t)(3 * pend.stride));
+        pend.pos.reset((size_t)(3 * pend.stride));
+        for (int j = 0; j < kMaxD; j++) cp.omin[j] = j < d ? m2l_table_omin(tx.geo.origin[j], ty.geo.origin[j], lx.edge) : 0;
+        pend.grid = (unsigned)cdiv((long long)nbx + 1, kListWaves);
+        la.nbx = nbx; la.parentx = lx.parent.get(); la.csy = py.childstart.get();
+        la.keep_pairs = keep_prev->pairs.get(); la.keep_rowptr = keep_prev->rowptr.get();
+        la.offx = lx.off.get(); la.offy = ly.off.get(); la.ctrx = lx.ctr.get(); la.ctry = ly.ctr.get();
+        la.cp = cp; la.cellx = lx.cellpack.get(); la.celly = ly.cellpack.get(); la.depth = k; la.one_tree = one_tree;
+        la.outliers = reinterpret_cast<unsigned long long *>(dtot + 3);
+        la.beyond = reinterpret_cast<unsigned long long *>(dtot + 6);
+        la.cnt = cnt.get();
+        la.grid = pend.grid;
+    }
+    // the division to depth k+1 (the lists above read depth k and k-1 only; the new level is appended at the end)
+    DividePending dx, dy;
+    BoundsArgs bx, by;
+    memset(&bx, 0, sizeof(bx));
+    memset(&by, 0, sizeof(by));
+    if (divide) {
+        bx = divide_prepare(tx, dx, s);
+        if (!one_tree) by = divide_prepare(ty, dy, s);
+    }
+    if (la.grid + bx.grid + by.grid == 0) return;
 #define F3M_CASE(DD)                                                                                                          \
     case DD:                                                                                                                  \
-        F3M_LAUNCH((lists_kernel<false, DD>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),    \
-                   keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), cp, \
-                   cellx, ly.cellpack.get(), k, one_tree, outl, beyond, cnt.get(), (const long long *)nullptr, (int *)nullptr, \
-                   (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr, (int *)nullptr);                            \
+        F3M_LAUNCH((level_count_kernel<DD>), la.grid + bx.grid + by.grid, kListWaves * 64, 0, s, la, bx, by);                 \
         break;
     switch (d) {
         F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -1062,12 +1311,40 @@ void lists_launch(const PairList &keep_prev, const Tree &tx, const Tree &ty, int
     default: throw Error(2, "dimension must be 1..10");
     }
 #undef F3M_CASE
-    check_launch("lists_count");
-    exclusive_scan_i64_batched(cnt.get(), nbx, pend.stride, 3, pend.pos.get(), s);
-    if (drow != nullptr) {
-        F3M_LAUNCH(list_rowstats_kernel, cdiv(nbx, kRowStatBlock), kRowStatBlock, 0, s, cnt.get(), pend.stride, lx.off.get(), nbx,
-                   reinterpret_cast<unsigned long long *>(drow));
-        check_launch("list_rowstats");
+    check_launch("level_count");
+    // the scans of both, and the row statistics of the small and the keep list, in one set of launches
+    ScanJob job;
+    if (lists) {
+        for (int c = 0; c < 3; c++) job.add(cnt.get() + c * pend.stride, pend.pos.get() + c * pend.stride, la.nbx, 0);
+        if (drow != nullptr) {
+            job.offx = la.offx;
+            job.rowstat = reinterpret_cast<unsigned long long *>(drow);
+            job.rs_ch[0] = 0;
+            job.rs_ch[1] = 2;
+        }
+    }
+    if (divide) {
+        job.add(dx.natpos.get(), dx.cid.get(), dx.ncand, 1);     // compact id = number of non-empty candidates before
+        if (!one_tree) job.add(dy.natpos.get(), dy.cid.get(), dy.ncand, 1);
+    }
+    if (!multi_scan(job, s)) {
+        // a level too large for the joint scans (more than kScanTile tiles per array): one scan after the other
+        if (lists) {
+            exclusive_scan_i64_batched(cnt.get(), la.nbx, pend.stride, 3, pend.pos.get(), s);
+            if (drow != nullptr) {
+                F3M_LAUNCH(list_rowstats_kernel, cdiv(la.nbx, kRowStatBlock), kRowStatBlock, 0, s, cnt.get(), pend.stride, la.offx,
+                           la.nbx, reinterpret_cast<unsigned long long *>(drow));
+                check_launch("list_rowstats");
+            }
+        }
+        if (divide) {
+            exclusive_scan_nonempty(dx.natpos.get(), dx.ncand, dx.cid.get(), s);
+            if (!one_tree) exclusive_scan_nonempty(dy.natpos.get(), dy.ncand, dy.cid.get(), s);
+        }
+    }
+    if (divide) {
+        divide_build(tx, dx, dstats_x, s);
+        if (!one_tree) divide_build(ty, dy, dstats_y, s);
     }
 }
 
@@ -1086,13 +1363,11 @@ static void lists_write(ListsPending &pend, const long long *cap, const PairList
     out.small_.rowptr.reset((size_t)pend.stride);
     out.far.rowptr.reset((size_t)pend.stride);
     out.keep.rowptr.reset((size_t)pend.stride);
-    const uint32_t *cellx = lx.cellpack.get();
 #define F3M_CASE(DD)                                                                                                          \
     case DD:                                                                                                                  \
-        F3M_LAUNCH((lists_kernel<true, DD>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),     \
+        F3M_LAUNCH((lists_write_kernel<DD>), pend.grid, kListWaves * 64, 0, s, nbx, lx.parent.get(), py.childstart.get(),     \
                    keep_prev.pairs.get(), keep_prev.rowptr.get(), lx.off.get(), ly.off.get(), lx.ctr.get(), ly.ctr.get(), cp, \
-                   cellx, ly.cellpack.get(), k, one_tree, (unsigned long long *)nullptr, (unsigned long long *)nullptr,        \
-                   (long long *)nullptr, (const long long *)pend.pos.get(), out.small_.pairs.get(), out.far.pairs.get(),       \
+                   k, one_tree, (const long long *)pend.pos.get(), out.small_.pairs.get(), out.far.pairs.get(),               \
                    out.keep.pairs.get(), out.small_.rowptr.get(), out.far.rowptr.get(), out.keep.rowptr.get());                \
         break;
     switch (d) {

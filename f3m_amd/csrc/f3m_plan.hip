@@ -312,10 +312,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
         return (float)P->tx.lev.back().maxcount > prm->min_points &&
                (sym || (float)P->ty_.lev.back().maxcount > prm->min_points) && (int)P->tx.lev.size() <= gx.L;
     };
-    auto start_division = [&]() {
-        divide_launch(P->tx, dres.get() + 8, s);
-        if (!sym) divide_launch(P->ty_, dres.get() + 10, s);
-    };
     auto finish_division = [&]() {
         divide_finish(P->tx, hres + 8);
         if (!sym) divide_finish(P->ty_, hres + 10);
@@ -323,7 +319,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     // The points (and the weights of a one-shot product) are moved into sorted order on the second stream while the
     // levels and lists are built here: those are many small kernels that leave the memory system idle, the moves are
     // bound by it.  The order of the first sort is final unless a deep level asks for more key bits to be sorted
-    // (divide_launch); then the moves wait for that and are done again at the end.
+    // (level_launch); then the moves wait for that and are done again at the end.
     bool early = false;
     // While work is queued on both streams, blocks that host code gives back are parked (a kernel of the other stream
     // may still use them, and the pool would hand them to the next request); they return to the pool at the end.
@@ -361,7 +357,11 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
     };
     if (need_tree && wants_division()) {
         settle_early();
-        start_division();
+        {
+            ClassifyParams none = classify_params(*P, 0.f);
+            ListsPending nopend;
+            level_launch(nullptr, P->tx, *P->ty, 0, none, nopend, nullptr, nullptr, true, dres.get() + 8, dres.get() + 10, s);
+        }
         // with the first division's counts, the fullest cell at the depth that the sorted key bits resolve
         // (words [14], [15] of the record)
         if (two_streams) {
@@ -387,10 +387,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             ClassifyParams cp = classify_params(*P, e);
             ListsPending pend;
             F3M_REQUIRE((int)P->levels.size() <= kMaxLevels, 23, "tree deeper than %d levels", kMaxLevels);
-            lists_launch(*keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()),
-                         drow.get() + 8 * (P->levels.size() - 1), s);
             const bool ahead = wants_division();
-            if (ahead) { settle_early(); start_division(); }
+            if (ahead) settle_early();
+            level_launch(keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()),
+                         drow.get() + 8 * (P->levels.size() - 1), ahead, dres.get() + 8, dres.get() + 10, s);
             // No further division: this is the deepest level, whose near lists will be summed.  Its source operands
             // are prepared on the second stream (behind the moves of the points) while its lists are built here.
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)

@@ -82,10 +82,9 @@ int f3m_plan_destroy(f3m_plan *plan);
  * run once before (otherwise error 41).  All calls on a GPU share the one scratch array: calls that overlap
  * on one GPU race, also from different plans or threads.  The call waits for the stream like the others,
  * except while the stream is being captured.  A captured call holds the addresses of the plan's tables: its
- * graph may be replayed only while the plan lives and no other entry point has rebuilt those tables in the
- * meantime (f3m_plan_near_level on a list the products do not sum, a product with another number of columns,
- * a change of the library's F3M_* environment switches); an error raised during capture leaves the capture
- * to the caller (the library then waits for nothing). */
+ * graph may be replayed while the plan lives (a table of a plan is built once and never replaced; destroying the
+ * plan frees them); an error raised during capture leaves the capture to the caller (the library then waits
+ * for nothing). */
 int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream);
 
 /* Introspection for parity tests (no counterpart is exported by the reference; the data are its

@@ -51,6 +51,16 @@ def test_tree_and_lists_bit_exact(oracle, name):
     assert w[0] == ora.work_near_pairs and w[1] == ora.work_far_pairs and w[2] == ora.work_interp_pts
 
 
+def test_level_scans_one_by_one(oracle, monkeypatch):
+    """The level loop scans its list counts and its "candidate box is not empty" flags in one set of launches; levels
+    with more than 2048 x 2048 boxes take the scans one after the other.  F3M_LEVEL_SCANS=separate forces that path:
+    same tree, same lists."""
+    monkeypatch.setenv("F3M_LEVEL_SCANS", "separate")
+    for name in ("uniform3", "asym3"):
+        X, Y = _cloud(name, np.random.default_rng(21))
+        assert_plan_matches_oracle(ee.Plan(X, Y, **PRM), oracle.Plan(X, Y, **PRM))
+
+
 def test_deep_tree_bit_exact(oracle):
     """A tight cluster inside a sparse cloud forces divisions down to the depth cap; the engine sorts
     further key bits only when a division needs them."""

@@ -188,6 +188,20 @@ def test_box_division_and_lists_bit_exact(eng, oracle, name):
     assert w["near_pairs"] + w["far_point_pairs"] == float(X.shape[0]) * M      # every pair exactly once
 
 
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4"])
+def test_level_scans_one_by_one(eng, oracle, monkeypatch, name):
+    """F3M_LEVEL_SCANS=separate: the scans of a level one after the other (the path of levels with more than
+    2048 x 2048 boxes) instead of in one set of launches: same tree and lists, and the same row statistics."""
+    print("case separate level scans", name, flush=True)
+    monkeypatch.setenv("F3M_LEVEL_SCANS", "separate")
+    X, Y, prm = clouds(name, np.random.default_rng(11))
+    plan = eng.Plan(dev(X), None if Y is None else dev(Y), **prm)
+    ora = oracle.Plan(X, Y, **prm)
+    assert_plan_matches_oracle(plan, ora)
+    for k in range(1, plan.depth + 1):
+        assert plan.list_rows(k) == expected_list_rows(ora.level(k - 1)), k
+
+
 @pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform5"])
 def test_box_lookup_by_cell(eng, oracle, name):
     """The HBM key -> index table (reference: F3M_src/linearprobing.cu:18-87): the cell of every point,
