@@ -34,6 +34,7 @@ struct TreeLevel {
     // Two tables, each built at most once and never replaced (a launch recorded into a graph keeps its address):
     // nearops_all holds every box, nearops only the source boxes of the level's one near list.
     mutable DBuf<unsigned char> nearops, nearops_all;
+    mutable DBuf<float> nearey, nearey_all;   // factored form only: exp2(-|y'|^2) per point, beside the table of the same slot
     mutable float nearops_sc = 0.f;
     // grid key -> box id table of this level (built on first use by lookup_boxes)
     // box of every 32nd point (npoints/32 + 2 entries, built on first use by box_table): kernels that

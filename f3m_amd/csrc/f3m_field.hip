@@ -414,9 +414,18 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 // slots 3D, 3D+1 = (hi, lo of the source's -|y'|^2) . 1 and slots 3D+2, 3D+3 = 1 . (hi, lo of the
 // target's -|x''|^2).  3D+4 slots in all: one instruction of 16 up to D = 4.
 // hi/lo hold C = D+2 values: the coordinates, then on the source side (-|y'|^2, 1), on the target side (1, -|x''|^2).
-__host__ __device__ constexpr int near_slots(int D) { return 3 * D + 4; }
-__host__ __device__ constexpr int near_insts(int D) { return (near_slots(D) + 15) / 16; }
-template <int D>
+//
+// Factored form (FACT): only the coordinates go through the matrix product, u = 2x''.y' in 3D slots, and
+//   exp2(t) b = exp2(-|x''|^2) . exp2(u) . (exp2(-|y'|^2) b):
+// the source factor rides on the weight (one multiplication per source and product, near_weights_kernel), the target
+// factor multiplies the sum over a run of sources once.  It takes one instruction where 3D+4 slots take two
+// (D = 5: 15 against 19 slots), at the price of exponentials whose arguments no longer cancel: |u| <= 10 D S^2 with
+// S = (box edge) sqrt(lcs log2 e), so the host takes the form only while that stays far from the exponent range.
+__host__ __device__ constexpr int near_slots(int D, bool fact = false) { return fact ? 3 * D : 3 * D + 4; }
+__host__ __device__ constexpr int near_insts(int D, bool fact = false) { return (near_slots(D, fact) + 15) / 16; }
+// dimensions whose factored form saves an instruction (the others never take it)
+__host__ __device__ constexpr bool near_fact_pays(int D) { return near_insts(D, true) < near_insts(D, false); }
+template <int D, bool FACT = false>
 __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, int hh, bool source)
 {
     h8 v;
@@ -426,7 +435,7 @@ __device__ inline h8 split_operand(const half_t *hi, const half_t *lo, int n, in
         if (slot < 3 * D) {
             const int c = slot / 3, tau = slot % 3;
             v[e] = source ? (tau == 2 ? lo[c] : hi[c]) : (tau == 1 ? lo[c] : hi[c]);
-        } else if (slot < near_slots(D)) {
+        } else if (slot < near_slots(D, FACT)) {
             const int sl = slot - 3 * D;
             if (source) v[e] = sl == 0 ? hi[D] : (sl == 1 ? lo[D] : hi[D + 1]);
             else v[e] = sl < 2 ? hi[D] : (sl == 2 ? hi[D + 1] : lo[D + 1]);
@@ -454,16 +463,17 @@ __device__ __forceinline__ float near_anchor(const Geo &geo, float edge, int cel
     return geo.origin[k] + (float)(2 * (cell >> 1) + 1) * edge;
 }
 
-template <int D>
+// FACT: the operands of the factored form, and ey[i] = exp2(-|y'_i|^2) (stride floats, zero past the end).
+template <int D, bool FACT>
 __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *__restrict__ ys, long long M,
                                                                   const int *__restrict__ off, int nb,
                                                                   const int *__restrict__ cell, Geo geo, float edge,
                                                                   float sc, long long stride,
                                                                   const int *__restrict__ need, const int *__restrict__ box32,
-                                                                  h8 *__restrict__ ops)
+                                                                  h8 *__restrict__ ops, float *__restrict__ ey)
 {
     constexpr int C = D + 2;                        // coordinates, -|y'|^2, and a 1 that carries the target's -|x''|^2
-    constexpr int NS = near_insts(D);
+    constexpr int NS = near_insts(D, FACT);
     __shared__ int bounds[kOpsBlock];
     const int tid = threadIdx.x;
     const long long i0 = (long long)blockIdx.x * kOpsBlock, i = i0 + tid;
@@ -484,6 +494,7 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
     __syncthreads();
     if (i >= stride) return;
     half_t hi[C], lo[C];
+    float ny2 = 0.f;
     if (i < M) {
         auto box_of = [&](long long p) {            // p >= i0: number of box starts <= p among the following boxes
             int a = 0, b = kOpsBlock;
@@ -498,7 +509,6 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
             const int first = (i - 31 >= i0) ? box_of(i - 31) : b0m;
             if (need[box + 1] - need[first] == 0) return;
         }
-        float ny2 = 0.f;
 #pragma unroll
         for (int k = 0; k < C; k++) {
             float v;
@@ -520,9 +530,21 @@ __global__ void __launch_bounds__(kOpsBlock) near_operands_kernel(const float *_
     }
 #pragma unroll
     for (int n = 0; n < NS; n++) {
-        ops[(long long)(n * 2 + 0) * stride + i] = split_operand<D>(hi, lo, n, 0, true);
-        ops[(long long)(n * 2 + 1) * stride + i] = split_operand<D>(hi, lo, n, 1, true);
+        ops[(long long)(n * 2 + 0) * stride + i] = split_operand<D, FACT>(hi, lo, n, 0, true);
+        ops[(long long)(n * 2 + 1) * stride + i] = split_operand<D, FACT>(hi, lo, n, 1, true);
     }
+    if (FACT) ey[i] = i < M ? fast_exp2(ny2) : 0.f;
+}
+
+// weights of the factored form: ws[c][j] = bs[c][j] exp2(-|y'_j|^2), the padding tile included; columns of bs are
+// bstride apart, those of ws stride
+__global__ void near_weights_kernel(const float *__restrict__ bs, const float *__restrict__ ey, long long stride, int nc,
+                                    long long bstride, float *__restrict__ ws)
+{
+    const long long j = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= stride) return;
+    const float e = ey[j];
+    for (int c = 0; c < nc; c++) ws[c * stride + j] = bs[c * bstride + j] * e;
 }
 
 // Near field, matrix-pipe form.  One wavefront per TPW*32 targets of an x box (TPW tiles of 32; lanes
@@ -549,7 +571,8 @@ struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floa
 
 // NC right-hand sides at once: the exponential of a pair is computed once and multiplies NC weights
 // (columns of bs, bstride apart; results to NC columns of outs, ostride apart).
-template <int D, int TPW, int NC>
+// FACT: the factored form (see near_slots): bs then holds the weights times exp2(-|y'|^2).
+template <int D, int TPW, int NC, bool FACT = false>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 && NC == 1) ? 5 : 2) near_g_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
@@ -558,7 +581,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
-    constexpr int NS = near_insts(D);
+    constexpr int NS = near_insts(D, FACT);
     const int lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31;
     // Workgroups are handed to the 8 XCDs round-robin.  Work items are in Morton order of their x box
     // and neighbouring boxes share their source boxes, so the work items are cut into stripes of
@@ -660,6 +683,13 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
         for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
         // target operands relative to the anchor of this run
         h8 bop[TPW][NS];
+        float ex[TPW], run[TPW][NC];                  // factored form: exp2(-|x''|^2) and the sums of this run
+#pragma unroll
+        for (int q = 0; q < TPW; q++) {
+            ex[q] = 0.f;
+#pragma unroll
+            for (int c = 0; c < NC; c++) run[q][c] = 0.f;
+        }
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
             if (q >= nlive) continue;                 // uniform per wavefront: tiles without targets need no operands
@@ -680,9 +710,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             }
 #pragma unroll
             for (int n = 0; n < NS; n++) {
-                h8 v0 = split_operand<D>(hi, lo, n, 0, false), v1 = split_operand<D>(hi, lo, n, 1, false);
+                h8 v0 = split_operand<D, FACT>(hi, lo, n, 0, false), v1 = split_operand<D, FACT>(hi, lo, n, 1, false);
                 bop[q][n] = half ? v1 : v0;
             }
+            if (FACT) ex[q] = fast_exp2(nx2);
         }
         for (int j0 = s0; j0 < s1; j0 += 32) {
             h8 a[NS];
@@ -716,7 +747,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                 for (int r = 0; r < 16; r++) {
                     const float e = fast_exp2(t[r]);
 #pragma unroll
-                    for (int c = 0; c < NC; c++) acc[q][c] = fmaf(e, bq[c][r], acc[q][c]);
+                    for (int c = 0; c < NC; c++) {
+                        if (FACT) run[q][c] = fmaf(e, bq[c][r], run[q][c]);
+                        else acc[q][c] = fmaf(e, bq[c][r], acc[q][c]);
+                    }
                 }
             };
             if (nlive == TPW) {
@@ -729,6 +763,12 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                 for (int q = 0; q < TPW; q++)
                     if (q < nlive) tile(q);              // uniform per wavefront
             }
+        }
+        if (FACT) {
+#pragma unroll
+            for (int q = 0; q < TPW; q++)
+#pragma unroll
+                for (int c = 0; c < NC; c++) acc[q][c] = fmaf(run[q][c], ex[q], acc[q][c]);
         }
       }
     }
@@ -785,21 +825,44 @@ static bool near_on_matrix_pipe(int d, float lcs, float edge)
     return use_mfma;
 }
 
+// whether the near field of a level takes the factored form (see near_slots): only where it saves a matrix
+// instruction, and while the exponent 2x''.y' (at most 10 d S^2, targets within five edges of the anchor and sources
+// within one) stays below 60.  F3M_NEAR_FACT=0|1 overrides (1: wherever the form saves an instruction).
+static bool near_factored(int d, float lcs, float edge)
+{
+    const bool pays = d == 5 || d == 10;             // near_fact_pays(d)
+    const float S = sqrtf(lcs * kLog2e) * edge;
+    bool fact = pays && 10.f * (float)d * S * S <= 60.f;
+    if (const char *env = getenv("F3M_NEAR_FACT")) fact = pays && atoi(env) != 0;
+    return fact;
+}
+
+struct NearOps {
+    const h8 *ops;
+    const float *ey;       // factored form only
+};
+
 // The split-f16 source operands of a level, kept with it.  only (nullable): operands are needed for the source boxes
 // of this list alone (at most levels a small part of the boxes); otherwise for every box.
 // Returns the table to use: the one of every box if it exists, else (for a list that is the level's only one) the table
 // of that list's source boxes; whichever is missing is built, none is ever rebuilt.
-static const h8 *build_near_operands(int d, const Tree &ty, const TreeLevel &ly, float sc, const PairList *only, hipStream_t s)
+static NearOps build_near_operands(int d, const Tree &ty, const TreeLevel &ly, float sc, bool fact, const PairList *only,
+                                   hipStream_t s)
 {
     const bool only_list = only != nullptr;
     F3M_REQUIRE(ly.nearops_sc == 0.f || ly.nearops_sc == sc, 38, "near-field operands of a level asked for with another lengthscale");
-    if (ly.nearops_all.size() != 0) return reinterpret_cast<const h8 *>(ly.nearops_all.get());
-    if (only_list && ly.nearops.size() != 0) return reinterpret_cast<const h8 *>(ly.nearops.get());
-    const int NS = near_insts(d);
+    if (ly.nearops_all.size() != 0) return NearOps{reinterpret_cast<const h8 *>(ly.nearops_all.get()), ly.nearey_all.get()};
+    if (only_list && ly.nearops.size() != 0) return NearOps{reinterpret_cast<const h8 *>(ly.nearops.get()), ly.nearey.get()};
+    const int NS = near_insts(d, fact);
     const long long stride = ty.n + 32;
     require_tables_may_be_built("the near-field source operands of a level");
     DBuf<unsigned char> &table = only_list ? ly.nearops : ly.nearops_all;
+    DBuf<float> &eytab = only_list ? ly.nearey : ly.nearey_all;
     table.reset((size_t)NS * 2 * stride * 16);
+    if (fact) {
+        eytab.reset((size_t)stride);
+        dev_fill(eytab.get(), 0, sizeof(float) * (size_t)stride, s);     // points that the operands skip keep a zero factor
+    }
     ly.nearops_sc = sc;
     DBuf<int> need;
     if (only_list) {
@@ -813,10 +876,19 @@ static const h8 *build_near_operands(int d, const Tree &ty, const TreeLevel &ly,
     const int *box32 = box_table(ly, ty.n, s);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        F3M_LAUNCH((near_operands_kernel<DD>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,          \
+        if constexpr (near_fact_pays(DD)) {                                                                           \
+            if (fact) {                                                                                               \
+                F3M_LAUNCH((near_operands_kernel<DD, true>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(),  \
+                           ty.n, ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                    \
+                           only_list ? need.get() : (const int *)nullptr, box32,                                      \
+                           reinterpret_cast<h8 *>(table.get()), eytab.get());                                         \
+                break;                                                                                                \
+            }                                                                                                         \
+        }                                                                                                             \
+        F3M_LAUNCH((near_operands_kernel<DD, false>), cdiv(stride, kOpsBlock), kOpsBlock, 0, s, ty.pts.get(), ty.n,   \
                    ly.off.get(), ly.nb, ly.cell.get(), ty.geo, ly.edge, sc, stride,                                  \
                    only_list ? need.get() : (const int *)nullptr, box32,                                              \
-                   reinterpret_cast<h8 *>(table.get()));                                                              \
+                   reinterpret_cast<h8 *>(table.get()), (float *)nullptr);                                            \
         break;
     switch (d) {
         F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -825,7 +897,7 @@ static const h8 *build_near_operands(int d, const Tree &ty, const TreeLevel &ly,
     }
 #undef F3M_CASE
     check_launch("near_operands");
-    return reinterpret_cast<const h8 *>(table.get());
+    return NearOps{reinterpret_cast<const h8 *>(table.get()), fact ? eytab.get() : nullptr};
 }
 
 // The operands of every box of a level, ahead of the near field (the plan calls this for its deepest level, beside
@@ -833,7 +905,7 @@ static const h8 *build_near_operands(int d, const Tree &ty, const TreeLevel &ly,
 void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs, hipStream_t s)
 {
     if (!near_on_matrix_pipe(d, lcs, ly.edge)) return;
-    build_near_operands(d, ty, ly, sqrtf(lcs * kLog2e), nullptr, s);
+    build_near_operands(d, ty, ly, sqrtf(lcs * kLog2e), near_factored(d, lcs, ly.edge), nullptr, s);
 }
 
 // the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
@@ -920,7 +992,9 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     float sc = sqrtf(lcs * kLog2e);
     if (use_mfma) {
         const long long stride = ty.n + 32;
-        const h8 *srcops = build_near_operands(d, ty, ly, sc, only_list ? &list : nullptr, s);
+        // the form of a table is decided when it is built and read off the table afterwards (ey comes with the factored one)
+        const NearOps src = build_near_operands(d, ty, ly, sc, near_factored(d, lcs, ly.edge), only_list ? &list : nullptr, s);
+        const bool fact = src.ey != nullptr;
         if (prepare_only) return;
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
@@ -940,28 +1014,36 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         int nblk = (int)cdiv((long long)ntiles * nsplit, kNearWavesPerBlock);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
+        // weights of the factored form: the sorted weights times exp2(-|y'|^2) of their point (one pass per product)
+        DBuf<float> ws;
+        const float *wsrc = bs;
+        long long wstride = bstride;
+        if (fact) {
+            ws.reset((size_t)stride * nc);
+            wstride = stride;
+            F3M_LAUNCH(near_weights_kernel, cdiv(stride, 256), 256, 0, s, bs, src.ey, stride, nc, bstride, ws.get());
+            check_launch("near_weights");
+            wsrc = ws.get();
+        }
+        auto go = [&](auto kern) {
+            F3M_LAUNCH(kern, ngrid, kNearWavesPerBlock * 64, 0, s, tx.pts.get(), tx.n, src.ops, stride, wsrc, wstride, outs,
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(),
+                       list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);
+        };
+#define F3M_NEAR_FORM(DD, FF)                                                                                         \
+    if (tpw == 5) go(near_g_kernel<DD, 5, 1, FF>);                                                                    \
+    else if (nc == 4) go(near_g_kernel<DD, 4, 4, FF>);                                                                \
+    else if (nc == 2) go(near_g_kernel<DD, 4, 2, FF>);                                                                \
+    else go(near_g_kernel<DD, 4, 1, FF>);
 #define F3M_CASE(DD)                                                                                                  \
     case DD:                                                                                                          \
-        if (tpw == 5)                                                                                                 \
-            F3M_LAUNCH((near_g_kernel<DD, 5, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
-        else if (nc == 4)                                                                                             \
-            F3M_LAUNCH((near_g_kernel<DD, 4, 4>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
-        else if (nc == 2)                                                                                             \
-            F3M_LAUNCH((near_g_kernel<DD, 4, 2>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
-        else                                                                                                          \
-            F3M_LAUNCH((near_g_kernel<DD, 4, 1>), ngrid, kNearWavesPerBlock * 64, 0, s,                               \
-                       tx.pts.get(), tx.n, srcops, stride, bs                                 , bstride, outs, \
-                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(), list.rowptr.get(), \
-                       tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);                                         \
+        if constexpr (near_fact_pays(DD)) {                                                                           \
+            if (fact) {                                                                                               \
+                F3M_NEAR_FORM(DD, true)                                                                               \
+                break;                                                                                                \
+            }                                                                                                         \
+        }                                                                                                             \
+        F3M_NEAR_FORM(DD, false)                                                                                      \
         break;
         switch (d) {
             F3M_CASE(1) F3M_CASE(2) F3M_CASE(3) F3M_CASE(4) F3M_CASE(5)
@@ -969,6 +1051,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         default: throw Error(2, "dimension must be 1..10");
         }
 #undef F3M_CASE
+#undef F3M_NEAR_FORM
         if (nsplit > 1) {
             check_launch("near_g");
             F3M_LAUNCH(near_reduce_kernel, cdiv((long long)ntiles * tpw * 32, 256), 256, 0, s, part.get(), nsplit, nc, ntiles,

@@ -326,6 +326,28 @@ def test_mfma_near_field(oracle, monkeypatch):
                 assert np.array_equal(eng.apply(b[:, col:col + 1]), got[:, col:col + 1])
 
 
+@pytest.mark.parametrize("form", ["0", "1"])
+def test_mfma_near_field_five_dimensions(oracle, monkeypatch, form):
+    """d = 5: two matrix instructions per tile in the plain form, one in the factored form (the weights carry
+    exp2(-|y'|^2), the sum of a run of sources is multiplied by exp2(-|x''|^2)); one and three columns."""
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_NEAR_FACT", form)
+    rng = np.random.default_rng(5)
+    n = 420
+    X = rng.random((n, 5), dtype=f32)
+    Y = (rng.random((n - 100, 5)) * 1.1).astype(f32)
+    prm = dict(ls=0.7, min_points=40, nr_of_interpolation=32, small_field_points=30)
+    ora = oracle.Plan(X, Y, **prm)
+    for nc in (1, 3) if form == "1" else (1,):
+        b = rng.standard_normal((n - 100, nc)).astype(f32)
+        eng = ee.Plan(X, Y, **prm)
+        assert eng.depth == 1 and eng.level_sizes(1)["nsmall"] == 1024
+        if nc == 1:
+            assert rel_l2(eng.near_level(1, "small", b), ora.near_level(0, "small", b)) < 1e-5
+        else:           # the product goes through the four-column kernel
+            assert rel_l2(eng.apply(b), ora.apply(b)) < 1e-5
+
+
 def test_no_division_returns_exact_product(oracle):
     rng = np.random.default_rng(2)
     X = rng.random((200, 3), dtype=f32)

@@ -173,6 +173,50 @@ def test_near_field_kernel_switch_at_its_threshold(eng, oracle, monkeypatch, d, 
         assert np.array_equal(auto, valu)
 
 
+@pytest.mark.parametrize("d,n,boxes", [(5, 200000, [0, 100, 341, 682, 900, 1023]), (10, 120000, [0, 341, 1023])])
+@pytest.mark.parametrize("side", ["below", "above"])
+def test_near_field_factored_form_at_its_threshold(eng, oracle, monkeypatch, d, n, boxes, side):
+    """In 5 and 10 dimensions the matrix-pipe near field takes its factored form (exp2(-|x''|^2) exp2(2x''.y')
+    exp2(-|y'|^2) b, one matrix instruction fewer per tile) while 10 d (sc edge)^2 <= 60, the plain form beyond.
+    Lengthscales 1 % below and above that switch: both forms within 1e-5 of the oracle's sums on both sides, and the
+    library's own choice (fixed when a level's operand table is built, hence one plan per setting) has the bits of the
+    factored form below and of the plain form above."""
+    print("case near factored d=%d %s" % (d, side), flush=True)
+    rng = np.random.default_rng(22)
+    X = rng.random((n, d), dtype=f32)
+    b = rng.standard_normal((n, 2)).astype(f32)
+    prm = dict(min_points=1000, nr_of_interpolation=32 if d == 5 else 64)
+    probe = eng.Plan(dev(X), None, ls=1.0, **prm)
+    depth = probe.depth
+    edge = float(probe.level_sizes(depth)["edge"])
+    probe.close()
+    s_edge = np.sqrt(60.0 / (10.0 * d)) * (0.99 if side == "below" else 1.01)
+    ls = float(np.sqrt(np.log2(np.e) / 2.0) * edge / s_edge)
+    ora = oracle.Plan(X, None, ls=ls, **prm)
+    assert ora.nlevels == depth
+    sc_edge = np.sqrt(float(ora.lcs) * np.log2(np.e)) * edge
+    assert (10 * d * sc_edge ** 2 <= 60) == (side == "below")
+    L = ora.level(depth - 1)
+    which = "small" if len(L["small"]) else "keep"
+    rows = np.concatenate([L["permx"][L["offx"][bx]:L["offx"][bx + 1]] for bx in boxes])
+    want = ora.near_level(depth - 1, which, b, rows=rows)[rows]
+    assert np.abs(want).max() > 0
+    got = {}
+    for form in (None, "0", "1"):
+        if form is None:
+            monkeypatch.delenv("F3M_NEAR_FACT", raising=False)
+        else:
+            monkeypatch.setenv("F3M_NEAR_FACT", form)
+        plan = eng.Plan(dev(X), None, ls=ls, **prm)
+        got[form] = plan.near_level(depth, which, dev(b)).cpu().numpy()[rows]
+        plan.close()
+    e_plain, e_fact = rel_l2(got["0"], want), rel_l2(got["1"], want)
+    print("sc*edge %.4f  rel-L2 vs oracle: plain %.3e, factored %.3e" % (sc_edge, e_plain, e_fact), flush=True)
+    assert e_plain < 1e-5 and e_fact < 1e-5
+    assert not np.array_equal(got["0"], got["1"])
+    assert np.array_equal(got[None], got["1" if side == "below" else "0"])
+
+
 @pytest.mark.parametrize("name", NAMES)
 def test_box_division_and_lists_bit_exact(eng, oracle, name):
     print("case", name, flush=True)
