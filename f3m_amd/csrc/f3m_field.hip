@@ -634,6 +634,16 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
         thi = (int)((long long)ttot * (slice + 1) / nsplit);
     }
     int tcur = 0;                                    // tiles of the row before the current y box
+    h8 bop[TPW][NS];                                 // target operands of the current anchor
+    float ex[TPW];                                   // factored form: exp2(-|x''|^2)
+#pragma unroll
+    for (int q = 0; q < TPW; q++) {
+        ex[q] = 0.f;
+#pragma unroll
+        for (int n = 0; n < NS; n++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) bop[q][n][e] = to_half(0.f);
+    }
     // The list is consumed 64 y boxes at a time: every lane fetches the range and the anchor of one y
     // box, then the wavefront walks through them (one round of memory latency per 64 boxes).  Boxes
     // that follow each other in the list, in memory and under one parent share their anchor and are
@@ -657,15 +667,20 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
           }
       }
       const int mcnt = min(64, m1 - mb);
-      // continues the run of the lane before (sliced lists keep one box per run: slices count tiles per box)
+      // same: under the parent cell of the lane before (same anchor, the target operands stay as they are);
+      // cont: also next to it in memory, i.e. continues its run
+      // (sliced lists keep one box per run: slices count tiles per box)
       const int before = (lane + 63) & 63;
-      bool cont = (wave_shfl_i(byv, before) + 1 == byv);
+      bool same = lane > 0 && mi < m1 && nsplit == 1;
 #pragma unroll
-      for (int k = 0; k < D; k++) cont = (wave_shfl_i(pcv[k], before) == pcv[k]) && cont;
-      cont = cont && lane > 0 && mi < m1 && nsplit == 1;
+      for (int k = 0; k < D; k++) same = (wave_shfl_i(pcv[k], before) == pcv[k]) && same;
+      const int byprev = wave_shfl_i(byv, before);   // by every lane: an exchange inside a branch sees the branch's lanes only
+      const bool cont = same && byprev + 1 == byv;
       unsigned long long heads = wave_ballot(mi < m1 && !cont);
+      const unsigned long long anchors = wave_ballot(mi < m1 && !same);
       while (heads) {
         const int mj = __builtin_ctzll(heads);
+        const bool new_anchor = (anchors >> mj) & 1;   // uniform
         heads &= heads - 1;
         const int mlast = heads ? __builtin_ctzll(heads) - 1 : mcnt - 1;
         int s0 = wave_readlane(s0v, mj), s1 = wave_readlane(s1v, mlast);
@@ -678,18 +693,17 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             tcur += nt;
             if (a >= b) continue;                    // uniform
         }
+        float run[TPW][NC];                           // factored form: the sums of this run
+#pragma unroll
+        for (int q = 0; q < TPW; q++)
+#pragma unroll
+            for (int c = 0; c < NC; c++) run[q][c] = 0.f;
+        // target operands relative to the anchor of this run; runs under one parent cell follow each other in the
+        // list and share them
+        if (new_anchor) {
         float cy[D];
 #pragma unroll
         for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
-        // target operands relative to the anchor of this run
-        h8 bop[TPW][NS];
-        float ex[TPW], run[TPW][NC];                  // factored form: exp2(-|x''|^2) and the sums of this run
-#pragma unroll
-        for (int q = 0; q < TPW; q++) {
-            ex[q] = 0.f;
-#pragma unroll
-            for (int c = 0; c < NC; c++) run[q][c] = 0.f;
-        }
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
             if (q >= nlive) continue;                 // uniform per wavefront: tiles without targets need no operands
@@ -714,6 +728,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                 bop[q][n] = half ? v1 : v0;
             }
             if (FACT) ex[q] = fast_exp2(nx2);
+        }
         }
         for (int j0 = s0; j0 < s1; j0 += 32) {
             h8 a[NS];
