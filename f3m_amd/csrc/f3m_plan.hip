@@ -185,7 +185,7 @@ static ClassifyParams classify_params(const f3m_plan &P, float edge)
 // events that fork it from and join it to the caller's stream.  Default priority, kept for the life of the process.
 struct SideStream {
     hipStream_t stream = nullptr;
-    hipEvent_t fork = nullptr, join = nullptr;
+    hipEvent_t fork = nullptr, join = nullptr, tables = nullptr;
 };
 static SideStream &side_stream()
 {
@@ -199,6 +199,7 @@ static SideStream &side_stream()
         F3M_HIP(hipStreamCreateWithFlags(&ss.stream, hipStreamNonBlocking));
         F3M_HIP(hipEventCreateWithFlags(&ss.fork, hipEventDisableTiming));
         F3M_HIP(hipEventCreateWithFlags(&ss.join, hipEventDisableTiming));
+        F3M_HIP(hipEventCreateWithFlags(&ss.tables, hipEventDisableTiming));
     }
     return ss;
 }
@@ -708,37 +709,55 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         {
             ParkingLot lot;
             lot.start();
+            // The lists of the deepest level come first: they are the long launches, and their tables are ready or
+            // nearly so (the plan prepared the source operands beside its level loop).  The tables of the shallower
+            // levels' lists (kept with the plan from then on) are built on the second stream meanwhile, ahead of the
+            // far field; those lists follow on the caller's stream once their tables are there.  The order of the
+            // launches, and with it the order in which a target's sums are added, is the same on one stream.
+            const bool deepest_only_list = keep_of(depth).n == 0;
             if (overlap) {
-                // The near field's own tables first (kept with the plan from then on), so that its long launches
-                // follow without delay; the streams part after that: the far field then runs beside those launches.
-                for (int k = 1; k <= depth; k++)
-                    near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc, bstride,
-                               ostride, /*only_list=*/k < depth || keep_of(depth).n == 0, /*prepare_only=*/true);
+                near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], small_of(depth), bs.get(), outs.get(), P->lcs, s, nc,
+                           bstride, ostride, /*only_list=*/deepest_only_list, /*prepare_only=*/true);
                 near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(), outs.get(), P->lcs, s, nc,
                            bstride, ostride, false, /*prepare_only=*/true);
                 F3M_HIP(hipEventRecord(side_stream().fork, s));
                 F3M_HIP(hipStreamWaitEvent(side_stream().stream, side_stream().fork, 0));
             }
-            // the near field first: it is the long pole, and the host needs a while to queue the far field's many
-            // small kernels
             DirectOut dnear;
             if (direct) { dnear.perm = TX.perm.get(); dnear.out = out; dnear.c = c; dnear.col = col; dnear.ncol = ncol; }
             const DirectOut *dn = direct ? &dnear : nullptr;
-            for (int k = 1; k <= depth; k++) {
-                // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
-                near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
-                           bstride, ostride, /*only_list=*/k < depth || keep_of(depth).n == 0, false, dn);
-                if (per_level) {
+            if (per_level) {
+                for (int k = 1; k <= depth; k++) {
+                    // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
+                    near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
+                               bstride, ostride, /*only_list=*/k < depth || deepest_only_list, false, dn);
                     const size_t mark = arena_mark();
                     for (int q = 0; q < ncol; q++) {
                         arena_rewind(mark);
                         far_level(P, k, bs.get() + q * bstride, outs.get() + q * ostride, nullptr, nullptr, s);
                     }
                 }
+                // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
+                near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
+                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
+            } else {
+                // F3M_src/n_tree.cu:1018-1051 and :1092-1094: exact sums of the small pairs of every level and of what
+                // is still "keep" after the last division
+                near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], small_of(depth), bs.get(), outs.get(), P->lcs, s, nc,
+                           bstride, ostride, /*only_list=*/deepest_only_list, false, dn);
+                near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
+                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
+                if (overlap) {       // (queued after the long launches: the host needs a while for these many small kernels)
+                    for (int k = 1; k < depth; k++)
+                        near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs,
+                                   side_stream().stream, nc, bstride, ostride, /*only_list=*/true, /*prepare_only=*/true);
+                    F3M_HIP(hipEventRecord(side_stream().tables, side_stream().stream));
+                    F3M_HIP(hipStreamWaitEvent(s, side_stream().tables, 0));
+                }
+                for (int k = 1; k < depth; k++)
+                    near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
+                               bstride, ostride, /*only_list=*/true, false, dn);
             }
-            // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
-            near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
-                       outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
             // the far field: beside the near field on the second stream into its own array, or after it on the one
             // stream; either way a result is (near sums) + (far sum)
             if (!per_level) {
