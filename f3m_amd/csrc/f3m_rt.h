@@ -431,29 +431,38 @@ inline void dev_fill(void *p, int byte, size_t bytes, hipStream_t s)
 
 // ---- wave helpers ---------------------------------------------------------------------------
 #ifdef F3M_CPU_EMU
-__device__ inline unsigned long long wave_ballot(bool p) { return emu::ballot(p); }
+// Every wave-wide operation carries the source line of its call: the emulation stops when the lanes of one wavefront
+// arrive at operations of different lines, as they do when an exchange sits inside a branch that only some lanes
+// take (on the GPU such an exchange sees the lanes of the branch only).
+__device__ inline unsigned long long wave_ballot(bool p, int site = __builtin_LINE()) { return emu::ballot(p, site); }
 // orders the LDS accesses of the lanes of one wavefront (the lanes run in lockstep on the GPU)
-__device__ inline void wave_sync() { (void)emu::ballot(false); }
+__device__ inline void wave_sync(int site = __builtin_LINE()) { (void)emu::ballot(false, site); }
 __device__ inline unsigned lane_id() { return emu::S().cur->tid % 64; }
 __device__ inline float fast_exp2(float x) { return exp2f(x); }
 __device__ inline float fast_rcp(float x) { return 1.0f / x; }
-__device__ inline float wave_shfl_f(float v, int src)
+__device__ inline float wave_shfl_f(float v, int src, int site = __builtin_LINE())
 {
     uint32_t u;
     memcpy(&u, &v, 4);
-    u = emu::shfl_bits(u, src);
+    u = emu::shfl_bits(u, src, site);
     memcpy(&v, &u, 4);
     return v;
 }
 // value of lane (l & ~3) | K of the same group of four lanes
-template <int K> __device__ inline float quad_bcast(float v) { return wave_shfl_f(v, (int)((lane_id() & ~3u) | K)); }
-__device__ inline int wave_shfl_i(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }
-__device__ inline int wave_readlane(int v, int src) { return (int)emu::shfl_bits((uint32_t)v, src); }   // src uniform
-__device__ inline float wave_shfl_xor_f(float v, int mask)
+template <int K> __device__ inline float quad_bcast(float v, int site = __builtin_LINE())
+{
+    return wave_shfl_f(v, (int)((lane_id() & ~3u) | K), site);
+}
+__device__ inline int wave_shfl_i(int v, int src, int site = __builtin_LINE()) { return (int)emu::shfl_bits((uint32_t)v, src, site); }
+__device__ inline int wave_readlane(int v, int src, int site = __builtin_LINE())   // src uniform
+{
+    return (int)emu::shfl_bits((uint32_t)v, src, site);
+}
+__device__ inline float wave_shfl_xor_f(float v, int mask, int site = __builtin_LINE())
 {
     uint32_t u;
     memcpy(&u, &v, 4);
-    u = emu::shfl_bits(u, (int)(lane_id() ^ (unsigned)mask));
+    u = emu::shfl_bits(u, (int)(lane_id() ^ (unsigned)mask), site);
     memcpy(&v, &u, 4);
     return v;
 }
@@ -514,13 +523,13 @@ struct h8 {
 // D = A(32x16) B(16x32) + C with f16 inputs and fp32 accumulation: lane l supplies row l%32 of A and
 // column l%32 of B for the eight inner indices of its half-wave and holds D[8(r/4) + 4(l/32) + r%4][l%32]
 // in element r
-__device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c)
+__device__ inline f32x16 mfma_32x32x16_f16(h8 a, h8 b, f32x16 c, int site = __builtin_LINE())
 {
     uint32_t A[4][64], B[4][64];
     uint32_t wa[4], wb[4];
     memcpy(wa, &a, 16);
     memcpy(wb, &b, 16);
-    for (int w = 0; w < 4; w++) { emu::gather_bits(wa[w], A[w]); emu::gather_bits(wb[w], B[w]); }
+    for (int w = 0; w < 4; w++) { emu::gather_bits(wa[w], A[w], site); emu::gather_bits(wb[w], B[w], site); }
     const unsigned l = lane_id(), j = l & 31, h = l >> 5;
     for (int r = 0; r < 16; r++) {
         unsigned i = 8 * (r / 4) + 4 * h + (r % 4);

@@ -135,6 +135,7 @@ struct Wave {
     uint64_t bits[2];
     uint32_t vals[2][WAVE];
     int arrived, gen, alive;
+    int site;          // source line of the wave-wide operation that the lanes of this generation are arriving at
 };
 
 struct Fiber {
@@ -233,41 +234,50 @@ inline void syncthreads()
 
 inline Wave &wave() { State &s = S(); return s.waves[s.cur->tid / WAVE]; }
 
-inline void wave_barrier(Wave &w)
+// site: the source line of the calling wave-wide operation.  Lanes of one wavefront that meet here from different
+// lines have diverged around an exchange (one sits in a branch that not every lane takes): on the GPU such an exchange
+// reads lanes that are switched off, so the emulation refuses to go on.
+inline void wave_barrier(Wave &w, int site)
 {
     int my = w.gen;
+    if (w.arrived == 0) w.site = site;
+    else if (w.site != site) {
+        fprintf(stderr, "emu: lanes of one wavefront are at different wave-wide operations (source lines %d and %d): "
+                        "an exchange inside a branch that only some lanes take?\n", w.site, site);
+        abort();
+    }
     if (++w.arrived == w.alive) { w.arrived = 0; w.bits[(w.gen & 1) ^ 1] = 0; w.gen++; }
     else while (w.gen == my) yield();
 }
 
-inline uint64_t ballot(bool pred)
+inline uint64_t ballot(bool pred, int site)
 {
     Wave &w = wave();
     int slot = w.gen & 1;
     unsigned lane = S().cur->tid % WAVE;
     if (pred) w.bits[slot] |= 1ull << lane;
-    wave_barrier(w);
+    wave_barrier(w, site);
     return w.bits[slot];
 }
 
-inline uint32_t shfl_bits(uint32_t v, int src)
+inline uint32_t shfl_bits(uint32_t v, int src, int site)
 {
     Wave &w = wave();
     int slot = w.gen & 1;
     unsigned lane = S().cur->tid % WAVE;
     w.vals[slot][lane] = v;
-    wave_barrier(w);
+    wave_barrier(w, site);
     return w.vals[slot][src & (WAVE - 1)];
 }
 
 // every lane's value of the wave (exited lanes keep their last deposit)
-inline void gather_bits(uint32_t v, uint32_t *out)
+inline void gather_bits(uint32_t v, uint32_t *out, int site)
 {
     Wave &w = wave();
     int slot = w.gen & 1;
     unsigned lane = S().cur->tid % WAVE;
     w.vals[slot][lane] = v;
-    wave_barrier(w);
+    wave_barrier(w, site);
     memcpy(out, w.vals[slot], sizeof(uint32_t) * WAVE);
 }
 

@@ -367,3 +367,20 @@ def test_error_paths():
         ee.kmvm(np.zeros((50, 11), f32), None, b)
     # all points identical: cannot be divided, exact product
     assert np.allclose(ee.kmvm(np.ones((50, 3), f32), None, b, min_points=10), b.sum(0), rtol=1e-5)
+
+
+def test_emulation_refuses_exchange_in_divergent_branch(tmp_path):
+    """A lane exchange that only some lanes of a wavefront reach (here: on the right of `&&`) reads switched-off lanes
+    on the GPU.  The emulation tags every wave-wide operation with its source line and stops when the lanes of a
+    wavefront meet at different ones; the same kernel with the exchange made by every lane runs through."""
+    import os
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpu_emu")
+    exe = str(tmp_path / "divergent_exchange")
+    subprocess.check_call(["g++", "-O1", "-std=c++17", "-DF3M_CPU_EMU", "-I", here, "-I",
+                           os.path.join(here, "..", "..", "f3m_amd", "csrc"), "-w",
+                           os.path.join(here, "divergent_exchange.cpp"), "-o", exe, "-lpthread"])
+    good = subprocess.run([exe, "good"], capture_output=True, text=True)
+    assert good.returncode == 0 and good.stdout.strip() == "32"
+    bad = subprocess.run([exe, "bad"], capture_output=True, text=True)
+    assert bad.returncode != 0 and "different wave-wide operations" in bad.stderr
