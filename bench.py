@@ -128,7 +128,10 @@ def run_config(name, n, steps, warmup, subsample, keep_inputs=False, nodes=None,
            "points_per_s": n / (dt / steps), "tree_depth": depth, "boxes": nbx,
            "stage_ms_per_step": split_stages(stage, steps),
            "near": {"achieved_tflops": achieved, "frac": achieved / PEAK_FP32_TFLOPS, "launches_per_step": near_n // max(steps, 1),
-                    "ms_per_step": near_t / steps * 1e3, "flops_per_pair": F},
+                    "ms_per_step": near_t / steps * 1e3, "flops_per_pair": F,
+                    # the part of a pair that stays on the vector ALU whatever the dimension: one exp2 and one FMA, 12
+                    # issue cycles per 64 pairs, which at 3-D is the same figure as `frac` (12 flops per pair)
+                    "valu_frac": 12 * work["near_pairs"] * steps / max(near_t, 1e-12) / 1e12 / PEAK_FP32_TFLOPS},
            "work": work}
     if one_stream_steps:
         # the same product with everything on the caller's stream (F3M_OVERLAP=0): every stage alone on the GPU
@@ -159,7 +162,8 @@ def extra_record(r, steps):
     return {"ms_per_step": r["ms_per_step"], "ms_per_step_median": r["ms_per_step_median"],
             "rel_l2_error": r.get("rel_l2_error"), "meets_1e-3": r.get("meets_1e-3"),
             "algorithm_error_at_this_config": r.get("algorithm_error_at_this_config"),
-            "near_frac": r["near"]["frac"], "near_ms": r["near"]["ms_per_step"],
+            "near_frac": r["near"]["frac"], "near_flops_per_pair": r["near"]["flops_per_pair"],
+            "near_valu_frac": r["near"]["valu_frac"], "near_ms": r["near"]["ms_per_step"],
             "near_launches": r["near"]["launches_per_step"], "tree_depth": r["tree_depth"],
             "stage_ms_per_step": r["stage_ms_per_step"], "steps": steps}
 
@@ -318,6 +322,10 @@ def main():
             extra[other]["node_sweep"] = sweep
         if not args.no_falkon and N == 10_000_000:
             extra["falkon_krr"] = falkon_record()
+        extra["note"] = ("near_frac = (3d+3) algorithmic flops per near pair / near-field time, against the fp32 peak; the 3d "
+                         "flops of the distance run on the f16 matrix pipe, so beyond 3-D (where 3d+3 = 12 and the two figures "
+                         "coincide) near_frac can pass 1; near_valu_frac counts the 12 vector-ALU issue cycles per 64 pairs "
+                         "(one exp2, one FMA) that remain on the vector ALU in every dimension")
         res["extra"] = extra
     print(json.dumps(res))
 
