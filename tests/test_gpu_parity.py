@@ -689,6 +689,37 @@ def test_repeated_products_have_the_same_bits(eng):
             assert np.array_equal(plans[i].apply(b).cpu().numpy(), first[i]), (rep, i, "plan")
 
 
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "clustered_xy", "uniform5_243"])
+def test_one_stream_and_two_streams_give_the_same_bits(eng, monkeypatch, name):
+    """The far field runs on a second stream beside the near field, and on clouds with near lists on several levels
+    the tables of the shallower levels' lists are built there while the deepest level's lists are summed.  With
+    F3M_OVERLAP=0 everything is queued on the caller's stream.  The launches that add to a target come in the same
+    order either way (deepest level first), and near and far sums meet in one addition: the bits must not depend on the
+    mode, for a one-shot product and for a kept plan, with one and three columns."""
+    print("case one stream / two streams", name, flush=True)
+    rng = np.random.default_rng(31)
+    X, Y, prm = clouds(name, rng)
+    M = X.shape[0] if Y is None else Y.shape[0]
+    Xd, Yd = dev(X), None if Y is None else dev(Y)
+    for c in (1, 3):
+        b = dev(rng.standard_normal((M, c)).astype(f32))
+        two = eng.kmvm(Xd, Yd, b, **prm).cpu().numpy()
+        plan = eng.Plan(Xd, Yd, **prm)
+        lists = sum(1 for k in range(1, plan.depth + 1) for w in ("nsmall", "nkeep")
+                    if plan.level_sizes(k)[w] and (w == "nsmall" or k == plan.depth))
+        if name == "normal3":
+            assert lists >= 2                      # the case the order of launches matters for
+        assert np.array_equal(plan.apply(b).cpu().numpy(), two)
+        plan.close()
+        monkeypatch.setenv("F3M_OVERLAP", "0")
+        one = eng.kmvm(Xd, Yd, b, **prm).cpu().numpy()
+        plan = eng.Plan(Xd, Yd, **prm)
+        one_plan = plan.apply(b).cpu().numpy()
+        plan.close()
+        monkeypatch.delenv("F3M_OVERLAP")
+        assert np.array_equal(one, two) and np.array_equal(one_plan, two)
+
+
 @pytest.mark.parametrize("c", [1, 3, 6])
 def test_results_added_straight_into_the_output_array(eng, monkeypatch, c):
     """Where the near field is one launch with one wavefront per work item and the far field is evaluated once, both
