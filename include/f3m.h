@@ -84,7 +84,11 @@ int f3m_plan_destroy(f3m_plan *plan);
  * except while the stream is being captured.  A captured call holds the addresses of the plan's tables: its
  * graph may be replayed while the plan lives (a table of a plan is built once and never replaced; destroying the
  * plan frees them); an error raised during capture leaves the capture to the caller (the library then waits
- * for nothing). */
+ * for nothing).  The library itself asks for no memory here; the HIP runtime, however, reserves its own
+ * per-queue scratch memory the first time a kernel that keeps registers there runs on a queue (some M2L and
+ * near-field instances do: a few dozen bytes per lane), and f3m_plan_apply runs the far field on the library's
+ * second stream.  A caller that must not see the device's free memory change runs one
+ * f3m_plan_apply_noalloc on its stream beforehand. */
 int f3m_plan_apply_noalloc(f3m_plan *plan, const float *b, int c, float *out, void *stream);
 
 /* Introspection for parity tests (no counterpart is exported by the reference; the data are its

@@ -165,3 +165,30 @@ def test_apply_without_allocation_under_graph_capture(eng):
     torch.cuda.synchronize()
     assert torch.equal(out, want2)
     plan.close()
+
+
+def test_apply_without_allocation_five_dimensions(eng):
+    """5-D: the near field takes its factored form, whose weights (the sorted b times exp2(-|y'|^2)) are one more
+    temporary per column group; it comes from the static scratch memory like the others.  One and three columns."""
+    import torch
+    print("case no-alloc: 5-D 200000 points, 243 nodes, 1 and 3 columns", flush=True)
+    rng = np.random.default_rng(35)
+    X = dev(rng.random((200000, 5), dtype=f32))
+    plan = eng.Plan(X, None, ls=1.0, nr_of_interpolation=243, min_points=1000, small_field_points=243)
+    assert plan.depth >= 2
+    for c in (1, 3):
+        b = dev(rng.standard_normal((200000, c)).astype(f32))
+        want = plan.apply(b)
+        out = torch.full((200000, c), float("nan"), device="cuda")
+        # The far field of plan.apply ran on the library's second stream.  Here its kernels run on the caller's stream
+        # for the first time, and the 5-D M2L kernel keeps some registers in the runtime's scratch memory, which the
+        # runtime reserves per queue when such a kernel first runs there: one product beforehand, as the header says.
+        plan.apply_noalloc(b, out)
+        torch.cuda.synchronize()
+        out.fill_(float("nan"))
+        eng.release_cache()
+        free0 = torch.cuda.mem_get_info()[0]
+        plan.apply_noalloc(b, out)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free0
+        assert np.array_equal(out.cpu().numpy(), want.cpu().numpy())
