@@ -40,6 +40,10 @@ def clouds(name, rng):
     if name == "uniform5":
         return rng.random((60000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=32, min_points=100,
                                                               small_field_points=40)
+    if name == "normal5":            # near lists on several levels in 5-D (the factored near-field form, operand
+        # tables of listed boxes only, two columns at a time)
+        return rng.standard_normal((60000, 5)).astype(f32), None, dict(ls=2.0, nr_of_interpolation=32, min_points=300,
+                                                                        small_field_points=100)
     if name == "uniform5_243":       # config 4: 3^5 nodes per box; 390 points per box at depth 2, so pairs of boxes
         # there hold more than 2 * 243 points and are far wherever they are two or more boxes apart
         return rng.random((400000, 5), dtype=f32), None, dict(ls=1.0, nr_of_interpolation=243, min_points=1000,
@@ -290,7 +294,7 @@ def test_exact_kernels(eng, oracle, d):
     assert rel_l2(eng.exact_grad_f32(dev(X), dev(Y), dev(b), ls).cpu().numpy(), oracle.exact_grad_f32(X, Y, b, ls)) < 1e-5
 
 
-@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform5_243",
+@pytest.mark.parametrize("name", ["normal3", "clustered_xy", "uniform4", "uniform2", "uniform5", "uniform5_243", "normal5",
                                   "uniform3_varcomp", "uniform3_125", "uniform3_216"])
 def test_stages_against_oracle(eng, oracle, name):
     print("case stages", name, flush=True)
