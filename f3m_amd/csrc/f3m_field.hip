@@ -420,7 +420,8 @@ __global__ void __launch_bounds__(512) near_kernel(const float *__restrict__ xs,
 // the source factor rides on the weight (one multiplication per source and product, near_weights_kernel), the target
 // factor multiplies the sum over a run of sources once.  It takes one instruction where 3D+4 slots take two
 // (D = 5: 15 against 19 slots), at the price of exponentials whose arguments no longer cancel: |u| <= 10 D S^2 with
-// S = (box edge) sqrt(lcs log2 e), so the host takes the form only while that stays far from the exponent range.
+// S = (box edge) sqrt(lcs log2 e), so the host takes the form only while that stays far from the exponent range
+// (near_factored).
 __host__ __device__ constexpr int near_slots(int D, bool fact = false) { return fact ? 3 * D : 3 * D + 4; }
 __host__ __device__ constexpr int near_insts(int D, bool fact = false) { return (near_slots(D, fact) + 15) / 16; }
 // dimensions whose factored form saves an instruction (the others never take it)
@@ -842,12 +843,14 @@ static bool near_on_matrix_pipe(int d, float lcs, float edge)
 
 // whether the near field of a level takes the factored form (see near_slots): only where it saves a matrix
 // instruction, and while the exponent 2x''.y' (at most 10 d S^2, targets within five edges of the anchor and sources
-// within one) stays below 60.  F3M_NEAR_FACT=0|1 overrides (1: wherever the form saves an instruction).
+// within one) stays below 30: the sum of a run, exp2(2x''.y') times weights, then stays below 2^30 times the weights'
+// sum, so that weights up to ~1e28 cannot overflow where the plain form (every term at most its weight) would not.
+// F3M_NEAR_FACT=0|1 overrides (1: wherever the form saves an instruction).
 static bool near_factored(int d, float lcs, float edge)
 {
     const bool pays = d == 5 || d == 10;             // near_fact_pays(d)
     const float S = sqrtf(lcs * kLog2e) * edge;
-    bool fact = pays && 10.f * (float)d * S * S <= 60.f;
+    bool fact = pays && 10.f * (float)d * S * S <= 30.f;
     if (const char *env = getenv("F3M_NEAR_FACT")) fact = pays && atoi(env) != 0;
     return fact;
 }
