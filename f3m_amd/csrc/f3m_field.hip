@@ -694,6 +694,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             tcur += nt;
             if (a >= b) continue;                    // uniform
         }
+        // (both are the same in every lane, which the compiler cannot see through the slicing above: as scalars they
+        // keep the loop over the tiles of the run off the vector ALU)
+        s0 = wave_uniform(s0);
+        s1 = wave_uniform(s1);
         float run[TPW][NC];                           // factored form: the sums of this run
 #pragma unroll
         for (int q = 0; q < TPW; q++)
@@ -746,9 +750,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                     bq[c][4 * g + 0] = f.x; bq[c][4 * g + 1] = f.y; bq[c][4 * g + 2] = f.z; bq[c][4 * g + 3] = f.w;
                 }
             if (j0 + 32 > s1) {
+                const int lim = s1 - j0 - 4 * half;      // rows of this lane's half of the tile that are left in the box
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const bool in = j0 + 8 * (r / 4) + 4 * half + (r % 4) < s1;
+                    const bool in = 8 * (r / 4) + (r % 4) < lim;
 #pragma unroll
                     for (int c = 0; c < NC; c++) bq[c][r] = in ? bq[c][r] : 0.f;
                 }

@@ -454,6 +454,7 @@ template <int K> __device__ inline float quad_bcast(float v, int site = __builti
     return wave_shfl_f(v, (int)((lane_id() & ~3u) | K), site);
 }
 __device__ inline int wave_shfl_i(int v, int src, int site = __builtin_LINE()) { return (int)emu::shfl_bits((uint32_t)v, src, site); }
+__device__ inline int wave_uniform(int v) { return v; }
 __device__ inline int wave_readlane(int v, int src, int site = __builtin_LINE())   // src uniform
 {
     return (int)emu::shfl_bits((uint32_t)v, src, site);
@@ -561,6 +562,8 @@ template <int K> __device__ __forceinline__ float quad_bcast(float v)
 __device__ __forceinline__ int wave_shfl_i(int v, int src) { return __shfl(v, src, 64); }
 // value of one lane, the same lane for the whole wavefront (v_readlane_b32: the result is scalar)
 __device__ __forceinline__ int wave_readlane(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
+// a value that is the same in every lane, as a scalar (no exchange: the first active lane's copy)
+__device__ __forceinline__ int wave_uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 __device__ __forceinline__ float wave_shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, 64); }
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half_t;
