@@ -933,17 +933,15 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 
 // the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
 // the list, the exact number of work items (else -1)
-static void near_shape(int d, float lcs, const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw,
-                       long long &items_exact)
+static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact)
 {
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
     const long long tiles = (avg_points + 31) / 32;
     tpw = (tiles == 5 && nc == 1) ? 5 : 4;
-    // The factored 5-D kernel has the registers for a fifth tile at the same number of wavefronts per SIMD (117 and
-    // 128 registers): five wherever that cuts a typical box into fewer work items (ten tiles: 5 + 5 instead of
-    // 4 + 4 + 2; N=1e7, 5-D: near field beside the far field 39.2 -> 36.9 ms).  In 3-D the fifth tile costs a
-    // wavefront per SIMD (9.5 -> 9.8 ms per product).
-    if (d == 5 && nc == 1 && near_factored(d, lcs, lx.edge) && (tiles + 4) / 5 < (tiles + 3) / 4) tpw = 5;
+    // (The factored 5-D kernel with a fifth tile, ten tiles of a box as 5 + 5 instead of 4 + 4 + 2, takes 127 registers:
+    // four wavefronts then fill the 512 of a SIMD and the far field's wavefronts get in beside them only now and
+    // then.  N=1e7: the fastest products 39.8 ms against 40.9, but single products up to 48.9 and means of 40.8-42.8
+    // against a steady 41.0 with four tiles, 115 registers.  Four it is.)
     if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
     items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
 }
@@ -953,7 +951,7 @@ bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList
     if (list.n == 0 || !near_on_matrix_pipe(d, lcs, lx.edge)) return false;
     int tpw;
     long long items_exact;
-    near_shape(d, lcs, tx, lx, list, nc, tpw, items_exact);
+    near_shape(tx, lx, list, nc, tpw, items_exact);
     return items_exact >= 16384;          // fewer work items: the lists are cut into slices with partial sums
 }
 
@@ -985,7 +983,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     int tpw;
     long long items_exact;
-    near_shape(d, lcs, tx, lx, list, nc, tpw, items_exact);
+    near_shape(tx, lx, list, nc, tpw, items_exact);
     // From five dimensions on the work items are long and their lists differ a lot in length (3^5 boxes around
     // an interior box, 2^5 around a corner): the boxes with the longest lists go first, which shortens the
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
