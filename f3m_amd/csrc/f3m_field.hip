@@ -1798,8 +1798,10 @@ __global__ void __launch_bounds__(MAXT) m2l_sib_kernel(const float *__restrict__
                                                         const int *__restrict__ childstart,
                                                         const int *__restrict__ cell, const int *__restrict__ pairs,
                                                         const int *__restrict__ rowptr, const float *__restrict__ mom,
-                                                        float *__restrict__ loc)
+                                                        float *__restrict__ loc, const unsigned char *__restrict__ taken)
 {
+    // taken (nullable): one byte per parent and regular table cell, set for the cells that m2l_shared_kernel has summed
+    // already (its results are in loc; this kernel then leaves those cells out and adds to loc)
     // H = 2: the n0 x n1 nodes of a lane are shared by two lanes, n1/2 values of a1 each (a workgroup of
     // 2^D siblings x R2 lanes would otherwise fill half a wavefront in 3-D); NN = nodes of a lane
     // W: row length of the padded tables of the first two factors (rows are read as vectors of four)
@@ -1880,7 +1882,10 @@ __global__ void __launch_bounds__(MAXT) m2l_sib_kernel(const float *__restrict__
                 const int code = sib_code<D>(dg);
                 if (code >= 0) {
                     const int c = code - pass * chunk;
-                    if (c >= 0 && c < chunk) { tby[c] = by; atomicOr(&tmask[c], 1u << s2); }
+                    if (c >= 0 && c < chunk && !(taken != nullptr && taken[(long long)px * NCODE + code])) {
+                        tby[c] = by;
+                        atomicOr(&tmask[c], 1u << s2);
+                    }
                 } else if (code <= -2 && pass == 0) { xby[-2 - code] = by; atomicOr(&xmask[-2 - code], 1u << s2); }
             }
         }
@@ -2089,6 +2094,11 @@ __global__ void __launch_bounds__(MAXT) m2l_sib_kernel(const float *__restrict__
     if (have) flush_upto(D - 1);
     if (live) {
         float *dst = loc + (long long)mybox * P + (long long)NN * r2h;
+        if (taken != nullptr) {
+#pragma unroll
+            for (int i = 0; i < NN; i++) dst[i] += acc[D - 1][i];
+            return;
+        }
 #pragma unroll
         for (int i = 0; i + 4 <= NN; i += 4) {
             fvec<4> r;
@@ -2098,6 +2108,205 @@ __global__ void __launch_bounds__(MAXT) m2l_sib_kernel(const float *__restrict__
         }
 #pragma unroll
         for (int i = NN & ~3; i < NN; i++) dst[i] = acc[D - 1][i];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Sibling-group M2L, the far cells that EVERY child of a parent lists (most of them: all cells that are not next to the
+// parent's own block of children).  For such a cell the 2^D siblings differ only in the tables they apply, and the
+// table of dimension j depends on the sibling's bit j alone: E_j[u_j - b_j].  So the sums are formed once per
+// combination of bits seen so far, not once per sibling: after factor 0 there are two variants (b0), after factor 1
+// four (b0, b1), ... and only after the last factor one per sibling.  Lane (b0, c1, .., c_{D-1}) holds, for its b0 and
+// its position c_j among the nodes of dimensions >= 1, the N values over the nodes of dimension 0 of every variant
+// (b1..bj) of level j: N (2^D - 1) partial sums in registers.  Per far box a lane loads N moments and does N^2
+// multiply-adds, where m2l_sib_kernel spends N^2 n1 multiply-adds in each of 2^D siblings' lanes; factor j+1 is applied
+// when the offsets of dimensions > j change, with the values exchanged through LDS between the lanes that differ in
+// c_{j+1}.  One workgroup per parent, 2 N^(D-1) lanes.  The cells taken are flagged in `taken` (one byte per parent and
+// cell) for m2l_sib_kernel, which runs afterwards on the rest -- cells next to the parent's block, cells of the
+// extension table -- and adds to loc.  Same sums up to rounding.  Preconditions: N nodes in every dimension, one
+// tree, every far pair inside the tables (as for m2l_sib_kernel).
+__host__ __device__ constexpr int ipow_c(int b, int e) { return e == 0 ? 1 : b * ipow_c(b, e - 1); }
+
+template <int D, int N>
+__global__ void __launch_bounds__(256) m2l_shared_kernel(const float *__restrict__ tables, int ntab, SepMeta sm, int P, int npass,
+                                                          const int *__restrict__ order, const int *__restrict__ childstart,
+                                                          const int *__restrict__ cell, const int *__restrict__ pairs,
+                                                          const int *__restrict__ rowptr, const float *__restrict__ mom,
+                                                          float *__restrict__ loc, unsigned char *__restrict__ taken)
+{
+    constexpr int NCODE = sib_codes(D), NSIB = 1 << D, R = ipow_c(N, D - 1), LANES = 2 * R, NB = 8;
+    constexpr int XV = N << (D - 2);                                // most values a lane hands over in one exchange
+    constexpr int NACC = N * (NSIB - 1);                            // level j: 2^j variants of N values, from N (2^j - 1) on
+    F3M_DYN_SHARED(float, smem);
+    const int tid = threadIdx.x, BD = blockDim.x, lane = tid & 63;
+    const int chunk = NCODE / npass;
+    // chunk: y box of a table cell (below 2^24, checked by the host) + 2^24 times the number of siblings that list it
+    // while the table is filled, then the box of a cell that is taken or -1
+    int *tby = reinterpret_cast<int *>(smem);
+    float *xbuf = smem + chunk;                                     // XV * BD: exchange buffer
+    float *tabg = xbuf + XV * BD;                                   // ntab: E_j[o][a][q], row length sm.NT
+    int *sib = reinterpret_cast<int *>(tabg + ((ntab + 3) & ~3));   // NSIB: box of each sibling or -1
+    const int px = order ? order[blockIdx.x] : blockIdx.x;
+    unsigned char *tk = taken + (long long)px * NCODE;
+
+    for (int e = tid; e < ntab; e += BD) tabg[e] = tables[e];
+    if (tid < NSIB) sib[tid] = -1;
+    __syncthreads();
+    const int c0 = childstart[px], c1 = childstart[px + 1];
+    for (int c = c0 + tid; c < c1; c += BD) {
+        int code = 0;
+#pragma unroll
+        for (int j = 0; j < D; j++) code |= (cell[(long long)c * D + j] & 1) << j;
+        sib[code] = c;
+    }
+    int pc[D];
+#pragma unroll
+    for (int j = 0; j < D; j++) pc[j] = 2 * (cell[(long long)c0 * D + j] >> 1) - 2;
+    __syncthreads();
+    int nlive = 0;
+    for (int s2 = 0; s2 < NSIB; s2++) nlive += sib[s2] >= 0 ? 1 : 0;
+
+    // part `pass` of the table from the far rows of every sibling; then only the cells that every sibling lists stay
+    auto fill_tables = [&](int pass) __attribute__((always_inline)) {
+        for (int e = tid; e < chunk; e += BD) tby[e] = 0;
+        __syncthreads();
+        for (int s2 = 0; s2 < NSIB; s2++) {
+            const int bx = sib[s2];
+            if (bx < 0) continue;                          // uniform over the workgroup
+            const int m1 = rowptr[bx + 1];
+            for (int m = rowptr[bx] + tid; m < m1; m += BD) {
+                const int by = pairs[2 * (long long)m + 1];
+                int dg[D];
+#pragma unroll
+                for (int j = 0; j < D; j++) dg[j] = cell[(long long)by * D + j] - pc[j];
+                const int code = sib_code<D>(dg);
+                const int c = code - pass * chunk;
+                if (code >= 0 && c >= 0 && c < chunk) { atomicOr(&tby[c], by); atomicAdd(&tby[c], 1 << 24); }
+            }
+        }
+        __syncthreads();
+        for (int e = tid; e < chunk; e += BD) {
+            const int w = tby[e];
+            const bool full = (w >> 24) == nlive;
+            tby[e] = full ? (w & 0xffffff) : -1;
+            tk[pass * chunk + e] = full ? 1 : 0;
+        }
+        __syncthreads();
+    };
+
+    // this lane: bit 0 of its siblings, and its position among the nodes of dimensions >= 1
+    const bool valid = tid < LANES;
+    const int b0 = tid & 1, cidx = valid ? tid >> 1 : 0;
+    int cj[D], lstride[D];
+    {
+        int rem = cidx, st = 2;
+        cj[0] = 0; lstride[0] = 0;
+#pragma unroll
+        for (int j = 1; j < D; j++) { cj[j] = rem % N; rem /= N; lstride[j] = st; st *= N; }     // lstride: in lanes
+    }
+    const float *mine = mom + (long long)N * cidx;
+    float acc[NACC];
+#pragma unroll
+    for (int i = 0; i < NACC; i++) acc[i] = 0.f;
+    int curpk = 0;
+    bool have = false;
+    auto digit2 = [](int pk, int j) __attribute__((always_inline)) { return (pk >> (4 * j)) & 15; };      // digit j + 2
+    // table row E_j[o][a][.] for the offset of the current far cell in dimension j and a sibling with bit b
+    auto table_row = [&](int pk, int j, int b, int a) __attribute__((always_inline)) {
+        int oi = digit2(pk, j) - (4 + b + sm.omin[j]);
+        oi = min(max(oi, 0), kM2LOffsets - 1);
+        return tabg + ((j * kM2LOffsets + oi) * sm.NT + a) * sm.NT;
+    };
+    // applies factor l+1 to the 2^l variants of level l, adds the results to the 2^(l+1) variants of level l+1 and
+    // clears level l
+    auto flush = [&](auto level) __attribute__((always_inline)) {
+        constexpr int l = decltype(level)::value, j = l + 1, NV = 1 << l, src0 = N * (NV - 1), dst0 = N * (2 * NV - 1);
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < N * NV; i++) xbuf[i * BD + tid] = acc[src0 + i];
+        __syncthreads();
+        if (valid) {
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                const float *row = table_row(curpk, j, b, cj[j]);
+                for (int q = 0; q < N; q++) {
+                    const float w = row[q];
+                    const float *src = xbuf + tid + (q - cj[j]) * lstride[j];
+#pragma unroll
+                    for (int i = 0; i < N * NV; i++)
+                        acc[dst0 + N * NV * b + i] = fmaf(w, src[i * BD], acc[dst0 + N * NV * b + i]);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < N * NV; i++) acc[src0 + i] = 0.f;
+    };
+    auto flush_upto = [&](int jt) __attribute__((always_inline)) {       // levels 0 .. jt-1, jt uniform over the workgroup
+        if (jt > 0) flush(std::integral_constant<int, 0>());
+        if constexpr (D > 2) { if (jt > 1) flush(std::integral_constant<int, 1>()); }
+        if constexpr (D > 3) { if (jt > 2) flush(std::integral_constant<int, 2>()); }
+        if constexpr (D > 4) { if (jt > 3) flush(std::integral_constant<int, 3>()); }
+    };
+    // one far box: pk = its packed digits (uniform), v = its moments at this lane's nodes of dimension 0
+    auto far_box = [&](int pk, const float (&v)[N]) __attribute__((always_inline)) {
+        if (have) {
+            const int diff = (pk ^ curpk) >> 4;             // digits 1.. that change
+            flush_upto(diff ? (31 - __builtin_clz(diff)) / 4 + 1 : 0);   // up to the highest of them
+        }
+        curpk = pk;
+        have = true;
+#pragma unroll
+        for (int a0 = 0; a0 < N; a0++) {
+            const float *row = table_row(pk, 0, b0, a0);
+#pragma unroll
+            for (int q = 0; q < N; q++) acc[a0] = fmaf(row[q], v[q], acc[a0]);
+        }
+    };
+
+    for (int pass = 0; pass < npass; pass++) {
+        if (pass > 0) __syncthreads();                     // every wavefront is done with the previous part
+        fill_tables(pass);
+        for (int base = 0; base < chunk; base += 64) {
+            const int idx = base + lane;
+            const int byl = idx < chunk ? tby[idx] : -1;
+            int pkl = 0;                                   // packed digits of this lane's cell
+            {
+                int rem = pass * chunk + idx;
+#pragma unroll
+                for (int j = 0; j < D; j++) { pkl |= (rem % kSibSpan + 2) << (4 * j); rem /= kSibSpan; }
+            }
+            unsigned long long bal = wave_ballot(byl >= 0);
+            while (bal) {                                  // identical in every wavefront of the workgroup
+                int ls[NB], cnt = 0;
+                float v[NB][N];
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    ls[u] = 0;
+                    if (bal) { ls[u] = __ffsll(bal) - 1; bal &= bal - 1; cnt++; }
+                    // (past the last cell of this round the loads repeat box 0: lane 0's cell may be one not taken, -1)
+                    const int by = u < cnt ? wave_readlane(byl, ls[u]) : 0;
+#pragma unroll
+                    for (int q = 0; q < N; q++) v[u][q] = mine[(long long)by * P + q];
+                }
+#pragma unroll
+                for (int u = 0; u < NB; u++) {
+                    if (u >= cnt) break;                   // uniform
+                    far_box(wave_readlane(pkl, ls[u]), v[u]);
+                }
+            }
+        }
+    }
+    if (have) flush_upto(D - 1);
+    if (valid) {
+        constexpr int last0 = N * ((1 << (D - 1)) - 1);
+#pragma unroll
+        for (int var = 0; var < (1 << (D - 1)); var++) {
+            const int bx = sib[b0 | (var << 1)];
+            if (bx < 0) continue;
+            float *dst = loc + (long long)bx * P + (long long)N * cidx;
+#pragma unroll
+            for (int a0 = 0; a0 < N; a0++) dst[a0] = acc[last0 + N * var + a0];
+        }
     }
 }
 
@@ -2352,6 +2561,50 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
             // (instances bound to 128 threads for the groups of four siblings that run beside the near field, 4-D and 5-D,
             // have no spilled values but one wavefront per SIMD less: same time, not kept)
             const int maxt = (d == 3 && ns.n[0] >= 5) ? 64 : 1024;
+            // 3^4 grid beside the near field: the cells that every child of a parent lists are summed once per combination
+            // of sibling bits first (m2l_shared_kernel); the sibling kernel then takes what is left and adds.  A parent's
+            // cells are then walked by one wavefront instead of by three or more, with a sixth of the vector
+            // instructions: beside the near field, which is short of exactly those, the product gains (N=1e7, 4-D:
+            // 14.2 -> 13.7 ms); alone on the GPU the longer walk costs more than the instructions save (M2L 2.1 -> 2.4
+            // ms), and in 5-D, 1024 parents with 7776 cells each, it does not end before the near field does (40.9 ->
+            // 47.7 ms).  F3M_M2L_SHARED=0|1 overrides (1: 3^4 and 3^5 grids, in either mode).
+            const bool shared_fits = (d == 4 || d == 5) && sibH == 1 && ly.nb < (1 << 24) && ns.n[0] == 3 && ns.n[1] == 3 &&
+                                     ns.n[2] == 3 && ns.n[3] == 3 && (d == 4 || ns.n[4] == 3);
+            bool shared = shared_fits && d == 4 && beside_near;
+            if (const char *e = getenv("F3M_M2L_SHARED")) shared = shared_fits && atoi(e) != 0;
+            DBuf<unsigned char> taken;
+            if (shared) {
+                const int lanes = 2 * P / 3, sbd = ((lanes + kWave - 1) / kWave) * kWave, xv = 3 << (d - 2);
+                int spass = 1;
+                size_t shs3 = 0;
+                for (int np : {1, 2, 3, 6}) {
+                    spass = np;
+                    shs3 = sizeof(float) * ((size_t)(sib_codes(d) / np) + (size_t)xv * sbd + (size_t)((ntab + 3) & ~3)) +
+                           sizeof(int) * ((size_t)1 << d);
+                    if (shs3 <= 150 * 1024) break;
+                }
+                taken.reset((size_t)par.nb * sib_codes(d));
+                if (getenv("F3M_DEBUG"))
+                    fprintf(stderr, "m2l depth %d: shared sums first (%d lanes per parent, table parts %d, %zu bytes of LDS)\n", lx.depth,
+                            lanes, spass, shs3);
+#ifndef F3M_CPU_EMU
+#define F3M_SHARED_ATTR(DD)                                                                                            \
+    F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_shared_kernel<DD, 3>),                             \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shs3));
+#else
+#define F3M_SHARED_ATTR(DD)
+#endif
+#define F3M_SHARED(DD)                                                                                                 \
+    if (d == DD) {                                                                                                     \
+        F3M_SHARED_ATTR(DD)                                                                                            \
+        F3M_LAUNCH((m2l_shared_kernel<DD, 3>), par.nb, sbd, shs3, s, dtab.get(), ntab, sm, P, spass, sibOrd,           \
+                   par.childstart.get(), lx.cell.get(), far.pairs.get(), far.rowptr.get(), mom, loc, taken.get());     \
+    }
+                F3M_SHARED(4) F3M_SHARED(5)
+#undef F3M_SHARED
+#undef F3M_SHARED_ATTR
+                check_launch("m2l_shared");
+            }
 #ifndef F3M_CPU_EMU
 #define F3M_SIB_ATTR(DD, NNODE, HH, MT)                                                                                \
     F3M_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&m2l_sib_kernel<DD, NNODE, HH, MT>),                    \
@@ -2364,7 +2617,7 @@ void m2l_level(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const
         F3M_SIB_ATTR(DD, NNODE, HH, MT)                                                                                \
         F3M_LAUNCH((m2l_sib_kernel<DD, NNODE, HH, MT>), par.nb * nsub, bd, shsib, s, dtab.get(), ntab, sm, nm, sibR2,  \
                    sibGS, nsub, sibPass, sibOrd, par.childstart.get(), lx.cell.get(), far.pairs.get(),                 \
-                   far.rowptr.get(), mom, loc);                                                                        \
+                   far.rowptr.get(), mom, loc, shared ? taken.get() : (const unsigned char *)nullptr);                 \
     }
             F3M_SIB(3, 2, 2, 1024) F3M_SIB(3, 3, 1, 1024) F3M_SIB(3, 4, 2, 1024) F3M_SIB(3, 2, 1, 1024) F3M_SIB(3, 4, 1, 1024)
             F3M_SIB(3, 5, 1, 64) F3M_SIB(3, 6, 1, 64)

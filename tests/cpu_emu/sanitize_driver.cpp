@@ -2,7 +2,9 @@
 // the kernel sources under -fsanitize=address,undefined (tests/cpu_emu/build_emu.py: build_sanitize_driver).  It runs a
 // few small seeded problems -- one tree and two, 1 to 6 dimensions, several columns, variance compression, the
 // transposed product -- so that an access outside an array or undefined arithmetic in a kernel stops the program with a
-// report.  Usage: sanitize_driver <first case> <number of cases> [points].
+// report.  Usage: sanitize_driver <first case> <number of cases> [points [dimension nodes min_points small_field_points]]
+// (the last four replace what the case number would choose: e.g. 4 81 8 2 with 20000 points is a 4-D tree of three
+// levels on the 3^4 grid, whose M2L takes the cells that all siblings list first).
 #include "../../include/f3m.h"
 
 #include <cmath>
@@ -22,7 +24,7 @@ int main(int argc, char **argv)
         std::normal_distribution<float> Nn(0.f, 1.f);
         const int dims[] = {1, 2, 3, 3, 4, 5, 6, 3};
         const int nodes_by_d[] = {0, 8, 16, 27, 16, 32, 64};
-        const int d = dims[cs % 8];
+        const int d = argc > 7 ? atoi(argv[4]) : dims[cs % 8];
         const bool two = (cs % 3) == 1;
         const long long N = base + (long long)(g() % (unsigned)base), M = two ? base / 2 + (long long)(g() % (unsigned)base) : N;
         const int c = 1 + (cs % 4);
@@ -33,6 +35,12 @@ int main(int argc, char **argv)
         p.var_compression = (cs % 4) == 3;
         p.eff_var_limit = 0.3f;
         p.small_field_points = 5 + (int)(g() % 30);
+        if (argc > 7) {
+            p.nr_of_interpolation = atoi(argv[5]);
+            p.min_points = (float)atof(argv[6]);
+            p.small_field_points = atoi(argv[7]);
+            p.ls = 0.6f;
+        }
         std::vector<float> X((size_t)N * d), Y((size_t)M * d), b((size_t)M * c), out((size_t)N * c), out2((size_t)N * c),
             u((size_t)N), outT((size_t)M);
         const bool normal = cs % 2;

@@ -224,6 +224,27 @@ def test_m2l_forms_agree(monkeypatch, d, n, P, mp):
     assert rel_l2(grouped, direct) < 3e-6
 
 
+@pytest.mark.parametrize("d,n", [(4, 2000), (5, 5000)])
+def test_m2l_cells_listed_by_every_sibling_summed_once(oracle, monkeypatch, d, n):
+    """3^4 and 3^5 grids: the far cells that every child of a parent lists are summed once per combination of sibling
+    bits (m2l_shared_kernel), the sibling-group kernel adds the rest.  A thin slab (two long dimensions) reaches the
+    third level, where such cells exist, with a few thousand points.  Same sums as the sibling-group kernel alone up
+    to rounding, and as the oracle's."""
+    rng = np.random.default_rng(9)
+    X = rng.random((n, d), dtype=f32)
+    X[:, 2:] *= 0.12
+    b = rng.standard_normal((n, 1)).astype(f32)
+    prm = dict(ls=0.3, min_points=50, nr_of_interpolation=3 ** d, small_field_points=2)
+    eng = ee.Plan(X, None, **prm)
+    assert eng.depth == 3 and eng.level_sizes(2)["nfar"] > 100
+    monkeypatch.setenv("F3M_M2L_SHARED", "1")
+    shared = eng.apply(b)
+    monkeypatch.setenv("F3M_M2L_SHARED", "0")
+    plain = eng.apply(b)
+    assert 0 < rel_l2(shared, plain) < 1e-6            # not the same bits: some cells did go the other way
+    assert rel_l2(shared, oracle.Plan(X, None, **prm).apply(b)) < 3e-6
+
+
 @pytest.mark.parametrize("P", [125, 216])
 def test_grids_of_five_and_six_nodes_per_dimension(oracle, monkeypatch, P):
     """5 x 5 x 5 and 6 x 6 x 6 nodes (the grids of the reference's own sweep, experiments/experiments.py:47-49) on

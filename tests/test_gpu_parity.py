@@ -524,6 +524,17 @@ def test_m2l_forms_agree(eng, monkeypatch, name):
     # the direct form evaluates exp per node pair in fp32 (243 x 243 terms per far pair at 3^5 nodes, 1024 x 1024 at 4^5,
     # over the ~900 far boxes of a box in five dimensions), the separable tables are rounded once from fp64
     assert rel_l2(grouped, direct) < (2e-5 if name in ("uniform5_243", "uniform5_1024") else 5e-6)
+    if name in ("uniform4", "uniform5_243"):
+        # 3^4 and 3^5 grids: the cells that every child of a parent lists summed once per combination of sibling bits
+        # (m2l_shared_kernel, which the library takes by itself in 4-D beside the near field), the rest by the
+        # sibling-group kernel; against the sibling-group kernel alone
+        monkeypatch.delenv("F3M_M2L")
+        monkeypatch.setenv("F3M_M2L_SHARED", "1")
+        shared = plan.apply(dev(b)).cpu().numpy()
+        monkeypatch.setenv("F3M_M2L_SHARED", "0")
+        alone = plan.apply(dev(b)).cpu().numpy()
+        assert 0 < rel_l2(shared, alone) < 2e-6
+        assert rel_l2(shared, direct) < (2e-5 if name == "uniform5_243" else 5e-6)
 
 
 @pytest.mark.parametrize("name,parts", [("C1_uniform3", 2), ("C1_uniform3", 3), ("uniform4", 6), ("uniform5_243", 2)])
