@@ -200,11 +200,13 @@ void set_node_offsets(NodeSet &ns, float edge, hipStream_t s);
 void gather_points(const float *X, const int *perm, long long n, int d, float *pts, hipStream_t s, bool background = false);
 void gather_column(const float *b, const int *perm, long long n, int c, int col, float *bs, hipStream_t s);
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s);
-// ncol (1..4) neighbouring columns at once, one access per row; the scatter adds outs2 (same layout) if it is given
+// ncol (1..4) neighbouring columns at once, one access per row; the scatter adds outs2 (same layout) if it is given,
+// and to its one column the fixed-point sums of a symmetric near field (see SymSums) if those are given
+struct SymSums;
 void gather_columns(const float *b, const int *perm, long long n, int c, int col, int ncol, float *bs, long long bstride,
                     hipStream_t s, bool background = false);
 void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
-                     int ncol, float *out, hipStream_t s);
+                     int ncol, float *out, hipStream_t s, const SymSums *symsums = nullptr);
 
 // Results added straight into the caller's array instead of the sorted one: out[perm[i] * c + col + q] += value by a
 // hardware atomic addition.  The array is cleared before, and at most two values are added to an element (the near
@@ -217,6 +219,34 @@ struct DirectOut {
 // whether near_field would take this list in one launch of the matrix-pipe kernel with one wavefront per work item
 // (the condition for DirectOut: every target is then written by exactly one wavefront)
 bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList &list, float lcs, int nc);
+// The symmetric near field (one tree: K is symmetric and the lists name (A,B) exactly when they name (B,A)) evaluates the
+// tiles of a pair of boxes once and adds them in both directions.  The sums of the second direction reach a point from
+// many wavefronts in no fixed order, so they are added as 64-bit fixed-point numbers (integer addition is associative: the
+// result does not depend on the order) with one scale for the whole product: 2^61 over a power of two above
+// (number of sources) x (largest |weight|), which no sum can exceed.  One unit is below 1e-18 of that bound, far under
+// the rounding of the fp32 sums it joins.  absmax: bit pattern of the largest |weight| (written by sym_absmax; not finite:
+// the kernel adds floats atomically instead, the results are not finite anyway).
+struct SymSums {
+    long long *fix = nullptr;          // one per sorted point, cleared by the caller; null: not used
+    const unsigned *absmax = nullptr;
+    long long nsrc = 0;
+};
+// scale of the fixed-point sums as a power of two (0: weights not finite)
+__host__ __device__ inline float sym_scale(unsigned absmax_bits, long long nsrc)
+{
+    if (absmax_bits >= 0x7f800000u) return 0.f;
+    int lg = 0;
+    while ((1ll << lg) < nsrc) lg++;
+    const int e = (int)(absmax_bits >> 23) - 127 + 1;          // |w| < 2^e
+    int se = 61 - lg - e;
+    if (se > 127) se = 127;                                    // (tiny weights: coarser than it could be, still exact enough)
+    if (se < -126) se = -126;
+    return __builtin_bit_cast(float, (unsigned)(se + 127) << 23);
+}
+// whether near_field would take this list in the symmetric form, given a place for the sums of the second direction
+bool near_symmetric(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const PairList &list, float lcs, int nc);
+// absmax[0] = bit pattern of the largest |bs[i]|, i < n
+void sym_absmax(const float *bs, long long n, unsigned *absmax, hipStream_t s);
 // builds the table "box of every 32nd point" of a level now, on stream s, if it does not exist yet (kernels of
 // the near field and of L2P start from it; when those run on different streams the table must exist before)
 void ensure_box_table(const TreeLevel &lev, long long npoints, hipStream_t s);
@@ -227,7 +257,8 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 // prepare_only: build the tables of the list that are kept with the plan (tile table, source operands), launch nothing else
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc = 1, long long bstride = 0,
-                long long ostride = 0, bool only_list = false, bool prepare_only = false, const DirectOut *direct = nullptr);
+                long long ostride = 0, bool only_list = false, bool prepare_only = false, const DirectOut *direct = nullptr,
+                const SymSums *symsums = nullptr);
 void far_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &far,
                NodeSet &ns, const float *bs, float *outs, float lcs, int m2l_mode,
                float *mom_out, float *loc_out, hipStream_t s);

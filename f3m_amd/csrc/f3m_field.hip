@@ -105,26 +105,63 @@ void gather_column(const float *b, const int *perm, long long n, int c, int col,
 // beside the near field), q < NC, one store of NC floats per row
 template <int NC>
 __global__ void scatter_columns_kernel(const float *__restrict__ outs, const float *__restrict__ outs2, long long ostride,
-                                       const int *__restrict__ perm, long long n, int c, int col, float *__restrict__ out)
+                                       const int *__restrict__ perm, long long n, int c, int col, float *__restrict__ out,
+                                       SymSums sym)
 {
     long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     fvec<NC> row;
 #pragma unroll
-    for (int q = 0; q < NC; q++) row.v[q] = outs[q * ostride + i] + (outs2 ? outs2[q * ostride + i] : 0.f);
+    for (int q = 0; q < NC; q++) row.v[q] = outs[q * ostride + i];
+    if (NC == 1 && sym.fix != nullptr) {
+        const float scale = sym_scale(sym.absmax[0], sym.nsrc);
+        if (scale != 0.f) row.v[0] += (float)sym.fix[i] * (1.0f / scale);      // (a power of two: both steps round once in all)
+    }
+    if (outs2 != nullptr) {
+#pragma unroll
+        for (int q = 0; q < NC; q++) row.v[q] += outs2[q * ostride + i];
+    }
     *reinterpret_cast<fvec<NC> *>(out + (long long)perm[i] * c + col) = row;
 }
 void scatter_columns(const float *outs, const float *outs2, long long ostride, const int *perm, long long n, int c, int col,
-                     int ncol, float *out, hipStream_t s)
+                     int ncol, float *out, hipStream_t s, const SymSums *symsums)
 {
+    const SymSums sym = symsums ? *symsums : SymSums();
+    F3M_REQUIRE(sym.fix == nullptr || ncol == 1, 34, "fixed-point sums belong to a single column");
     switch (ncol) {
-    case 1: F3M_LAUNCH((scatter_columns_kernel<1>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
-    case 2: F3M_LAUNCH((scatter_columns_kernel<2>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
-    case 3: F3M_LAUNCH((scatter_columns_kernel<3>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
-    case 4: F3M_LAUNCH((scatter_columns_kernel<4>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out); break;
+    case 1: F3M_LAUNCH((scatter_columns_kernel<1>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out, sym); break;
+    case 2: F3M_LAUNCH((scatter_columns_kernel<2>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out, sym); break;
+    case 3: F3M_LAUNCH((scatter_columns_kernel<3>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out, sym); break;
+    case 4: F3M_LAUNCH((scatter_columns_kernel<4>), cdiv(n, 256), 256, 0, s, outs, outs2, ostride, perm, n, c, col, out, sym); break;
     default: throw Error(34, "1 to 4 columns at a time");
     }
     check_launch("scatter_columns");
+}
+// absmax[0] = max(absmax[0], bit pattern of the largest |bs[i]|): one atomic maximum per workgroup (the bit patterns of
+// non-negative floats order like the floats, NaN above infinity)
+__global__ void __launch_bounds__(256) absmax_kernel(const float *__restrict__ bs, long long n, unsigned *__restrict__ absmax)
+{
+    __shared__ unsigned wmax[4];
+    unsigned m = 0;
+    const long long n4 = n / 4, step = (long long)gridDim.x * blockDim.x;
+    struct alignas(16) u4 { unsigned x, y, z, w; };
+    const u4 *b4 = reinterpret_cast<const u4 *>(bs);                // (bs is the start of a device allocation)
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += step) {
+        const u4 v = b4[i];
+        m = max(max(m, v.x & 0x7fffffffu), max(max(v.y & 0x7fffffffu, v.z & 0x7fffffffu), v.w & 0x7fffffffu));
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)(n - 4 * n4))
+        m = max(m, __builtin_bit_cast(unsigned, bs[4 * n4 + threadIdx.x]) & 0x7fffffffu);
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (unsigned)wave_shfl_i((int)m, (int)(lane_id() ^ (unsigned)off)));
+    if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(absmax, max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+}
+void sym_absmax(const float *bs, long long n, unsigned *absmax, hipStream_t s)
+{
+    dev_fill(absmax, 0, sizeof(unsigned), s);
+    F3M_LAUNCH(absmax_kernel, (unsigned)std::min<long long>(cdiv(n, 4096), 1024), 256, 0, s, bs, n, absmax);
+    check_launch("absmax");
 }
 void scatter_column(const float *outs, const int *perm, long long n, int c, int col, float *out, hipStream_t s)
 {
@@ -573,13 +610,42 @@ struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floa
 // NC right-hand sides at once: the exponential of a pair is computed once and multiplies NC weights
 // (columns of bs, bstride apart; results to NC columns of outs, ostride apart).
 // FACT: the factored form (see near_slots): bs then holds the weights times exp2(-|y'|^2).
-template <int D, int TPW, int NC, bool FACT = false>
-__global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 && NC == 1) ? 5 : 2) near_g_kernel(
+//
+// SYM (one tree, X = Y: the list names (A,B) exactly when it names (B,A), and K is symmetric): a wavefront of box A takes
+// only the listed boxes B >= A.  The exponentials of a tile of B > A serve both directions: weighted with the sources'
+// weights they are summed over the rows into the targets of A as always, and weighted with the targets' weights they are
+// summed over the columns into the sources of B -- 16 more accumulators per lane, kept over the target tiles of the
+// work item, then added up across the 32 columns through the wavefront's own LDS block and added to the sums of B
+// atomically, as fixed-point numbers (SymSums): integer additions give the same result in any order.  Half the
+// exponentials per listed pair of points.
+constexpr int kSymRedStride = 33;                  // floats per row of the reduction block (32 columns + 1: no bank conflicts)
+__device__ __forceinline__ void atomic_add_i64(long long *p, long long v)
+{
+#ifdef F3M_CPU_EMU
+    *p += v;
+#else
+    atomicAdd(reinterpret_cast<unsigned long long *>(p), (unsigned long long)v);
+#endif
+}
+__device__ __forceinline__ void atomic_add_f32(float *p, float v)
+{
+#ifdef F3M_CPU_EMU
+    *p += v;
+#else
+    unsafeAtomicAdd(p, v);
+#endif
+}
+// (The symmetric form is held to 120 registers: four wavefronts per SIMD then leave 32 of its 512 free, as five of the
+// plain form's 96 do, and the small workgroups of the far field find room beside a running near field; at 128 they
+// wait for its end.)
+template <int D, int TPW, int NC, bool FACT, bool SYM>
+__device__ __forceinline__ void near_g_body(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
-    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
+    const int *__restrict__ offy, const int *__restrict__ celly, const Geo &geoy, float edgey,
     const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
-    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout)
+    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, const DirectOut &dout,
+    const SymSums &symsums)
 {
     constexpr int C = D + 2;                        // coordinates, the source's -|y'|^2, the target's -|x''|^2
     constexpr int NS = near_insts(D, FACT);
@@ -605,18 +671,37 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
     const int x0 = offx[bx] + (wid - tileoff[slot]) * (TPW * 32), x1 = offx[bx + 1];
     int nlive = (x1 - x0 + 31) / 32;                 // tiles with targets (uniform per wavefront)
     if (nlive > TPW) nlive = TPW;
-    float xr[TPW][D];
+    float xr[SYM ? 1 : TPW][D];                      // (SYM: read again at every new anchor, the registers are needed elsewhere)
+    if constexpr (!SYM) {
 #pragma unroll
-    for (int q = 0; q < TPW; q++) {
-        const int i = x0 + q * 32 + col;
+        for (int q = 0; q < TPW; q++) {
+            const int i = x0 + q * 32 + col;
 #pragma unroll
-        for (int k = 0; k < D; k++) xr[q][k] = (i < x1) ? xs[(long long)k * N + i] : 0.f;
+            for (int k = 0; k < D; k++) xr[q][k] = (i < x1) ? xs[(long long)k * N + i] : 0.f;
+        }
     }
     float acc[TPW][NC];
 #pragma unroll
     for (int q = 0; q < TPW; q++)
 #pragma unroll
         for (int c = 0; c < NC; c++) acc[q][c] = 0.f;
+    static_assert(!SYM || (NC == 1 && !FACT), "the symmetric form takes one column and the plain exponent");
+    // SYM: the wavefront's LDS block: 32 rows of the column reduction, then the weights of its targets (one tree: sources
+    // and targets are the same points in the same order), kept there to spare registers
+    constexpr int kSymBlock = 32 * kSymRedStride + TPW * 32;
+    __shared__ float red_all[SYM ? kNearWavesPerBlock * kSymBlock : 1];
+    float *const red = red_all + (SYM ? (threadIdx.x >> 6) * kSymBlock : 0);
+    float *const btl = red + 32 * kSymRedStride;
+    float fixscale = 0.f;                            // SYM: scale of the fixed-point sums (0: weights not finite)
+    if constexpr (SYM) {
+#pragma unroll
+        for (int q = 0; q < TPW; q++) {
+            const int i = x0 + q * 32 + col;
+            if (half == 0) btl[q * 32 + col] = i < x1 ? bs[i] : 0.f;
+        }
+        wave_sync();
+        fixscale = sym_scale(symsums.absmax[0], symsums.nsrc);
+    }
     const int m0 = rowptr[bx], m1 = rowptr[bx + 1];
     // slice of this wavefront, in 32-source tiles counted along the whole row: [tlo, thi)
     int tlo = 0, thi = 0x7fffffff;
@@ -664,9 +749,12 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
           for (int k = 0; k < D; k++) {
               const int cl = celly[(long long)byv * D + k];
               pcv[k] = cl >> 1;
-              cyv[k] = near_anchor(geoy, edgey, cl, k);
+              if constexpr (!SYM) cyv[k] = near_anchor(geoy, edgey, cl, k);   // (SYM reads the cell again at a new anchor: registers)
           }
       }
+      // SYM: boxes before this one are left to their own wavefronts (each stays in the walk as a run without sources)
+      const bool mine = !SYM || byv >= bx;
+      if (SYM && !mine) { s0v = 0; s1v = 0; }
       const int mcnt = min(64, m1 - mb);
       // same: under the parent cell of the lane before (same anchor, the target operands stay as they are);
       // cont: also next to it in memory, i.e. continues its run
@@ -676,7 +764,9 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
 #pragma unroll
       for (int k = 0; k < D; k++) same = (wave_shfl_i(pcv[k], before) == pcv[k]) && same;
       const int byprev = wave_shfl_i(byv, before);   // by every lane: an exchange inside a branch sees the branch's lanes only
-      const bool cont = same && byprev + 1 == byv;
+      if (SYM) same = same && mine && byprev >= bx;  // the operands of a skipped box were never set up
+      // (SYM: the box itself is a run of its own, it takes one direction only)
+      const bool cont = same && byprev + 1 == byv && !(SYM && (byprev == bx || byv == bx));
       unsigned long long heads = wave_ballot(mi < m1 && !cont);
       const unsigned long long anchors = wave_ballot(mi < m1 && !same);
       while (heads) {
@@ -698,6 +788,9 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
         // keep the loop over the tiles of the run off the vector ALU)
         s0 = wave_uniform(s0);
         s1 = wave_uniform(s1);
+        const int byhead = SYM ? wave_readlane(byv, mj) : 0;
+        if (SYM && byhead < bx) continue;            // a skipped box (uniform)
+        const bool both = SYM && byhead != bx;       // uniform: the tiles of this run serve both directions
         float run[TPW][NC];                           // factored form: the sums of this run
 #pragma unroll
         for (int q = 0; q < TPW; q++)
@@ -708,7 +801,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
         if (new_anchor) {
         float cy[D];
 #pragma unroll
-        for (int k = 0; k < D; k++) cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
+        for (int k = 0; k < D; k++) {
+            if constexpr (SYM) cy[k] = near_anchor(geoy, edgey, celly[(long long)byhead * D + k], k);
+            else cy[k] = __builtin_bit_cast(float, wave_readlane(__builtin_bit_cast(int, cyv[k]), mj));
+        }
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
             if (q >= nlive) continue;                 // uniform per wavefront: tiles without targets need no operands
@@ -719,7 +815,10 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             for (int k = 0; k < C; k++) {
                 float v = 1.f;
                 if (k < D) {
-                    v = ok ? sc * (xr[q][k] - cy[k]) : 0.f;
+                    float xv;
+                    if constexpr (SYM) xv = ok ? xs[(long long)k * N + x0 + q * 32 + col] : 0.f;
+                    else xv = xr[q][k];
+                    v = ok ? sc * (xv - cy[k]) : 0.f;
                     nx2 -= v * v;
                 } else if (k == D + 1) {
                     v = nx2;
@@ -774,7 +873,49 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                     }
                 }
             };
-            if (nlive == TPW) {
+            if (both) {
+                if constexpr (SYM) {
+                    float sacc[16];                  // sums over this lane's column of every target tile, per source row
+#pragma unroll
+                    for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+                    auto tile2 = [&](int q) {
+                        const float btq = btl[q * 32 + col];
+                        f32x16 t;
+#pragma unroll
+                        for (int r = 0; r < 16; r++) t[r] = 0.f;
+#pragma unroll
+                        for (int n = 0; n < NS; n++) t = mfma_32x32x16_f16(a[n], bop[q][n], t);
+#pragma unroll
+                        for (int r = 0; r < 16; r++) {
+                            const float e = fast_exp2(t[r]);
+                            acc[q][0] = fmaf(e, bq[0][r], acc[q][0]);
+                            sacc[r] = fmaf(e, btq, sacc[r]);
+                        }
+                    };
+                    if (nlive == TPW) {              // the usual case, free of branches (see below)
+#pragma unroll
+                        for (int q = 0; q < TPW; q++) tile2(q);
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < TPW; q++)
+                            if (q < nlive) tile2(q);     // uniform per wavefront
+                    }
+                    // across the 32 columns: element r of half h is source row 8(r/4) + 4h + r%4 of the tile
+#pragma unroll
+                    for (int r = 0; r < 16; r++) red[(half * 16 + r) * kSymRedStride + col] = sacc[r];
+                    wave_sync();
+                    const int rho = ((col >> 2) & 1) * 16 + 4 * (col >> 3) + (col & 3);   // where source row `col` sits
+                    float sum = 0.f;
+#pragma unroll
+                    for (int k = 0; k < 16; k++) sum += red[rho * kSymRedStride + 16 * half + k];
+                    wave_sync();
+                    sum += wave_shfl_xor_f(sum, 32);
+                    if (half == 0 && j0 + col < s1) {
+                        if (fixscale != 0.f) atomic_add_i64(symsums.fix + j0 + col, llrintf(sum * fixscale));
+                        else atomic_add_f32(outs + j0 + col, sum);
+                    }
+                }
+            } else if (nlive == TPW) {
                 // the usual case, free of branches: the compiler may start the matrix products of the
                 // next tiles while the vector ALU works on the exponentials of this one
 #pragma unroll
@@ -801,11 +942,43 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
             float total = acc[q][c] + wave_shfl_xor_f(acc[q][c], 32);
             if (half == 0 && i < x1) {
                 if (nsplit > 1) part[(((long long)slice * NC + c) * nitems + wid) * (TPW * 32) + q * 32 + col] = total;
+                else if (SYM && fixscale == 0.f) atomic_add_f32(outs + c * ostride + i, total);
                 else if (dout.out == nullptr) outs[c * ostride + i] += total;
                 else if (c < dout.ncol) direct_add(dout, i, c, total);
             }
         }
     }
+}
+
+template <int D, int TPW, int NC, bool FACT = false>
+__global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 && NC == 1) ? 5 : 2) near_g_kernel(
+    const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
+    long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
+    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
+    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout)
+{
+    near_g_body<D, TPW, NC, FACT, false>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+                                         rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, SymSums());
+}
+
+// the symmetric form: four target tiles per wavefront, one column, the plain exponent
+#ifdef F3M_CPU_EMU
+#define F3M_NEAR_SYM_REGS
+#else
+#define F3M_NEAR_SYM_REGS __attribute__((amdgpu_num_vgpr(60)))      // counted in pairs on this target: 120 registers
+#endif
+template <int D>
+__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
+    const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
+    long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
+    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
+    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
+    SymSums symsums)
+{
+    near_g_body<D, 4, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+                                      rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
 // outs += the slices of a split near field, in slice order; one thread per target slot of a work item
@@ -955,9 +1128,24 @@ bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList
     return items_exact >= 16384;          // fewer work items: the lists are cut into slices with partial sums
 }
 
+// Whether near_field takes a list in the symmetric form (see near_g_kernel): one tree (then every list of the plan names
+// (A,B) exactly when it names (B,A): the class of a pair depends on the distance of the centres and on the sum of the
+// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to three dimensions, four target
+// tiles per wavefront.  F3M_NEAR_SYM=0 turns it off.
+bool near_symmetric(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const PairList &list, float lcs, int nc)
+{
+    if (&tx != &ty || nc != 1 || d > 3 || list.n == 0) return false;
+    if (const char *e = getenv("F3M_NEAR_SYM")) if (atoi(e) == 0) return false;
+    if (!near_on_matrix_pipe(d, lcs, lx.edge) || near_factored(d, lcs, lx.edge)) return false;
+    int tpw;
+    long long items_exact;
+    near_shape(tx, lx, list, nc, tpw, items_exact);
+    return tpw == 4;                     // (lists cut into slices, see near_field, take the plain form)
+}
+
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
                 const float *bs, float *outs, float lcs, hipStream_t s, int nc, long long bstride, long long ostride,
-                bool only_list, bool prepare_only, const DirectOut *direct)
+                bool only_list, bool prepare_only, const DirectOut *direct, const SymSums *symsums)
 {
     if (list.n == 0) return;
     F3M_REQUIRE(nc == 1 || nc == 2 || nc == 4, 34, "near field takes 1, 2 or 4 columns at a time");
@@ -1024,6 +1212,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         const NearOps src = build_near_operands(d, ty, ly, sc, near_factored(d, lcs, ly.edge), only_list ? &list : nullptr, s);
         const bool fact = src.ey != nullptr;
         if (prepare_only) return;
+        const bool sym = !fact && symsums != nullptr && symsums->fix != nullptr && near_symmetric(d, tx, lx, ty, list, lcs, nc);
+        F3M_REQUIRE(!(sym && direct), 35, "direct output and the symmetric near field exclude each other");
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
         // Few targets against long lists (the transposed product of a tall kernel matrix): too few work
@@ -1058,7 +1248,15 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(),
                        list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);
         };
+        auto go_sym = [&](auto kern) {
+            F3M_LAUNCH(kern, ngrid, kNearWavesPerBlock * 64, 0, s, tx.pts.get(), tx.n, src.ops, stride, wsrc, wstride, outs,
+                       ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(),
+                       list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout, *symsums);
+        };
 #define F3M_NEAR_FORM(DD, FF)                                                                                         \
+    if constexpr (DD <= 3 && !FF) {                                                                                   \
+        if (sym && nsplit == 1) { go_sym(near_sym_kernel<DD>); break; }                                     \
+    }                                                                                                                 \
     if (tpw == 5) go(near_g_kernel<DD, 5, 1, FF>);                                                                    \
     else if (nc == 4) go(near_g_kernel<DD, 4, 4, FF>);                                                                \
     else if (nc == 2) go(near_g_kernel<DD, 4, 2, FF>);                                                                \

@@ -734,6 +734,21 @@ __device__ inline void child_bounds_body(unsigned blk, const BoundsArgs &a)
     int q = (int)(nat >> a.d);
     uint32_t target = (a.prefix_prev[q] << a.d) | (uint32_t)(nat & ((1 << a.d) - 1));
     int lo = a.off_prev[q], hi = a.off_prev[q + 1];
+    // first position in [lo, hi) whose key is not below the target.  The range is cut in eight per step, seven probes
+    // whose loads do not wait for each other, instead of in two: the kernel's time is the chain of dependent loads
+    // (23 steps of ~1 us in a parent of 1e7 points, now 8).
+    while (hi - lo > 8) {
+        const int step = (hi - lo) >> 3;
+        bool below[7];
+#pragma unroll
+        for (int u = 0; u < 7; u++) below[u] = (a.keys[lo + (u + 1) * step] >> a.shift) < target;
+        int nb = 0;                                   // probes below the target (they are a prefix: the keys are sorted)
+#pragma unroll
+        for (int u = 0; u < 7; u++) nb += below[u] ? 1 : 0;
+        const int nlo = nb ? lo + nb * step + 1 : lo;
+        hi = nb < 7 ? lo + (nb + 1) * step : hi;
+        lo = nlo;
+    }
     while (lo < hi) {
         int mid = lo + ((hi - lo) >> 1);
         if ((a.keys[mid] >> a.shift) < target) lo = mid + 1; else hi = mid;

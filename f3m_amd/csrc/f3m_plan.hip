@@ -95,6 +95,8 @@ struct f3m_plan {
     // one-shot products: the first column group of b, already in sorted order (gathered while the lists were built)
     DBuf<float> early_bs;
     DBuf<float> early_outs, early_outs_far;   // the result arrays of that column group, cleared beside the last level's lists
+    DBuf<long long> early_symfix;             // with them, for a single column on one tree: the cleared fixed-point sums of the
+    DBuf<unsigned> early_symmax;              // symmetric near field and the largest |weight| (SymSums)
     const float *early_b = nullptr;
     int early_c = 0, early_ncol = 0;
     float *early_out = nullptr;               // the caller's result array, cleared beside the last level's lists (N x early_c floats)
@@ -403,6 +405,12 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
                     dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
                     dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
+                    if (sym && P->early_c == 1 && d <= 3) {     // (wherever near_symmetric may say yes)
+                        P->early_symfix.reset((size_t)P->N);
+                        P->early_symmax.reset(1);
+                        dev_fill(P->early_symfix.get(), 0, sizeof(long long) * (size_t)P->N, side_stream().stream);
+                        sym_absmax(P->early_bs.get(), P->M, P->early_symmax.get(), side_stream().stream);
+                    }
                     if (out_early != nullptr) {     // and the caller's array, for a product that adds its results straight into it
                         dev_fill(out_early, 0, sizeof(float) * (size_t)P->N * P->early_c, side_stream().stream);
                         P->early_out = out_early;
@@ -638,7 +646,8 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 // every column group of this product (four columns while three or more are left, then two or one)
                 for (int left = c; left > 0 && direct;) {
                     const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);
-                    direct = near_single_pass(P->d, TX, TX.lev[k], *l, P->lcs, nc);
+                    direct = near_single_pass(P->d, TX, TX.lev[k], *l, P->lcs, nc) &&
+                             !near_symmetric(P->d, TX, TX.lev[k], TY, *l, P->lcs, nc);
                     left -= std::min(nc, left);
                 }
             }
@@ -675,12 +684,43 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
     // column's far field) can take the place of the previous one's: the need does not grow with the number of columns,
     // and the first group, which has the most columns, is the one that decides whether the product fits -- before
     // anything has been written to `out`.
+    // The symmetric near field (one tree, a single column: half the exponentials) adds the sums of its second direction
+    // as fixed-point numbers into an array of their own, which the scatter pass folds in.  With an arena only where
+    // that array is a small part of it (a product that fits without must not be refused because of it).
+    DBuf<long long> symfix;
+    DBuf<unsigned> symmax;
     const size_t group_mark = arena_mark();
     for (int col = 0; col < c;) {
         arena_rewind(group_mark);
         const int left = c - col;
         const int nc = left >= 3 ? 4 : (left == 2 ? 2 : 1);   // columns of this pass (past `left`: zero weights)
         const int ncol = std::min(nc, left);
+        bool use_sym = false;
+        if (P->symmetric && nc == 1) {
+            for (int k = 1; k <= depth && !use_sym; k++)
+                use_sym = near_symmetric(P->d, TX, TX.lev[k], TY, small_of(k), P->lcs, nc) ||
+                          (k == depth && near_symmetric(P->d, TX, TX.lev[k], TY, keep_of(k), P->lcs, nc));
+            if (g_arena != nullptr && sizeof(long long) * (size_t)NT > (g_arena->cap - g_arena->used) / 4) use_sym = false;
+        }
+        // (prepared while the plan was built, together with this group's weights and cleared result arrays)
+        const bool sym_early = use_sym && col == 0 && !transposed && P->early_b == b && P->early_c == c && P->early_ncol == ncol &&
+                               P->early_bs.size() > 0 && P->early_outs.size() > 0 && P->early_symfix.size() > 0;
+        SymSums symsums;
+        if (sym_early) {
+            std::swap(symfix, P->early_symfix);
+            std::swap(symmax, P->early_symmax);
+        } else if (use_sym) {
+            symfix.reset((size_t)NT);
+            symmax.reset(1);
+        }
+        P->early_symfix.free();
+        P->early_symmax.free();
+        if (use_sym) {
+            symsums.fix = symfix.get();
+            symsums.absmax = symmax.get();
+            symsums.nsrc = NS;
+        }
+        const SymSums *sym = use_sym ? &symsums : nullptr;
         {
             Scope sc(kPerm, s);
             bool cleared = false;
@@ -702,6 +742,10 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             if (!cleared && !direct) {
                 dev_fill(outs.get(), 0, sizeof(float) * (size_t)ostride * nc, s);
                 if (overlap) dev_fill(outs_far.get(), 0, sizeof(float) * (size_t)ostride * ncol, s);
+            }
+            if (use_sym && !sym_early) {
+                dev_fill(symfix.get(), 0, sizeof(long long) * (size_t)NT, s);
+                sym_absmax(bs.get(), NS, symmax.get(), s);
             }
         }
         // Every temporary that is given back while this column group is being queued is parked until the streams
@@ -730,7 +774,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 for (int k = 1; k <= depth; k++) {
                     // F3M_src/n_tree.cu:1018-1051: exact sums of the small pairs, then the far field
                     near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
-                               bstride, ostride, /*only_list=*/k < depth || deepest_only_list, false, dn);
+                               bstride, ostride, /*only_list=*/k < depth || deepest_only_list, false, dn, sym);
                     const size_t mark = arena_mark();
                     for (int q = 0; q < ncol; q++) {
                         arena_rewind(mark);
@@ -739,14 +783,14 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 }
                 // F3M_src/n_tree.cu:1092-1094: what is still "keep" after the last division is summed exactly
                 near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
-                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
+                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn, sym);
             } else {
                 // F3M_src/n_tree.cu:1018-1051 and :1092-1094: exact sums of the small pairs of every level and of what
                 // is still "keep" after the last division
                 near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], small_of(depth), bs.get(), outs.get(), P->lcs, s, nc,
-                           bstride, ostride, /*only_list=*/deepest_only_list, false, dn);
+                           bstride, ostride, /*only_list=*/deepest_only_list, false, dn, sym);
                 near_field(P->d, TX, TX.lev[depth], TY, TY.lev[depth], keep_of(depth), bs.get(),
-                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn);
+                           outs.get(), P->lcs, s, nc, bstride, ostride, false, false, dn, sym);
                 if (overlap) {       // (queued after the long launches: the host needs a while for these many small kernels)
                     for (int k = 1; k < depth; k++)
                         near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs,
@@ -756,7 +800,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
                 }
                 for (int k = 1; k < depth; k++)
                     near_field(P->d, TX, TX.lev[k], TY, TY.lev[k], small_of(k), bs.get(), outs.get(), P->lcs, s, nc,
-                               bstride, ostride, /*only_list=*/true, false, dn);
+                               bstride, ostride, /*only_list=*/true, false, dn, sym);
             }
             // the far field: beside the near field on the second stream into its own array, or after it on the one
             // stream; either way a result is (near sums) + (far sum)
@@ -779,7 +823,7 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             }
             Scope sc(kPerm, s);
             if (!direct)
-                scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s);
+                scatter_columns(outs.get(), overlap ? outs_far.get() : nullptr, ostride, TX.perm.get(), NT, c, col, ncol, out, s, sym);
         }
         col += ncol;
     }

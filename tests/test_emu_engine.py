@@ -347,6 +347,36 @@ def test_mfma_near_field(oracle, monkeypatch):
                 assert np.array_equal(eng.apply(b[:, col:col + 1]), got[:, col:col + 1])
 
 
+@pytest.mark.parametrize("name", ["uniform3", "normal2", "uniform1", "dups_faces"])
+def test_symmetric_near_field(oracle, monkeypatch, name):
+    """One tree, one column: the tiles of a pair of boxes are evaluated once and added in both directions, the second
+    one through the wavefront's LDS block and as fixed-point sums.  (F3M_SPLIT_TARGET=1: one wavefront per work item on
+    these tiny clouds, which the symmetric form needs.)  Against the oracle, against the plain form (close, and not the
+    same bits: the symmetric kernel did run), and with a weight that is not finite (the kernel then adds floats)."""
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    rng = np.random.default_rng(9)
+    X, _ = _cloud(name, rng)
+    X = X[:1500]
+    b = rng.standard_normal((X.shape[0], 1)).astype(f32)
+    prm = dict(ls=0.4, min_points=50, nr_of_interpolation=8, small_field_points=30)
+    sym = ee.kmvm(X, None, b, **prm)
+    assert rel_l2(sym, oracle.kmvm(X, None, b, **prm)) < 1e-5
+    assert np.array_equal(ee.kmvm(X, None, b, **prm), sym)
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    plain = ee.kmvm(X, None, b, **prm)
+    assert 0 < rel_l2(sym, plain) < 1e-6
+    if name == "uniform3":
+        b[7] = np.inf
+        plain = ee.kmvm(X, None, b, **prm)
+        monkeypatch.setenv("F3M_NEAR_SYM", "1")
+        sym = ee.kmvm(X, None, b, **prm)
+        assert not np.isfinite(sym[7]).any() and not np.isfinite(plain[7]).any()
+        both = np.isfinite(sym[:, 0]) & np.isfinite(plain[:, 0])        # (the far field carries the weight to most targets)
+        assert np.array_equal(np.isfinite(sym), np.isfinite(plain))
+        assert not both.any() or rel_l2(sym[both], plain[both]) < 1e-5
+
+
 @pytest.mark.parametrize("form", ["0", "1"])
 def test_mfma_near_field_five_dimensions(oracle, monkeypatch, form):
     """d = 5: two matrix instructions per tile in the plain form, one in the factored form (the weights carry

@@ -741,6 +741,98 @@ def test_one_stream_and_two_streams_give_the_same_bits(eng, monkeypatch, name):
         assert np.array_equal(one, two) and np.array_equal(one_plan, two)
 
 
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "uniform2", "uniform1", "lattice_faces_dups", "uniform3_varcomp"])
+def test_symmetric_near_field_against_oracle(eng, oracle, monkeypatch, name):
+    """One tree and one column: the near field evaluates the tiles of a pair of boxes once and adds them in both
+    directions (half the exponentials), the second direction as fixed-point sums.  On these small clouds the lists
+    would be cut into slices, which take the plain form; F3M_SPLIT_TARGET=1 keeps one wavefront per work item, so the
+    symmetric kernel runs.  Against the oracle to 1e-5 level by level and for the product; against the plain form to
+    1e-6 (and not the same bits: the symmetric kernel did run); the same bits when repeated."""
+    print("case symmetric near field", name, flush=True)
+    rng = np.random.default_rng(77)
+    X, Y, prm = clouds(name, rng)
+    assert Y is None
+    b = rng.standard_normal((X.shape[0], 1)).astype(f32)
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    Xd, bd = dev(X), dev(b)
+    sym = eng.kmvm(Xd, None, bd, **prm).cpu().numpy()
+    ora = oracle.Plan(X, None, **prm)
+    assert rel_l2(sym, ora.apply(b)) < 1e-5
+    plan = eng.Plan(Xd, None, **prm)
+    for rep in range(3):
+        assert np.array_equal(plan.apply(bd).cpu().numpy(), sym), rep
+        assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym), rep
+    plan.close()
+    monkeypatch.setenv("F3M_OVERLAP", "0")
+    assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym)
+    monkeypatch.delenv("F3M_OVERLAP")
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    plain = eng.kmvm(Xd, None, bd, **prm).cpu().numpy()
+    assert 0 < rel_l2(sym, plain) < 1e-6
+
+
+def test_symmetric_near_field_at_a_size_that_takes_it_by_itself(eng, monkeypatch):
+    """2.6e6 uniform points: 20480 work items, the symmetric form is the default.  Same bits from the one-shot call, a
+    kept plan and repetitions of both (integer additions commute); within 1e-6 of the plain form and within 1e-5 of
+    the fp32 exact sums on the rows of a few boxes."""
+    print("case symmetric near field, default path", flush=True)
+    import torch
+    rng = np.random.default_rng(43)
+    n = 2_600_000
+    X = dev(rng.random((n, 3), dtype=f32))
+    b = dev(rng.standard_normal((n, 1)).astype(f32))
+    first = eng.kmvm(X, None, b, ls=1.0)
+    plan = eng.Plan(X, None, ls=1.0)
+    for rep in range(3):
+        assert torch.equal(plan.apply(b), first), rep
+        assert torch.equal(eng.kmvm(X, None, b, ls=1.0), first), rep
+    plan.close()
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    plain = eng.kmvm(X, None, b, ls=1.0)
+    rel = float((first - plain).norm() / plain.norm())
+    assert 0 < rel < 1e-6
+    rows = torch.from_numpy(rng.choice(n, 2000, replace=False)).cuda()
+    exact = eng.exact_f64(X[rows].double(), X.double(), b.double(), 1.0)
+    err = lambda o: float((o[rows].double() - exact).norm() / exact.norm())
+    assert err(first) < 1e-4 and err(first) < 1.05 * err(plain) + 1e-7
+
+
+def test_symmetric_near_field_weights_of_any_size(eng, monkeypatch):
+    """The fixed-point sums are scaled by the largest |weight| of the product.  Weights of 2^83 beside weights of
+    order one, tiny weights (2^-100), and weights that are all zero: within 1e-6 of the plain form relative to the
+    largest result.  A weight that is not finite: the kernel adds floats instead, and the targets near that source are
+    not finite in either form."""
+    print("case symmetric near field, weights", flush=True)
+    rng = np.random.default_rng(45)
+    n = 60000
+    X = rng.random((n, 3), dtype=f32)
+    Xd = dev(X)
+    prm = dict(ls=0.5)
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    cases = {"mixed": rng.standard_normal((n, 1)).astype(f32), "tiny": (rng.standard_normal((n, 1)) * 2.0 ** -100).astype(f32),
+             "zero": np.zeros((n, 1), f32)}
+    cases["mixed"][::1000] *= f32(2.0 ** 83)
+    for what, b in cases.items():
+        monkeypatch.setenv("F3M_NEAR_SYM", "1")
+        sym = eng.kmvm(Xd, None, dev(b), **prm).cpu().numpy()
+        monkeypatch.setenv("F3M_NEAR_SYM", "0")
+        plain = eng.kmvm(Xd, None, dev(b), **prm).cpu().numpy()
+        assert np.isfinite(sym).all(), what
+        scale = np.abs(plain).max()
+        assert np.abs(sym.astype(np.float64) - plain).max() <= 1e-6 * scale, what
+    b = rng.standard_normal((n, 1)).astype(f32)
+    b[12345] = np.inf
+    monkeypatch.setenv("F3M_NEAR_SYM", "1")
+    sym = eng.kmvm(Xd, None, dev(b), **prm).cpu().numpy()
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    plain = eng.kmvm(Xd, None, dev(b), **prm).cpu().numpy()
+    close = np.linalg.norm(X - X[12345], axis=1) < 0.01
+    assert close.sum() > 1 and not np.isfinite(sym[close]).any() and not np.isfinite(plain[close]).any()
+    both = np.isfinite(sym[:, 0]) & np.isfinite(plain[:, 0])            # (the far field carries the weight to most targets)
+    assert np.array_equal(np.isfinite(sym), np.isfinite(plain))
+    assert not both.any() or rel_l2(sym[both], plain[both]) < 1e-5
+
+
 @pytest.mark.parametrize("c", [1, 3, 6])
 def test_results_added_straight_into_the_output_array(eng, monkeypatch, c):
     """Where the near field is one launch with one wavefront per work item and the far field is evaluated once, both
@@ -755,6 +847,9 @@ def test_results_added_straight_into_the_output_array(eng, monkeypatch, c):
     n = 2_600_000                                   # 4096 boxes of ~635 points: 20480 work items of 128 targets
     X = dev(rng.random((n, 3), dtype=f32))
     b = dev(rng.standard_normal((n, c)).astype(f32))
+    if c == 1:
+        # a single column on one tree would take the symmetric near field, whose sums go through the scatter pass
+        monkeypatch.setenv("F3M_NEAR_SYM", "0")
     monkeypatch.setenv("F3M_DIRECT", "0")
     want = eng.kmvm(X, None, b, ls=1.0)
     monkeypatch.setenv("F3M_DIRECT", "2")           # fails if the product does not take the direct path
