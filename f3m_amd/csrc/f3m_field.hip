@@ -112,14 +112,12 @@ __global__ void scatter_columns_kernel(const float *__restrict__ outs, const flo
     if (i >= n) return;
     fvec<NC> row;
 #pragma unroll
-    for (int q = 0; q < NC; q++) row.v[q] = outs[q * ostride + i];
+    for (int q = 0; q < NC; q++) row.v[q] = outs[q * ostride + i] + (outs2 ? outs2[q * ostride + i] : 0.f);
+    // the fixed-point sums come last: the far field's share is in outs already when everything ran on one stream, and
+    // the bits must not depend on that
     if (NC == 1 && sym.fix != nullptr) {
         const float scale = sym_scale(sym.absmax[0], sym.nsrc);
-        if (scale != 0.f) row.v[0] += (float)sym.fix[i] * (1.0f / scale);      // (a power of two: both steps round once in all)
-    }
-    if (outs2 != nullptr) {
-#pragma unroll
-        for (int q = 0; q < NC; q++) row.v[q] += outs2[q * ostride + i];
+        if (scale != 0.f) row.v[0] += (float)sym.fix[i] * (1.0f / scale);      // (a power of two: the two steps round once in all)
     }
     *reinterpret_cast<fvec<NC> *>(out + (long long)perm[i] * c + col) = row;
 }
@@ -1106,7 +1104,8 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 
 // the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
 // the list, the exact number of work items (else -1)
-static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact)
+static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact,
+                       bool sym = false)
 {
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
     const long long tiles = (avg_points + 31) / 32;
@@ -1116,6 +1115,7 @@ static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list
     // then.  N=1e7: the fastest products 39.8 ms against 40.9, but single products up to 48.9 and means of 40.8-42.8
     // against a steady 41.0 with four tiles, 115 registers.  Four it is.)
     if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
+    if (sym) tpw = 4;                     // the symmetric form has four tiles (and saves more than the fifth tile does)
     items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
 }
 
@@ -1130,17 +1130,14 @@ bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList
 
 // Whether near_field takes a list in the symmetric form (see near_g_kernel): one tree (then every list of the plan names
 // (A,B) exactly when it names (B,A): the class of a pair depends on the distance of the centres and on the sum of the
-// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to three dimensions, four target
-// tiles per wavefront.  F3M_NEAR_SYM=0 turns it off.
+// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to three dimensions.
+// F3M_NEAR_SYM=0 turns it off.
 bool near_symmetric(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const PairList &list, float lcs, int nc)
 {
     if (&tx != &ty || nc != 1 || d > 3 || list.n == 0) return false;
     if (const char *e = getenv("F3M_NEAR_SYM")) if (atoi(e) == 0) return false;
-    if (!near_on_matrix_pipe(d, lcs, lx.edge) || near_factored(d, lcs, lx.edge)) return false;
-    int tpw;
-    long long items_exact;
-    near_shape(tx, lx, list, nc, tpw, items_exact);
-    return tpw == 4;                     // (lists cut into slices, see near_field, take the plain form)
+    return near_on_matrix_pipe(d, lcs, lx.edge) && !near_factored(d, lcs, lx.edge);
+    // (lists cut into slices, see near_field, take the plain form all the same)
 }
 
 void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const TreeLevel &ly, const PairList &list,
@@ -1171,7 +1168,11 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     int tpw;
     long long items_exact;
-    near_shape(tx, lx, list, nc, tpw, items_exact);
+    // (the shape follows from what the list could take, not from whether this call brings a place for the fixed-point
+    // sums: the tile table of a list is then the same for every call)
+    const bool sym_capable = near_symmetric(d, tx, lx, ty, list, lcs, nc);
+    const bool sym_wanted = sym_capable && symsums != nullptr && symsums->fix != nullptr;
+    near_shape(tx, lx, list, nc, tpw, items_exact, sym_capable);
     // From five dimensions on the work items are long and their lists differ a lot in length (3^5 boxes around
     // an interior box, 2^5 around a corner): the boxes with the longest lists go first, which shortens the
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
@@ -1212,7 +1213,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         const NearOps src = build_near_operands(d, ty, ly, sc, near_factored(d, lcs, ly.edge), only_list ? &list : nullptr, s);
         const bool fact = src.ey != nullptr;
         if (prepare_only) return;
-        const bool sym = !fact && symsums != nullptr && symsums->fix != nullptr && near_symmetric(d, tx, lx, ty, list, lcs, nc);
+        const bool sym = !fact && sym_wanted;
         F3M_REQUIRE(!(sym && direct), 35, "direct output and the symmetric near field exclude each other");
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
