@@ -24,8 +24,8 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP32_TFLOPS = 157.3      # MI355X fp32 peak (vector or matrix pipe)
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "near_g_kernel_n1e7_uniform3d_counters.md")
-STATS_PROFILE = os.path.join(ROOT, "profiles", "near_g_kernel_n1e7_uniform3d_kernel_stats.md")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "near_sym_kernel_n1e7_uniform3d_counters.md")
+STATS_PROFILE = os.path.join(ROOT, "profiles", "near_sym_kernel_n1e7_uniform3d_kernel_stats.md")
 ORACLE_ERRORS = os.path.join(ROOT, "tests", "golden", "fullsize_oracle_errors.json")
 CRITICAL_STAGES = ("plan", "near", "perm")          # on the caller's stream; the far field runs beside the near field
 
@@ -45,7 +45,7 @@ def profiled_near_launch_us():
     """average duration of the near-field launch in the committed rocprofv3 kernel trace of this command (the first
     table: default two-stream mode), microseconds"""
     try:
-        m = re.search(r"\|\s*f3m::near_g_kernel<3, 4, 1>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
+        m = re.search(r"\|\s*f3m::near_sym_kernel<3>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
         return float(m.group(1)) if m else None
     except OSError:
         return None
@@ -121,17 +121,38 @@ def run_config(name, n, steps, warmup, subsample, keep_inputs=False, nodes=None,
     work = plan.work()
     depth = plan.depth
     nbx = plan.level_sizes(depth)["nbx"] if depth else 1
+    # One tree, one column, up to three dimensions: the library's near field takes the symmetric form, which evaluates a
+    # listed pair of boxes (A, B), A != B, once for both directions.  Point pairs inside one box (A, A) are evaluated
+    # one by one as before: their number comes from the lists.
+    symmetric = Y is None and b.shape[1] == 1 and d <= 3 and os.environ.get("F3M_NEAR_SYM", "1") != "0"
+    self_pairs = 0.0
+    if symmetric:
+        for k in range(1, depth + 1):
+            lev = plan.level(k)
+            cnt = np.diff(lev["offx"]).astype(np.float64)
+            for which in ("small", "keep") if k == depth else ("small",):
+                pr = lev[which]
+                if len(pr):
+                    same = pr[pr[:, 0] == pr[:, 1], 0]
+                    self_pairs += float((cnt[same] ** 2).sum())
     plan.close()
-    F = 3 * d + 3                                  # flops per kernel evaluation (d sub, d mul, d-1 add, scale, exp, fma)
+    work["near_pairs_in_one_box"] = self_pairs if symmetric else None
+    work["near_kernel_evaluations"] = (work["near_pairs"] + self_pairs) / 2 if symmetric else work["near_pairs"]
+    F = 3 * d + 3                                  # flops per listed pair (d sub, d mul, d-1 add, scale, exp, fma)
     achieved = F * work["near_pairs"] * steps / max(near_t, 1e-12) / 1e12
+    # vector-ALU issue cycles per 64 kernel evaluations: one exp2 (8) and one FMA (4); the symmetric form adds a second
+    # FMA to an evaluation that serves two listed pairs
+    valu_cycles = (8 * (work["near_pairs"] - self_pairs) + 12 * self_pairs) if symmetric else 12 * work["near_pairs"]
     rec = {"ms_per_step": dt / steps * 1e3, "ms_per_step_median": statistics.median(per_step) * 1e3,
            "points_per_s": n / (dt / steps), "tree_depth": depth, "boxes": nbx,
            "stage_ms_per_step": split_stages(stage, steps),
            "near": {"achieved_tflops": achieved, "frac": achieved / PEAK_FP32_TFLOPS, "launches_per_step": near_n // max(steps, 1),
                     "ms_per_step": near_t / steps * 1e3, "flops_per_pair": F,
-                    # the part of a pair that stays on the vector ALU whatever the dimension: one exp2 and one FMA, 12
-                    # issue cycles per 64 pairs, which at 3-D is the same figure as `frac` (12 flops per pair)
-                    "valu_frac": 12 * work["near_pairs"] * steps / max(near_t, 1e-12) / 1e12 / PEAK_FP32_TFLOPS},
+                    "symmetric": symmetric,
+                    # the part that stays on the vector ALU whatever the dimension: one exp2 and one FMA per evaluation,
+                    # 12 issue cycles per 64 of them (at 3-D the same figure as `frac` in the plain form: 12 flops per
+                    # pair); in the symmetric form 16 cycles per 64 evaluations, each serving two listed pairs
+                    "valu_frac": valu_cycles * steps / max(near_t, 1e-12) / 1e12 / PEAK_FP32_TFLOPS},
            "work": work}
     if one_stream_steps:
         # the same product with everything on the caller's stream (F3M_OVERLAP=0): every stage alone on the GPU
@@ -261,13 +282,18 @@ def main():
     near = rec["near"]
     roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
-                "kernel": "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
-                "note": "near field, bound by fp32 vector-ALU issue (one exp2 and one FMA per pair; the exponents come from the "
-                        "f16 matrix pipe with hi/lo-split operands, fp32 accumulate); achieved = %d flops x kernel evaluations / "
-                        "HIP-event time of the launch, priced against the fp32 peak; %d launches/step, %.3f ms per step, "
-                        "%.3e kernel evaluations/step; traffic = HBM bytes per launch from rocprofv3 FETCH_SIZE + WRITE_SIZE "
-                        "(profiles/near_g_kernel_n1e7_uniform3d_counters.md)"
-                        % (near["flops_per_pair"], near["launches_per_step"], near["ms_per_step"], rec["work"]["near_pairs"])}
+                "kernel": "near_sym_kernel<%d>" % d if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
+                "valu_issue_frac": near["valu_frac"],
+                "note": "near field, bound by fp32 vector-ALU issue (one exp2 and one FMA per kernel evaluation; the exponents "
+                        "come from the f16 matrix pipe with hi/lo-split operands, fp32 accumulate); achieved = %d algorithmic "
+                        "flops x listed point pairs / HIP-event time of the launch, priced against the fp32 peak; %d "
+                        "launches/step, %.3f ms per step, %.3e listed pairs/step%s; traffic = HBM bytes per launch from "
+                        "rocprofv3 FETCH_SIZE + WRITE_SIZE (%s)"
+                        % (near["flops_per_pair"], near["launches_per_step"], near["ms_per_step"], rec["work"]["near_pairs"],
+                           (" (X = Y: the kernel evaluates a pair of different boxes once for both directions, %.3e evaluations; "
+                            "valu_issue_frac = vector-ALU issue cycles of those evaluations, 8 for exp2 and 4 per FMA, against "
+                            "the same peak)" % rec["work"]["near_kernel_evaluations"]) if near["symmetric"] else "",
+                           os.path.relpath(TRAFFIC_PROFILE, ROOT))}
     prof_us = profiled_near_launch_us() if headline else None
     if prof_us:
         # the same fraction from the committed kernel trace's average launch (warm-up launch included): the low end
