@@ -61,6 +61,11 @@ int f3m_exact_f64(int d, const double *X, int64_t N, const double *Y, int64_t M,
 int f3m_plan_create(int d, const float *X, int64_t N, const float *Y, int64_t M, const f3m_params *params,
                     void *stream, f3m_plan **plan);
 int f3m_plan_apply(f3m_plan *plan, const float *b, int c, float *out, void *stream);
+/* (Results are reproducible: the same call on the same inputs gives the same bits, whatever the order in which
+ * the GPU runs the wavefronts.  Where sums of several wavefronts meet in one element -- the near field of a
+ * product on one tree with one column evaluates each pair of boxes once for both directions -- they are added
+ * as 64-bit fixed-point numbers scaled by the largest |b|, one unit below 1e-18 of (number of sources) x
+ * max |b|.  F3M_NEAR_SYM=0 in the environment selects the one-directional near field for such products.) */
 /* out(M,c) = K(X,Y)^T u, u (N,c), with the plan of (X, Y): the two trees swap roles and every interaction
  * list is read from its Y boxes (the lists of (Y, X) are the lists of (X, Y) with the boxes of each pair
  * swapped: the classification of F3M_src/1_d_conv.cu:927-952 depends on n_x + n_y and |c_y - c_x| only).
@@ -76,7 +81,11 @@ int f3m_plan_destroy(f3m_plan *plan);
  * need does not grow with c beyond four columns: the sorted copies of b and of the result for one group of
  * columns (4 (N + M) bytes for c = 1, 16 (N + M) bytes for c >= 2), the partial sums of that group's near
  * field, and the moments and local expansions of one column's far field; every further group and column
- * reuses that memory (N = M = 1e7 with one column just fits).  A product that needs more is refused with
+ * reuses that memory (N = M = 1e7 with one column just fits).  One tree and one column: f3m_plan_apply
+ * sums the near field in its symmetric form, which needs 8 N more bytes for fixed-point sums; this call
+ * takes that form only where those bytes are at most a quarter of the scratch memory still free (N up
+ * to about 3e6: the bits of f3m_plan_apply) and the plain form beyond (same sums in another order: equal
+ * to about 1e-6 relative, not bit for bit).  A product that needs more is refused with
  * error 42 while its first column group is being queued, before anything is written to out.  The plan's own
  * tables are built by the first f3m_plan_apply with the same number of columns, which must therefore have
  * run once before (otherwise error 41).  All calls on a GPU share the one scratch array: calls that overlap
