@@ -960,9 +960,9 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                                          rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, SymSums());
 }
 
-// the symmetric form: four target tiles per wavefront, one column, the plain exponent; and the factored form with five
-// target tiles: both held to 120 registers, so that four wavefronts leave 32 of a SIMD's 512 to the far field's small
-// workgroups on the second stream (the attribute counts register pairs on this target)
+// the symmetric form: four target tiles per wavefront, one column, the plain exponent; held to 120 registers, so that four
+// wavefronts leave 32 of a SIMD's 512 to the far field's small workgroups on the second stream (the attribute counts
+// register pairs on this target)
 #ifdef F3M_CPU_EMU
 #define F3M_NEAR_SYM_REGS
 #else
@@ -979,18 +979,6 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS 
 {
     near_g_body<D, 4, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
-}
-
-template <int D>
-__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_fact5_kernel(
-    const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
-    long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
-    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
-    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
-    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout)
-{
-    near_g_body<D, 5, 1, true, false>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
-                                      rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, SymSums());
 }
 
 // outs += the slices of a split near field, in slice order; one thread per target slot of a work item
@@ -1271,9 +1259,6 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #define F3M_NEAR_FORM(DD, FF)                                                                                         \
     if constexpr (DD <= 3 && !FF) {                                                                                   \
         if (sym && nsplit == 1) { go_sym(near_sym_kernel<DD>); break; }                                     \
-    }                                                                                                                 \
-    if constexpr (DD == 5 && FF) {                                                                                    \
-        if (tpw == 5) { go(near_fact5_kernel<DD>); break; }                                                           \
     }                                                                                                                 \
     if (tpw == 5) go(near_g_kernel<DD, 5, 1, FF>);                                                                    \
     else if (nc == 4) go(near_g_kernel<DD, 4, 4, FF>);                                                                \
