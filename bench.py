@@ -45,7 +45,7 @@ def profiled_near_launch_us():
     """average duration of the near-field launch in the committed rocprofv3 kernel trace of this command (the first
     table: default two-stream mode), microseconds"""
     try:
-        m = re.search(r"\|\s*f3m::near_sym_kernel<3>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
+        m = re.search(r"\|\s*f3m::near_sym_kernel<3, 4>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
         return float(m.group(1)) if m else None
     except OSError:
         return None
@@ -121,10 +121,10 @@ def run_config(name, n, steps, warmup, subsample, keep_inputs=False, nodes=None,
     work = plan.work()
     depth = plan.depth
     nbx = plan.level_sizes(depth)["nbx"] if depth else 1
-    # One tree, one column, up to three dimensions: the library's near field takes the symmetric form, which evaluates a
+    # One tree, one column, up to four dimensions: the library's near field takes the symmetric form, which evaluates a
     # listed pair of boxes (A, B), A != B, once for both directions.  Point pairs inside one box (A, A) are evaluated
     # one by one as before: their number comes from the lists.
-    symmetric = Y is None and b.shape[1] == 1 and d <= 3 and os.environ.get("F3M_NEAR_SYM", "1") != "0"
+    symmetric = Y is None and b.shape[1] == 1 and d <= 4 and os.environ.get("F3M_NEAR_SYM", "1") != "0"
     self_pairs = 0.0
     if symmetric:
         for k in range(1, depth + 1):
@@ -282,7 +282,7 @@ def main():
     near = rec["near"]
     roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
-                "kernel": "near_sym_kernel<%d>" % d if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
+                "kernel": "near_sym_kernel<%d,%d>" % (d, tiles_per_wave) if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
                 "valu_issue_frac": near["valu_frac"],
                 "note": "near field, bound by fp32 vector-ALU issue (one exp2 and one FMA per kernel evaluation; the exponents "
                         "come from the f16 matrix pipe with hi/lo-split operands, fp32 accumulate); achieved = %d algorithmic "

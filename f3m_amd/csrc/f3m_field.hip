@@ -909,7 +909,15 @@ __device__ __forceinline__ void near_g_body(
                     wave_sync();
                     sum += wave_shfl_xor_f(sum, 32);
                     if (half == 0 && j0 + col < s1) {
-                        if (fixscale != 0.f) atomic_add_i64(symsums.fix + j0 + col, llrintf(sum * fixscale));
+                        if (fixscale != 0.f) {
+                            // |v| < 2^61, and a float has 24 bits: both halves of the integer from exact float steps
+                            // (rounded down to a whole unit, which is below 1e-18 of the bound)
+                            const float v = sum * fixscale;
+                            const float hf = floorf(v * 2.3283064365386963e-10f);          // v / 2^32
+                            const float lf = fmaf(hf, -4294967296.f, v);                     // in [0, 2^32)
+                            const long long iv = (long long)(((unsigned long long)(unsigned)(int)hf << 32) | (unsigned)lf);
+                            atomic_add_i64(symsums.fix + j0 + col, iv);
+                        }
                         else atomic_add_f32(outs + j0 + col, sum);
                     }
                 }
@@ -960,15 +968,15 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
                                          rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, SymSums());
 }
 
-// the symmetric form: four target tiles per wavefront, one column, the plain exponent; held to 120 registers, so that four
-// wavefronts leave 32 of a SIMD's 512 to the far field's small workgroups on the second stream (the attribute counts
-// register pairs on this target)
+// the symmetric form: four or five target tiles per wavefront, one column, the plain exponent; held to 120 registers, so
+// that four wavefronts leave 32 of a SIMD's 512 to the far field's small workgroups on the second stream (the attribute
+// counts register pairs on this target; what does not fit is spilled outside the loops over the tiles)
 #ifdef F3M_CPU_EMU
 #define F3M_NEAR_SYM_REGS
 #else
 #define F3M_NEAR_SYM_REGS __attribute__((amdgpu_num_vgpr(60)))      // counted in pairs on this target: 120 registers
 #endif
-template <int D>
+template <int D, int TPW>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
@@ -977,7 +985,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS 
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
     SymSums symsums)
 {
-    near_g_body<D, 4, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+    near_g_body<D, TPW, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
@@ -1106,8 +1114,7 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 
 // the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
 // the list, the exact number of work items (else -1)
-static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact,
-                       bool sym = false)
+static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact)
 {
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
     const long long tiles = (avg_points + 31) / 32;
@@ -1117,7 +1124,6 @@ static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list
     // then.  N=1e7: the fastest products 39.8 ms against 40.9, but single products up to 48.9 and means of 40.8-42.8
     // against a steady 41.0 with four tiles, 115 registers.  Four it is.)
     if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
-    if (sym) tpw = 4;                     // the symmetric form has four tiles (and saves more than the fifth tile does)
     items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
 }
 
@@ -1132,11 +1138,11 @@ bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList
 
 // Whether near_field takes a list in the symmetric form (see near_g_kernel): one tree (then every list of the plan names
 // (A,B) exactly when it names (B,A): the class of a pair depends on the distance of the centres and on the sum of the
-// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to three dimensions.
+// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to four dimensions.
 // F3M_NEAR_SYM=0 turns it off.
 bool near_symmetric(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const PairList &list, float lcs, int nc)
 {
-    if (&tx != &ty || nc != 1 || d > 3 || list.n == 0) return false;
+    if (&tx != &ty || nc != 1 || d > 4 || list.n == 0) return false;
     if (const char *e = getenv("F3M_NEAR_SYM")) if (atoi(e) == 0) return false;
     return near_on_matrix_pipe(d, lcs, lx.edge) && !near_factored(d, lcs, lx.edge);
     // (lists cut into slices, see near_field, take the plain form all the same)
@@ -1170,11 +1176,10 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     int tpw;
     long long items_exact;
-    // (the shape follows from what the list could take, not from whether this call brings a place for the fixed-point
-    // sums: the tile table of a list is then the same for every call)
-    const bool sym_capable = near_symmetric(d, tx, lx, ty, list, lcs, nc);
-    const bool sym_wanted = sym_capable && symsums != nullptr && symsums->fix != nullptr;
-    near_shape(tx, lx, list, nc, tpw, items_exact, sym_capable);
+    // (the symmetric form has the tile shapes of the plain one, so the tile table of a list is the same for every call,
+    // whether it brings a place for the fixed-point sums or not)
+    const bool sym_wanted = symsums != nullptr && symsums->fix != nullptr && near_symmetric(d, tx, lx, ty, list, lcs, nc);
+    near_shape(tx, lx, list, nc, tpw, items_exact);
     // From five dimensions on the work items are long and their lists differ a lot in length (3^5 boxes around
     // an interior box, 2^5 around a corner): the boxes with the longest lists go first, which shortens the
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
@@ -1257,8 +1262,12 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                        list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout, *symsums);
         };
 #define F3M_NEAR_FORM(DD, FF)                                                                                         \
-    if constexpr (DD <= 3 && !FF) {                                                                                   \
-        if (sym && nsplit == 1) { go_sym(near_sym_kernel<DD>); break; }                                     \
+    if constexpr (DD <= 4 && !FF) {                                                                                   \
+        if (sym && nsplit == 1) {                                                                                     \
+            if (tpw == 5) go_sym((near_sym_kernel<DD, 5>));                                                           \
+            else go_sym((near_sym_kernel<DD, 4>));                                                                    \
+            break;                                                                                                    \
+        }                                                                                                             \
     }                                                                                                                 \
     if (tpw == 5) go(near_g_kernel<DD, 5, 1, FF>);                                                                    \
     else if (nc == 4) go(near_g_kernel<DD, 4, 4, FF>);                                                                \

@@ -405,7 +405,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
                     dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
                     dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
-                    if (sym && P->early_c == 1 && d <= 3) {     // (wherever near_symmetric may say yes)
+                    if (sym && P->early_c == 1 && d <= 4) {     // (wherever near_symmetric may say yes)
                         P->early_symfix.reset((size_t)P->N);
                         P->early_symmax.reset(1);
                         dev_fill(P->early_symfix.get(), 0, sizeof(long long) * (size_t)P->N, side_stream().stream);

@@ -347,7 +347,7 @@ def test_mfma_near_field(oracle, monkeypatch):
                 assert np.array_equal(eng.apply(b[:, col:col + 1]), got[:, col:col + 1])
 
 
-@pytest.mark.parametrize("name", ["uniform3", "normal2", "uniform1", "dups_faces"])
+@pytest.mark.parametrize("name", ["uniform3", "normal2", "uniform1", "uniform4", "dups_faces"])
 def test_symmetric_near_field(oracle, monkeypatch, name):
     """One tree, one column: the tiles of a pair of boxes are evaluated once and added in both directions, the second
     one through the wavefront's LDS block and as fixed-point sums.  (F3M_SPLIT_TARGET=1: one wavefront per work item on

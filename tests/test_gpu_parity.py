@@ -741,7 +741,8 @@ def test_one_stream_and_two_streams_give_the_same_bits(eng, monkeypatch, name):
         assert np.array_equal(one, two) and np.array_equal(one_plan, two)
 
 
-@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "uniform2", "uniform1", "lattice_faces_dups", "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "uniform2", "uniform1", "uniform4", "lattice_faces_dups",
+                                  "uniform3_varcomp"])
 def test_symmetric_near_field_against_oracle(eng, oracle, monkeypatch, name):
     """One tree and one column: the near field evaluates the tiles of a pair of boxes once and adds them in both
     directions (half the exponentials), the second direction as fixed-point sums.  On these small clouds the lists
@@ -763,9 +764,11 @@ def test_symmetric_near_field_against_oracle(eng, oracle, monkeypatch, name):
         assert np.array_equal(plan.apply(bd).cpu().numpy(), sym), rep
         assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym), rep
     plan.close()
-    monkeypatch.setenv("F3M_OVERLAP", "0")
-    assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym)
-    monkeypatch.delenv("F3M_OVERLAP")
+    if name != "uniform4":      # (on the 3^4 grid the far field shares M2L sums between siblings only beside a near field:
+        # other rounding of the far field in one-stream mode, whatever the near field's form)
+        monkeypatch.setenv("F3M_OVERLAP", "0")
+        assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym)
+        monkeypatch.delenv("F3M_OVERLAP")
     monkeypatch.setenv("F3M_NEAR_SYM", "0")
     plain = eng.kmvm(Xd, None, bd, **prm).cpu().numpy()
     assert rel_l2(sym, plain) < 1e-6
