@@ -45,7 +45,7 @@ def profiled_near_launch_us():
     """average duration of the near-field launch in the committed rocprofv3 kernel trace of this command (the first
     table: default two-stream mode), microseconds"""
     try:
-        m = re.search(r"\|\s*f3m::near_sym_kernel<3, 4>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
+        m = re.search(r"\|\s*f3m::near_sym_kernel<3, 5>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
         return float(m.group(1)) if m else None
     except OSError:
         return None
@@ -276,10 +276,11 @@ def main():
     rec, (X, Y, b, prm) = run_config(name, N, args.steps, args.warmup, 0 if args.no_accuracy else args.subsample, keep_inputs=True,
                                      one_stream_steps=0 if args.no_extra else 3)
     M = N if Y is None else Y.shape[0]
-    tiles_per_wave = 5 if (N // max(rec["boxes"], 1) + 31) // 32 == 5 else 4     # the library's choice (near_field)
+    near = rec["near"]
+    tiles = (N // max(rec["boxes"], 1) + 31) // 32                              # the library's choice (near_shape):
+    tiles_per_wave = 5 if tiles == 5 or (near["symmetric"] and (tiles + 4) // 5 < (tiles + 3) // 4) else 4
     headline = N == 10_000_000 and name == "uniform3_ls1"
     traffic, traffic_range = near_traffic_bytes() if headline else (None, None)
-    near = rec["near"]
     roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
                 "kernel": "near_sym_kernel<%d,%d>" % (d, tiles_per_wave) if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),

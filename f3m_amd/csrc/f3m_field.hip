@@ -1114,7 +1114,8 @@ void prepare_near_operands(int d, const Tree &ty, const TreeLevel &ly, float lcs
 
 // the launch shape near_field gives a list: target tiles per wavefront and, where the plan has counted the rows of
 // the list, the exact number of work items (else -1)
-static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact)
+static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list, int nc, int &tpw, long long &items_exact,
+                       bool sym_capable = false)
 {
     const long long avg_points = list.rows > 0 ? list.row_points / list.rows : tx.n / std::max(1, lx.nb);
     const long long tiles = (avg_points + 31) / 32;
@@ -1123,6 +1124,12 @@ static void near_shape(const Tree &tx, const TreeLevel &lx, const PairList &list
     // four wavefronts then fill the 512 of a SIMD and the far field's wavefronts get in beside them only now and
     // then.  N=1e7: the fastest products 39.8 ms against 40.9, but single products up to 48.9 and means of 40.8-42.8
     // against a steady 41.0 with four tiles, 115 registers.  Four it is.)
+    // A list that can take the symmetric form (four wavefronts per SIMD with either shape): five wherever that cuts a
+    // typical box into fewer work items, e.g. ten tiles as 5 + 5 instead of 4 + 4 + 2 -- the source tiles are then loaded,
+    // and their column sums added up and sent off, twice per box instead of three times (N=1e7, 3-D: 8.47 -> 8.12 ms).
+    // Only for a list that will not be cut into slices (whose sums, and so the bits of a column, depend on the number of
+    // work items: a column keeps the bits it has inside a group of columns).
+    if (sym_capable && nc == 1 && (tiles + 4) / 5 < (tiles + 3) / 4 && list.rows >= 0 && list.items160 >= 16384) tpw = 5;
     if (const char *e = getenv("F3M_NEAR_TPW")) tpw = (atoi(e) == 5 && nc == 1) ? 5 : 4;      // tuning aid
     items_exact = list.rows >= 0 ? (tpw == 5 ? list.items160 : list.items128) : -1;
 }
@@ -1176,10 +1183,11 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     // number of work items is exact; otherwise the mean over all boxes and an upper bound.
     int tpw;
     long long items_exact;
-    // (the symmetric form has the tile shapes of the plain one, so the tile table of a list is the same for every call,
-    // whether it brings a place for the fixed-point sums or not)
-    const bool sym_wanted = symsums != nullptr && symsums->fix != nullptr && near_symmetric(d, tx, lx, ty, list, lcs, nc);
-    near_shape(tx, lx, list, nc, tpw, items_exact);
+    // (the shape follows from what the list could take, not from whether this call brings a place for the fixed-point
+    // sums: the tile table of a list is then the same for every call)
+    const bool sym_capable = near_symmetric(d, tx, lx, ty, list, lcs, nc);
+    const bool sym_wanted = sym_capable && symsums != nullptr && symsums->fix != nullptr;
+    near_shape(tx, lx, list, nc, tpw, items_exact, sym_capable);
     // From five dimensions on the work items are long and their lists differ a lot in length (3^5 boxes around
     // an interior box, 2^5 around a corner): the boxes with the longest lists go first, which shortens the
     // end of the launch (N=1e7, 5-D: 44.6 -> 43.6 ms; 4-D and 3-D lose the Morton order's cache locality and
