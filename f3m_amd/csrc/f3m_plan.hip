@@ -394,6 +394,12 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             if (ahead) settle_early();
             level_launch(keep, P->tx, *P->ty, k, cp, pend, reinterpret_cast<long long *>(dres.get()),
                          drow.get() + 8 * (P->levels.size() - 1), ahead, dres.get() + 8, dres.get() + 10, s);
+            // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
+            // host has them, wherever an upper bound of the sizes is a modest allocation: it then runs during the wait.
+            fetch_level_begin(&pend, ahead);
+            lists_write_early(pend, *keep, P->tx, *P->ty, k, cp, L, s);
+            // (Queued after this level's own kernels: the host needs a while for these launches, and the caller's stream
+            // should not wait for it.)
             // No further division: this is the deepest level, whose near lists will be summed.  Its source operands
             // are prepared on the second stream (behind the moves of the points) while its lists are built here.
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)
@@ -417,10 +423,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     }
                 }
             }
-            // The sizes of the lists travel to the host; the pass that writes the lists is queued behind them, before the
-            // host has them, wherever an upper bound of the sizes is a modest allocation: it then runs during the wait.
-            fetch_level_begin(&pend, ahead);
-            lists_write_early(pend, *keep, P->tx, *P->ty, k, cp, L, s);
             fetch_level_wait();
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
                          reinterpret_cast<const long long *>(hres + 16), s);
