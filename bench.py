@@ -121,10 +121,10 @@ def run_config(name, n, steps, warmup, subsample, keep_inputs=False, nodes=None,
     work = plan.work()
     depth = plan.depth
     nbx = plan.level_sizes(depth)["nbx"] if depth else 1
-    # One tree, one column, up to four dimensions: the library's near field takes the symmetric form, which evaluates a
+    # One tree, one column, up to five dimensions: the library's near field takes the symmetric form, which evaluates a
     # listed pair of boxes (A, B), A != B, once for both directions.  Point pairs inside one box (A, A) are evaluated
     # one by one as before: their number comes from the lists.
-    symmetric = Y is None and b.shape[1] == 1 and d <= 4 and os.environ.get("F3M_NEAR_SYM", "1") != "0"
+    symmetric = Y is None and b.shape[1] == 1 and d <= 5 and os.environ.get("F3M_NEAR_SYM", "1") != "0"
     self_pairs = 0.0
     if symmetric:
         for k in range(1, depth + 1):

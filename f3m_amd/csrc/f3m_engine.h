@@ -230,6 +230,9 @@ struct SymSums {
     long long *fix = nullptr;          // one per sorted point, cleared by the caller; null: not used
     const unsigned *absmax = nullptr;
     long long nsrc = 0;
+    // factored form only (near_field fills them in): the sorted weights themselves (the kernel's weight argument then holds
+    // them times exp2(-|y'|^2)) and that factor per point
+    const float *braw = nullptr, *ey = nullptr;
 };
 // scale of the fixed-point sums as a power of two (0: weights not finite)
 __host__ __device__ inline float sym_scale(unsigned absmax_bits, long long nsrc)

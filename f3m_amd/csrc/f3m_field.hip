@@ -712,19 +712,21 @@ __device__ __forceinline__ void near_g_body(
     for (int q = 0; q < TPW; q++)
 #pragma unroll
         for (int c = 0; c < NC; c++) acc[q][c] = 0.f;
-    static_assert(!SYM || (NC == 1 && !FACT), "the symmetric form takes one column and the plain exponent");
+    static_assert(!SYM || NC == 1, "the symmetric form takes one column");
     // SYM: the wavefront's LDS block: 32 rows of the column reduction, then the weights of its targets (one tree: sources
     // and targets are the same points in the same order), kept there to spare registers
-    constexpr int kSymBlock = 32 * kSymRedStride + TPW * 32;
+    // (factored form: a second copy, the weights times the targets' factor exp2(-|x''|^2) of the current anchor)
+    constexpr int kSymBlock = 32 * kSymRedStride + TPW * 32 * (FACT ? 2 : 1);
     __shared__ float red_all[SYM ? kNearWavesPerBlock * kSymBlock : 1];
     float *const red = red_all + (SYM ? (threadIdx.x >> 6) * kSymBlock : 0);
     float *const btl = red + 32 * kSymRedStride;
+    float *const wtl = FACT ? btl + TPW * 32 : btl;
     float fixscale = 0.f;                            // SYM: scale of the fixed-point sums (0: weights not finite)
     if constexpr (SYM) {
 #pragma unroll
         for (int q = 0; q < TPW; q++) {
             const int i = x0 + q * 32 + col;
-            if (half == 0) btl[q * 32 + col] = i < x1 ? bs[i] : 0.f;
+            if (half == 0) btl[q * 32 + col] = i < x1 ? (FACT ? symsums.braw[i] : bs[i]) : 0.f;
         }
         wave_sync();
         fixscale = sym_scale(symsums.absmax[0], symsums.nsrc);
@@ -859,7 +861,11 @@ __device__ __forceinline__ void near_g_body(
                 bop[q][n] = half ? v1 : v0;
             }
             if (FACT) ex[q] = fast_exp2(nx2);
+            if constexpr (SYM && FACT) {
+                if (half == 0) wtl[q * 32 + col] = ex[q] * btl[q * 32 + col];
+            }
         }
+        if constexpr (SYM && FACT) wave_sync();
         }
         for (int j0 = s0; j0 < s1; j0 += 32) {
             h8 a[NS];
@@ -906,7 +912,7 @@ __device__ __forceinline__ void near_g_body(
 #pragma unroll
                     for (int r = 0; r < 16; r++) sacc[r] = 0.f;
                     auto tile2 = [&](int q) {
-                        const float btq = btl[q * 32 + col];
+                        const float btq = wtl[q * 32 + col];
                         f32x16 t;
 #pragma unroll
                         for (int r = 0; r < 16; r++) t[r] = 0.f;
@@ -915,7 +921,8 @@ __device__ __forceinline__ void near_g_body(
 #pragma unroll
                         for (int r = 0; r < 16; r++) {
                             const float e = fast_exp2(t[r]);
-                            acc[q][0] = fmaf(e, bq[0][r], acc[q][0]);
+                            if (FACT) run[q][0] = fmaf(e, bq[0][r], run[q][0]);
+                            else acc[q][0] = fmaf(e, bq[0][r], acc[q][0]);
                             sacc[r] = fmaf(e, btq, sacc[r]);
                         }
                     };
@@ -938,6 +945,7 @@ __device__ __forceinline__ void near_g_body(
                     wave_sync();
                     sum += wave_shfl_xor_f(sum, 32);
                     if (half == 0 && j0 + col < s1) {
+                        if (FACT) sum *= symsums.ey[j0 + col];       // the sources' factor exp2(-|y'|^2)
                         if (fixscale != 0.f) {
                             // |v| < 2^61, and a float has 24 bits: both halves of the integer from exact float steps
                             // (rounded down to a whole unit, which is below 1e-18 of the bound)
@@ -1005,7 +1013,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
 #else
 #define F3M_NEAR_SYM_REGS __attribute__((amdgpu_num_vgpr(60)))      // counted in pairs on this target: 120 registers
 #endif
-template <int D, int TPW>
+template <int D, int TPW, bool FACT = false>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
@@ -1014,7 +1022,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS 
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
     SymSums symsums)
 {
-    near_g_body<D, TPW, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+    near_g_body<D, TPW, 1, FACT, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
@@ -1174,13 +1182,15 @@ bool near_single_pass(int d, const Tree &tx, const TreeLevel &lx, const PairList
 
 // Whether near_field takes a list in the symmetric form (see near_g_kernel): one tree (then every list of the plan names
 // (A,B) exactly when it names (B,A): the class of a pair depends on the distance of the centres and on the sum of the
-// two boxes' counts), one column, the matrix-pipe kernel with the plain exponent, up to four dimensions.
+// two boxes' counts), one column, the matrix-pipe kernel: with the plain exponent up to four dimensions, with the
+// factored one in five.
 // F3M_NEAR_SYM=0 turns it off.
 bool near_symmetric(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, const PairList &list, float lcs, int nc)
 {
-    if (&tx != &ty || nc != 1 || d > 4 || list.n == 0) return false;
+    if (&tx != &ty || nc != 1 || d > 5 || list.n == 0) return false;
     if (const char *e = getenv("F3M_NEAR_SYM")) if (atoi(e) == 0) return false;
-    return near_on_matrix_pipe(d, lcs, lx.edge) && !near_factored(d, lcs, lx.edge);
+    // (in five dimensions the factored form only: the plain one has no registers left for it)
+    return near_on_matrix_pipe(d, lcs, lx.edge) && (d == 5) == near_factored(d, lcs, lx.edge);
     // (lists cut into slices, see near_field, take the plain form all the same)
 }
 
@@ -1267,7 +1277,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         const NearOps src = build_near_operands(d, ty, ly, sc, near_factored(d, lcs, ly.edge), only_list ? &list : nullptr, s);
         const bool fact = src.ey != nullptr;
         if (prepare_only) return;
-        const bool sym = !fact && sym_wanted;
+        const bool sym = sym_wanted && fact == (d == 5);
         F3M_REQUIRE(!(sym && direct), 35, "direct output and the symmetric near field exclude each other");
         int stripe = 128;   // consecutive workgroups per XCD stripe (0: 9.5 ms, 16: 9.3, 64-256: 9.15, 1024: 9.4 at N=1e7)
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
@@ -1304,15 +1314,18 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                        list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout);
         };
         auto go_sym = [&](auto kern) {
+            SymSums sums = *symsums;
+            sums.braw = bs;
+            sums.ey = src.ey;
             F3M_LAUNCH(kern, ngrid, kNearWavesPerBlock * 64, 0, s, tx.pts.get(), tx.n, src.ops, stride, wsrc, wstride, outs,
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(),
-                       list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout, *symsums);
+                       list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout, sums);
         };
 #define F3M_NEAR_FORM(DD, FF)                                                                                         \
-    if constexpr (DD <= 4 && !FF) {                                                                                   \
+    if constexpr ((DD <= 4 && !FF) || (DD == 5 && FF)) {                                                              \
         if (sym && nsplit == 1) {                                                                                     \
-            if (tpw == 5) go_sym((near_sym_kernel<DD, 5>));                                                           \
-            else go_sym((near_sym_kernel<DD, 4>));                                                                    \
+            if (tpw == 5) go_sym((near_sym_kernel<DD, 5, FF>));                                                       \
+            else go_sym((near_sym_kernel<DD, 4, FF>));                                                                \
             break;                                                                                                    \
         }                                                                                                             \
     }                                                                                                                 \

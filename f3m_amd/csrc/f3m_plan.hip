@@ -411,7 +411,7 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                     P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
                     dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
                     dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
-                    if (sym && P->early_c == 1 && d <= 4) {     // (wherever near_symmetric may say yes)
+                    if (sym && P->early_c == 1 && d <= 5) {     // (wherever near_symmetric may say yes)
                         P->early_symfix.reset((size_t)P->N);
                         P->early_symmax.reset(1);
                         dev_fill(P->early_symfix.get(), 0, sizeof(long long) * (size_t)P->N, side_stream().stream);
@@ -621,6 +621,13 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
         for (int k = 1; k <= depth; k++) any_far = any_far || (transposed ? P->levels[k - 1].farT.n : P->levels[k - 1].far.n) > 0;
         const char *oe = getenv("F3M_OVERLAP");
         overlap = any_far && !per_level && g_arena == nullptr && !(oe && atoi(oe) == 0);
+        // Five dimensions, symmetric near field: the far field follows the near field on the caller's stream.  Both are
+        // bound by the vector ALU there (M2L on 3^5 nodes takes 6 ms alone), beside each other they take as long as one
+        // after the other, and M2L has its faster form (whole families of siblings per workgroup) only alone on the GPU:
+        // N=1e7: 38.3 ms against 45.8 with the far field beside the (shorter) symmetric near field.
+        if (overlap && P->symmetric && c == 1 && P->d == 5 &&
+            near_symmetric(P->d, TX, TX.lev[depth], TY, small_of(depth), P->lcs, 1))
+            overlap = false;
     }
     // Where the whole near field is one launch in which every target belongs to one wavefront, and the far field is
     // evaluated at the points once, both add their sums straight into the caller's array (cleared before; two additions

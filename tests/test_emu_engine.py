@@ -377,6 +377,22 @@ def test_symmetric_near_field(oracle, monkeypatch, name):
         assert not both.any() or rel_l2(sym[both], plain[both]) < 1e-5
 
 
+def test_symmetric_near_field_five_dimensions(oracle, monkeypatch):
+    """d = 5: the symmetric form goes with the factored exponent (the second direction carries the targets' factor into
+    the sums and gets the sources' factor after the column sums)."""
+    monkeypatch.setenv("F3M_NEAR", "mfma")
+    monkeypatch.setenv("F3M_NEAR_FACT", "1")
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    rng = np.random.default_rng(13)
+    X = rng.random((2200, 5), dtype=f32)
+    b = rng.standard_normal((2200, 1)).astype(f32)
+    prm = dict(ls=1.0, min_points=80, nr_of_interpolation=32, small_field_points=40)
+    sym = ee.kmvm(X, None, b, **prm)
+    assert rel_l2(sym, oracle.kmvm(X, None, b, **prm)) < 1e-5
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    assert 0 < rel_l2(sym, ee.kmvm(X, None, b, **prm)) < 1e-6
+
+
 @pytest.mark.parametrize("form", ["0", "1"])
 def test_mfma_near_field_five_dimensions(oracle, monkeypatch, form):
     """d = 5: two matrix instructions per tile in the plain form, one in the factored form (the weights carry

@@ -741,8 +741,8 @@ def test_one_stream_and_two_streams_give_the_same_bits(eng, monkeypatch, name):
         assert np.array_equal(one, two) and np.array_equal(one_plan, two)
 
 
-@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "uniform2", "uniform1", "uniform4", "lattice_faces_dups",
-                                  "uniform3_varcomp"])
+@pytest.mark.parametrize("name", ["C1_uniform3", "normal3", "uniform2", "uniform1", "uniform4", "uniform5", "normal5",
+                                  "lattice_faces_dups", "uniform3_varcomp"])
 def test_symmetric_near_field_against_oracle(eng, oracle, monkeypatch, name):
     """One tree and one column: the near field evaluates the tiles of a pair of boxes once and adds them in both
     directions (half the exponentials), the second direction as fixed-point sums.  On these small clouds the lists
@@ -764,7 +764,7 @@ def test_symmetric_near_field_against_oracle(eng, oracle, monkeypatch, name):
         assert np.array_equal(plan.apply(bd).cpu().numpy(), sym), rep
         assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym), rep
     plan.close()
-    if name != "uniform4":      # (on the 3^4 grid the far field shares M2L sums between siblings only beside a near field:
+    if name != "uniform4":      # (5-D takes the factored exponent; on the 3^4 grid the far field shares M2L sums between siblings only beside a near field:
         # other rounding of the far field in one-stream mode, whatever the near field's form)
         monkeypatch.setenv("F3M_OVERLAP", "0")
         assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), sym)
