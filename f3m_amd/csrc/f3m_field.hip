@@ -1013,7 +1013,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
 #else
 #define F3M_NEAR_SYM_REGS __attribute__((amdgpu_num_vgpr(60)))      // counted in pairs on this target: 120 registers
 #endif
-template <int D, int TPW, bool FACT = false>
+template <int D, int TPW>
 __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
@@ -1022,8 +1022,23 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS 
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
     SymSums symsums)
 {
-    near_g_body<D, TPW, 1, FACT, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+    near_g_body<D, TPW, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
+}
+
+// the symmetric form with the factored exponent (five dimensions): the far field does not run beside it (plan_apply), so
+// it keeps the 128 registers of four wavefronts per SIMD
+template <int D, int TPW>
+__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) near_symf_kernel(
+    const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
+    long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
+    const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
+    const int *__restrict__ pairs, const int *__restrict__ rowptr, const int *__restrict__ tileoff, int nbx, float sc,
+    int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
+    SymSums symsums)
+{
+    near_g_body<D, TPW, 1, true, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
 // outs += the slices of a split near field, in slice order; one thread per target slot of a work item
@@ -1324,8 +1339,13 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
 #define F3M_NEAR_FORM(DD, FF)                                                                                         \
     if constexpr ((DD <= 4 && !FF) || (DD == 5 && FF)) {                                                              \
         if (sym && nsplit == 1) {                                                                                     \
-            if (tpw == 5) go_sym((near_sym_kernel<DD, 5, FF>));                                                       \
-            else go_sym((near_sym_kernel<DD, 4, FF>));                                                                \
+            if constexpr (FF) {                                                                                       \
+                if (tpw == 5) go_sym((near_symf_kernel<DD, 5>));                                                      \
+                else go_sym((near_symf_kernel<DD, 4>));                                                               \
+            } else {                                                                                                  \
+                if (tpw == 5) go_sym((near_sym_kernel<DD, 5>));                                                       \
+                else go_sym((near_sym_kernel<DD, 4>));                                                                \
+            }                                                                                                         \
             break;                                                                                                    \
         }                                                                                                             \
     }                                                                                                                 \
