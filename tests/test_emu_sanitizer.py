@@ -2,7 +2,7 @@
 sanitize_driver.cpp): an access outside an array in a kernel is a report here instead of a fault on a GPU.
 Compiling takes a minute or two and a case a minute or more (the emulation switches contexts at every barrier and
 shuffle), so the test runs only when F3M_SANITIZE is set: F3M_SANITIZE=1 runs three cases of ~400 points,
-F3M_SANITIZE=<first>,<count>,<points> any others."""
+F3M_SANITIZE=<first>,<count>,<points> any others.  F3M_SANITIZE=1 also runs the symmetric near field in 3, 4 and 5 dimensions."""
 import os
 import subprocess
 import sys
@@ -25,3 +25,14 @@ def test_kernels_under_address_and_undefined_behaviour_sanitizers():
     print(r.stderr[-4000:])
     assert r.returncode == 0 and "done" in r.stdout
     assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr
+    if "," in spec:
+        return
+    # the symmetric near field (one tree, one column, one wavefront per work item) in 3, 4 and 5 dimensions: its LDS block,
+    # the skipped boxes of a list, the fixed-point sums
+    for shape in (["3", "27", "60", "30"], ["4", "16", "60", "30"], ["5", "32", "60", "30"]):
+        env2 = dict(env, F3M_SPLIT_TARGET="1", F3M_NEAR="mfma", F3M_NEAR_FACT="1")
+        r = subprocess.run([exe, "0", "1", "500"] + shape, env=env2, capture_output=True, text=True, timeout=3600)
+        print(r.stdout[-2000:])
+        print(r.stderr[-2000:])
+        assert r.returncode == 0 and "done" in r.stdout
+        assert "ERROR: AddressSanitizer" not in r.stderr and "runtime error" not in r.stderr
