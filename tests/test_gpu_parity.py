@@ -470,6 +470,32 @@ def test_random_configurations_against_oracle(eng, oracle, case):
     plan.close()
 
 
+# draws of the same generator with one tree (every dimension up to five, every kind of cloud, variance compression)
+@pytest.mark.parametrize("case", [0, 2, 3, 7, 10, 13, 16, 19, 22, 28, 33, 42, 48, 50, 55, 62, 72])
+def test_random_configurations_symmetric_near_field(eng, oracle, monkeypatch, case):
+    """The symmetric near field (one column; F3M_SPLIT_TARGET=1 keeps one wavefront per work item on these small clouds)
+    on random one-tree configurations: no worse than 1.5x the oracle's error against the fp64 exact product, within
+    1e-5 of the one-directional form, the same bits from the one-shot call and from a plan applied twice."""
+    X, Y, b, prm, kind = random_configuration(case)
+    assert Y is None
+    b = np.ascontiguousarray(b[:, :1])
+    print("case random symmetric %d: d=%d %s n=%d %s" % (case, X.shape[1], kind, X.shape[0], prm), flush=True)
+    monkeypatch.setenv("F3M_SPLIT_TARGET", "1")
+    Xd, bd = dev(X), dev(b)
+    plan = eng.Plan(Xd, None, **prm)
+    got = plan.apply(bd).cpu().numpy()
+    assert np.array_equal(plan.apply(bd).cpu().numpy(), got)
+    plan.close()
+    assert np.array_equal(eng.kmvm(Xd, None, bd, **prm).cpu().numpy(), got)
+    want = oracle.kmvm(X, None, b, **prm)
+    exact = oracle.exact_f64(X, X, b, prm["ls"])
+    assert np.isfinite(got).all()
+    assert rel_l2(got, exact) <= 1.5 * rel_l2(want, exact) + 3e-6, (rel_l2(got, exact), rel_l2(want, exact))
+    monkeypatch.setenv("F3M_NEAR_SYM", "0")
+    # (another order of the same fp32 sums: up to 3e-6 where the lengthscale spans the cloud and the sums cancel)
+    assert rel_l2(got, eng.kmvm(Xd, None, bd, **prm).cpu().numpy()) < 1e-5
+
+
 PRODUCT_NAMES = ["C1_uniform3", "normal3", "clustered_xy", "uniform4", "uniform5_243", "uniform3_ls0.1", "uniform3_ls10",
                  "normal3_ls0.1", "normal3_ls10"]
 # Where the reference algorithm itself (the oracle, same nodes and lengthscale) misses the 1e-3 of the
