@@ -250,14 +250,17 @@ void exact_f64(int d, const double *X, long long N, const double *Y, long long M
 // tiles: work items (box, tile of `tile` consecutive points) for the boxes with flag != 0
 
 // order (nullable): slot k of the tile offsets stands for box order[k]
+// rowptr (nullable, instead of flag): the boxes with a row in that list
 __global__ void tiles_per_box_kernel(const int *__restrict__ off, const int *__restrict__ flag, int nb, int tile,
-                                     const int *__restrict__ order, int *__restrict__ ntiles)
+                                     const int *__restrict__ order, int *__restrict__ ntiles,
+                                     const int *__restrict__ rowptr)
 {
     int k = blockIdx.x * blockDim.x + threadIdx.x;
     if (k >= nb) return;
     const int b = order ? order[k] : k;
     int cnt = off[b + 1] - off[b];
-    ntiles[k] = (flag == nullptr || flag[b]) ? (cnt + tile - 1) / tile : 0;
+    const bool live = rowptr != nullptr ? rowptr[b + 1] > rowptr[b] : (flag == nullptr || flag[b]);
+    ntiles[k] = live ? (cnt + tile - 1) / tile : 0;
 }
 
 // Boxes ordered by the length of their list rows, longest first, in 256 classes of `unit` pairs (one
@@ -298,45 +301,16 @@ __global__ void mark_cols_kernel(const int *__restrict__ pairs, long long n, int
 // (nb + npoints/tile) to launch with; workgroups past tileoff[nb] exit at once, so the host never
 // waits for the exact count.
 static int build_tiles(const int *off, const int *flag, int nb, long long npoints, int tile, DBuf<int> &tileoff, hipStream_t s,
-                       const int *order = nullptr)
+                       const int *order = nullptr, const int *rowptr = nullptr)
 {
     DBuf<int> nt((size_t)nb);
     tileoff.reset((size_t)nb + 1);
-    F3M_LAUNCH(tiles_per_box_kernel, cdiv(nb, 256), 256, 0, s, off, flag, nb, tile, order, nt.get());
+    F3M_LAUNCH(tiles_per_box_kernel, cdiv(nb, 256), 256, 0, s, off, flag, nb, tile, order, nt.get(), rowptr);
     check_launch("tiles_per_box");
     exclusive_scan_i32(nt.get(), nb, tileoff.get(), s);
     long long bound = (long long)nb + npoints / tile;
     F3M_REQUIRE(bound < (1ll << 31) - 1, 32, "too many work items");
     return (int)bound;
-}
-
-// The tile table of a list in one launch, for up to kTileTableBoxes boxes in Morton order: tileoff (nb+1) = exclusive scan
-// of the work items per box, boxes without a row in the list (rowptr) count none.  One workgroup: every thread takes a
-// run of consecutive boxes, the runs' totals are scanned in LDS.  (Three launches and a scan's worth of small kernels
-// otherwise, between the last list and the near field's first launch.)
-constexpr int kTileTableBoxes = 65536, kTileTableThreads = 1024;
-__global__ void __launch_bounds__(kTileTableThreads) tile_table_kernel(const int *__restrict__ off, const int *__restrict__ rowptr,
-                                                                        int nb, int tile, int *__restrict__ tileoff)
-{
-    __shared__ int part[kTileTableThreads];
-    const int t = threadIdx.x, per = (nb + kTileTableThreads - 1) / kTileTableThreads;
-    const int b0 = min(nb, t * per), b1 = min(nb, b0 + per);
-    int sum = 0;
-    for (int b = b0; b < b1; b++) sum += rowptr[b + 1] > rowptr[b] ? (off[b + 1] - off[b] + tile - 1) / tile : 0;
-    part[t] = sum;
-    __syncthreads();
-    for (int step = 1; step < kTileTableThreads; step <<= 1) {       // inclusive scan of the runs' totals
-        const int v = t >= step ? part[t - step] : 0;
-        __syncthreads();
-        part[t] += v;
-        __syncthreads();
-    }
-    int run = part[t] - sum;
-    for (int b = b0; b < b1; b++) {
-        tileoff[b] = run;
-        run += rowptr[b + 1] > rowptr[b] ? (off[b + 1] - off[b] + tile - 1) / tile : 0;
-    }
-    if (t == kTileTableThreads - 1) tileoff[nb] = part[t];
 }
 
 __device__ inline int find_box(const int *__restrict__ tileoff, int nb, int tileid)
@@ -1256,14 +1230,9 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
     TileTable &tt = list.near_tiles[tilesize * 2 + (ordered ? 1 : 0)];
     if (tt.tileoff.size() == 0) {
         require_tables_may_be_built("the near-field tile table of a list");
-        if (!ordered && lx.nb <= kTileTableBoxes) {
-            tt.tileoff.reset((size_t)lx.nb + 1);
-            F3M_LAUNCH(tile_table_kernel, 1, kTileTableThreads, 0, s, lx.off.get(), list.rowptr.get(), lx.nb, tilesize,
-                       tt.tileoff.get());
-            check_launch("tile_table");
-            const long long bound = (long long)lx.nb + tx.n / tilesize;
-            F3M_REQUIRE(bound < (1ll << 31) - 1, 32, "too many work items");
-            tt.bound = (int)bound;
+        if (!ordered) {
+            // (the rows of the list mark the boxes: no pass of its own for the flags)
+            tt.bound = build_tiles(lx.off.get(), nullptr, lx.nb, tx.n, tilesize, tt.tileoff, s, nullptr, list.rowptr.get());
         } else {
         DBuf<int> flag((size_t)lx.nb);
         F3M_LAUNCH(mark_rows_kernel, cdiv(lx.nb, 256), 256, 0, s, list.rowptr.get(), lx.nb, flag.get());

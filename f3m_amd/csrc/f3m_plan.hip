@@ -344,6 +344,25 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
                            /*background=*/true);
             P->early_b = b_early;
             P->early_c = c_early;
+            // The result arrays of the product that follows are cleared here as well (and, for a single column on one
+            // tree, the fixed-point sums of the symmetric near field; the largest |weight| does not depend on the order
+            // of the weights): nothing of this waits for the tree, and what is queued after the last level -- the near
+            // field's source operands -- is then all that the near field still waits for.
+            P->early_outs.reset((size_t)P->N * (c_early >= 2 ? 4 : 1));
+            P->early_outs_far.reset((size_t)P->N * (c_early >= 2 ? 4 : 1));
+            dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, ss.stream);
+            dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, ss.stream);
+            const char *se = getenv("F3M_NEAR_SYM");
+            const bool maybe_sym = sym && c_early == 1 && d <= 5 && !(se && atoi(se) == 0);   // (wherever near_symmetric may say yes)
+            if (maybe_sym) {
+                P->early_symfix.reset((size_t)P->N);
+                P->early_symmax.reset(1);
+                dev_fill(P->early_symfix.get(), 0, sizeof(long long) * (size_t)P->N, ss.stream);
+                sym_absmax(P->early_bs.get(), P->M, P->early_symmax.get(), ss.stream);
+            } else if (out_early != nullptr) {   // the caller's array, for a product that adds its results straight into it
+                dev_fill(out_early, 0, sizeof(float) * (size_t)P->N * c_early, ss.stream);
+                P->early_out = out_early;
+            }
         }
         early = true;
         lot.start();
@@ -356,6 +375,10 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             early = false;
             P->early_b = nullptr;
             P->early_bs.free();
+            P->early_outs.free();
+            P->early_outs_far.free();
+            P->early_symfix.free();
+            P->early_symmax.free();
         }
     };
     if (need_tree && wants_division()) {
@@ -405,23 +428,6 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             // (The host has seen the counts of this level's division, so the level's arrays are complete.)
             if (!ahead && early) {
                 prepare_near_operands(d, *P->ty, P->ty->lev[k], P->lcs, side_stream().stream);
-                if (P->early_b != nullptr) {       // and the result arrays of the product that follows are cleared there
-                    const int nc = P->early_c >= 3 ? 4 : P->early_c;
-                    P->early_outs.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
-                    P->early_outs_far.reset((size_t)P->N * (P->early_c >= 2 ? 4 : 1));
-                    dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, side_stream().stream);
-                    dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, side_stream().stream);
-                    if (sym && P->early_c == 1 && d <= 5) {     // (wherever near_symmetric may say yes)
-                        P->early_symfix.reset((size_t)P->N);
-                        P->early_symmax.reset(1);
-                        dev_fill(P->early_symfix.get(), 0, sizeof(long long) * (size_t)P->N, side_stream().stream);
-                        sym_absmax(P->early_bs.get(), P->M, P->early_symmax.get(), side_stream().stream);
-                    }
-                    if (out_early != nullptr) {     // and the caller's array, for a product that adds its results straight into it
-                        dev_fill(out_early, 0, sizeof(float) * (size_t)P->N * P->early_c, side_stream().stream);
-                        P->early_out = out_early;
-                    }
-                }
             }
             fetch_level_wait();
             lists_finish(pend, reinterpret_cast<const long long *>(hres), *keep, P->tx, *P->ty, k, cp, L,
