@@ -353,7 +353,9 @@ static f3m_plan *plan_create(int d, const float *X, long long N, const float *Y,
             dev_fill(P->early_outs.get(), 0, sizeof(float) * (size_t)P->N * nc, ss.stream);
             dev_fill(P->early_outs_far.get(), 0, sizeof(float) * (size_t)P->N * P->early_ncol, ss.stream);
             const char *se = getenv("F3M_NEAR_SYM");
-            const bool maybe_sym = sym && c_early == 1 && d <= 5 && !(se && atoi(se) == 0);   // (wherever near_symmetric may say yes)
+            // (wherever near_symmetric may say yes; with variance compression the near lists are short or empty and the
+            // product prepares the sums itself if it turns out to need them)
+            const bool maybe_sym = sym && c_early == 1 && d <= 5 && !(se && atoi(se) == 0) && !prm->var_compression;
             if (maybe_sym) {
                 P->early_symfix.reset((size_t)P->N);
                 P->early_symmax.reset(1);
