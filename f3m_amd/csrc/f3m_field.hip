@@ -1267,8 +1267,13 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         if (const char *env = getenv("F3M_NEAR_STRIPE")) stripe = atoi(env);       // tuning aid
         // Few targets against long lists (the transposed product of a tall kernel matrix): too few work
         // items to fill the GPU, so every list is cut into slices with a wavefront each.
+        // (A list that takes the symmetric form stays whole from 4096 work items on: half the tiles outweigh the
+        // emptier end of the launch.  Uniform 3-D clouds, whole product with 4096 against 16384: N=6e5 0.82 against 0.86
+        // ms, 1.1e6 1.36 / 1.49, 1.5e6 1.81 / 2.01; with 2048 N=3e5 takes 1.05 against 0.83 ms.)
+        int single = sym ? 4096 : 16384;
+        if (const char *e = getenv("F3M_SYM_SINGLE")) single = sym ? atoi(e) : single;   // tuning aid
         int nsplit = 1;
-        if (ntiles < 16384) {
+        if (ntiles < single) {
             int target = 32768;      // wavefronts aimed at (K_nm^T u with 1e7 sources, 2e4 / 1e5 targets: 8192 -> 9.7 / 8.1 ms,
                                      // 16384 -> 7.6 / 6.8, 32768 -> 7.5 / 6.0)
             if (const char *e = getenv("F3M_SPLIT_TARGET")) target = atoi(e);
