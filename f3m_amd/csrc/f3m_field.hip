@@ -618,7 +618,8 @@ struct __attribute__((aligned(4))) float4u { float x, y, z, w; };   // four floa
 // summed over the columns into the sources of B -- 16 more accumulators per lane, kept over the target tiles of the
 // work item, then added up across the 32 columns through the wavefront's own LDS block and added to the sums of B
 // atomically, as fixed-point numbers (SymSums): integer additions give the same result in any order.  Half the
-// exponentials per listed pair of points.
+// exponentials per listed pair of points.  With FACT the second direction carries the targets' factor exp2(-|x''|^2) in
+// its weights (set up per anchor) and receives the sources' factor exp2(-|y'|^2) after the sum over the columns.
 constexpr int kSymRedStride = 33;                  // floats per row of the reduction block (32 columns + 1: no bank conflicts)
 __device__ __forceinline__ void atomic_add_i64(long long *p, long long v)
 {
