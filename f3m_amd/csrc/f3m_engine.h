@@ -233,6 +233,9 @@ struct SymSums {
     // factored form only (near_field fills them in): the sorted weights themselves (the kernel's weight argument then holds
     // them times exp2(-|y'|^2)) and that factor per point
     const float *braw = nullptr, *ey = nullptr;
+    // set by the caller where the far field that runs beside the near field is made of small one-wavefront workgroups
+    // (node grids up to 4 x 4 x 4): the near field then takes workgroups of one wavefront itself (see near_sym_waves)
+    bool small_far = false;
 };
 // scale of the fixed-point sums as a power of two (0: weights not finite)
 __host__ __device__ inline float sym_scale(unsigned absmax_bits, long long nsrc)

@@ -640,7 +640,7 @@ __device__ __forceinline__ void atomic_add_f32(float *p, float v)
 // (The symmetric form is held to 120 registers: four wavefronts per SIMD then leave 32 of its 512 free, as five of the
 // plain form's 96 do, and the small workgroups of the far field find room beside a running near field; at 128 they
 // wait for its end.)
-template <int D, int TPW, int NC, bool FACT, bool SYM>
+template <int D, int TPW, int NC, bool FACT, bool SYM, int WPB = kNearWavesPerBlock>
 __device__ __forceinline__ void near_g_body(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
@@ -665,7 +665,7 @@ __device__ __forceinline__ void near_g_body(
     // work item: TPW*32 targets of one box; with few targets and long lists (nsplit > 1) the list of a
     // work item is cut into nsplit slices, one wavefront each, whose sums go to `part` (nsplit x NC x
     // nitems x TPW*32 floats, indexed by work item) and are added up in a fixed order afterwards
-    const int wfull = vblock * kNearWavesPerBlock + (threadIdx.x >> 6);
+    const int wfull = vblock * WPB + (threadIdx.x >> 6);
     const int wid = wfull / nsplit, slice = wfull % nsplit;
     if (wid >= tileoff[nbx]) return;
     const int slot = find_box(tileoff, nbx, wid);
@@ -692,7 +692,7 @@ __device__ __forceinline__ void near_g_body(
     // and targets are the same points in the same order), kept there to spare registers
     // (factored form: a second copy, the weights times the targets' factor exp2(-|x''|^2) of the current anchor)
     constexpr int kSymBlock = 32 * kSymRedStride + TPW * 32 * (FACT ? 2 : 1);
-    __shared__ float red_all[SYM ? kNearWavesPerBlock * kSymBlock : 1];
+    __shared__ float red_all[SYM ? WPB * kSymBlock : 1];
     float *const red = red_all + (SYM ? (threadIdx.x >> 6) * kSymBlock : 0);
     float *const btl = red + 32 * kSymRedStride;
     float *const wtl = FACT ? btl + TPW * 32 : btl;
@@ -988,8 +988,14 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, (D <= 3 && TPW == 4 &
 #else
 #define F3M_NEAR_SYM_REGS __attribute__((amdgpu_num_vgpr(60)))      // counted in pairs on this target: 120 registers
 #endif
-template <int D, int TPW>
-__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
+// WPB wavefronts per workgroup.  One, up to three dimensions and where the far field beside it consists of small
+// workgroups: a freed place is taken at once, not when a second one is free as well (N=1e7 3-D: 8.07 -> 7.9 ms, N(0,I)
+// 12.85 -> 12.6).  The far field is pushed back by that: in 4-D, whose M2L is longer, the product gains nothing
+// (12.4 -> 12.4-12.7 ms), and the large M2L workgroups of the 5^3 and 6^3 grids come in so late that the products take
+// longer (216 nodes: 8.65 -> 9.4 ms): two wavefronts there.
+constexpr int near_sym_waves(int d, bool small_far) { return d <= 3 && small_far ? 1 : kNearWavesPerBlock; }
+template <int D, int TPW, int WPB>
+__global__ void __launch_bounds__(WPB * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
@@ -997,7 +1003,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) F3M_NEAR_SYM_REGS 
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
     SymSums symsums)
 {
-    near_g_body<D, TPW, 1, false, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+    near_g_body<D, TPW, 1, false, true, WPB>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                       rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
@@ -1284,7 +1290,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         if (nsplit > 1) part.reset((size_t)nsplit * nc * ntiles * tpw * 32);   // every slot of a live work item is written
         F3M_REQUIRE(direct == nullptr || nsplit == 1, 35, "direct output needs a near field of one wavefront per work item");
         const DirectOut dout = direct ? *direct : DirectOut();
-        int nblk = (int)cdiv((long long)ntiles * nsplit, kNearWavesPerBlock);
+        const int wpb = (sym && nsplit == 1 && !fact) ? near_sym_waves(d, symsums->small_far) : kNearWavesPerBlock;   // wavefronts per workgroup
+        int nblk = (int)cdiv((long long)ntiles * nsplit, wpb);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
         // weights of the factored form: the sorted weights times exp2(-|y'|^2) of their point (one pass per product)
@@ -1307,7 +1314,7 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
             SymSums sums = *symsums;
             sums.braw = bs;
             sums.ey = src.ey;
-            F3M_LAUNCH(kern, ngrid, kNearWavesPerBlock * 64, 0, s, tx.pts.get(), tx.n, src.ops, stride, wsrc, wstride, outs,
+            F3M_LAUNCH(kern, ngrid, wpb * 64, 0, s, tx.pts.get(), tx.n, src.ops, stride, wsrc, wstride, outs,
                        ostride, lx.off.get(), ly.off.get(), ly.cell.get(), ty.geo, ly.edge, list.pairs.get(),
                        list.rowptr.get(), tileoff.get(), lx.nb, sc, stripe, nsplit, part.get(), ntiles, ord, dout, sums);
         };
@@ -1318,8 +1325,15 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
                 if (tpw == 5) go_sym((near_symf_kernel<DD, 5>));                                                      \
                 else go_sym((near_symf_kernel<DD, 4>));                                                               \
             } else {                                                                                                  \
-                if (tpw == 5) go_sym((near_sym_kernel<DD, 5>));                                                       \
-                else go_sym((near_sym_kernel<DD, 4>));                                                                \
+                if constexpr (DD <= 3) {                                                                              \
+                    if (wpb == 1) {                                                                                   \
+                        if (tpw == 5) go_sym((near_sym_kernel<DD, 5, 1>));                                            \
+                        else go_sym((near_sym_kernel<DD, 4, 1>));                                                     \
+                        break;                                                                                        \
+                    }                                                                                                 \
+                }                                                                                                     \
+                if (tpw == 5) go_sym((near_sym_kernel<DD, 5, kNearWavesPerBlock>));                                   \
+                else go_sym((near_sym_kernel<DD, 4, kNearWavesPerBlock>));                                            \
             }                                                                                                         \
             break;                                                                                                    \
         }                                                                                                             \

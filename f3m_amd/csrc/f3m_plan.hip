@@ -736,6 +736,9 @@ static void plan_apply(f3m_plan *P, const float *b, int c, float *out, hipStream
             symsums.fix = symfix.get();
             symsums.absmax = symmax.get();
             symsums.nsrc = NS;
+            symsums.small_far = true;               // the far field's workgroups are single small wavefronts up to 4 x 4 x 4 nodes
+            for (int k = 1; k <= depth; k++)
+                if (P->levels[k - 1].far.n > 0 && P->levels[k - 1].num_nodes > 64) symsums.small_far = false;
         }
         const SymSums *sym = use_sym ? &symsums : nullptr;
         {
