@@ -45,7 +45,7 @@ def profiled_near_launch_us():
     """average duration of the near-field launch in the committed rocprofv3 kernel trace of this command (the first
     table: default two-stream mode), microseconds"""
     try:
-        m = re.search(r"\|\s*f3m::near_sym_kernel<3, 5>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
+        m = re.search(r"\|\s*f3m::near_sym_kernel<3, 5, 1>\s*\|\s*\d+\s*\|\s*[0-9.]+\s*\|\s*([0-9.]+)\s*\|", open(STATS_PROFILE).read())
         return float(m.group(1)) if m else None
     except OSError:
         return None
@@ -283,7 +283,8 @@ def main():
     traffic, traffic_range = near_traffic_bytes() if headline else (None, None)
     roofline = {"bound": "valu", "achieved": near["achieved_tflops"], "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                 "frac": near["frac"], "traffic": traffic, "traffic_range": traffic_range,
-                "kernel": "near_sym_kernel<%d,%d>" % (d, tiles_per_wave) if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
+                "kernel": "near_sym_kernel<%d,%d,%d>" % (d, tiles_per_wave, 1 if d <= 3 and cfg["nodes"] <= 64 else 2) if near["symmetric"] and d <= 4 else
+                          "near_symf_kernel<%d,%d>" % (d, tiles_per_wave) if near["symmetric"] else "near_g_kernel<%d,%d,1>" % (d, tiles_per_wave),
                 "valu_issue_frac": near["valu_frac"],
                 "note": "near field, bound by fp32 vector-ALU issue (one exp2 and one FMA per kernel evaluation; the exponents "
                         "come from the f16 matrix pipe with hi/lo-split operands, fp32 accumulate); achieved = %d algorithmic "
