@@ -1010,7 +1010,7 @@ __global__ void __launch_bounds__(WPB * 64, 4) F3M_NEAR_SYM_REGS near_sym_kernel
 // the symmetric form with the factored exponent (five dimensions): the far field does not run beside it (plan_apply), so
 // it keeps the 128 registers of four wavefronts per SIMD
 template <int D, int TPW>
-__global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) near_symf_kernel(
+__global__ void __launch_bounds__(64, 4) near_symf_kernel(
     const float *__restrict__ xs, long long N, const h8 *__restrict__ ops, long long stride, const float *__restrict__ bs,
     long long bstride, float *__restrict__ outs, long long ostride, const int *__restrict__ offx,
     const int *__restrict__ offy, const int *__restrict__ celly, Geo geoy, float edgey,
@@ -1018,7 +1018,7 @@ __global__ void __launch_bounds__(kNearWavesPerBlock * 64, 4) near_symf_kernel(
     int stripe, int nsplit, float *__restrict__ part, int nitems, const int *__restrict__ order, DirectOut dout,
     SymSums symsums)
 {
-    near_g_body<D, TPW, 1, true, true>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
+    near_g_body<D, TPW, 1, true, true, 1>(xs, N, ops, stride, bs, bstride, outs, ostride, offx, offy, celly, geoy, edgey, pairs,
                                        rowptr, tileoff, nbx, sc, stripe, nsplit, part, nitems, order, dout, symsums);
 }
 
@@ -1290,7 +1290,8 @@ void near_field(int d, const Tree &tx, const TreeLevel &lx, const Tree &ty, cons
         if (nsplit > 1) part.reset((size_t)nsplit * nc * ntiles * tpw * 32);   // every slot of a live work item is written
         F3M_REQUIRE(direct == nullptr || nsplit == 1, 35, "direct output needs a near field of one wavefront per work item");
         const DirectOut dout = direct ? *direct : DirectOut();
-        const int wpb = (sym && nsplit == 1 && !fact) ? near_sym_waves(d, symsums->small_far) : kNearWavesPerBlock;   // wavefronts per workgroup
+        // wavefronts per workgroup (the factored symmetric form, which nothing runs beside: one)
+        const int wpb = (sym && nsplit == 1) ? (fact ? 1 : near_sym_waves(d, symsums->small_far)) : kNearWavesPerBlock;
         int nblk = (int)cdiv((long long)ntiles * nsplit, wpb);
         int ngrid = stripe > 0 ? (int)cdiv(nblk, 8 * stripe) * 8 * stripe : nblk;
         timer_begin(kNear, s);
